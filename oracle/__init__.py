@@ -1,0 +1,223 @@
+"""CPU oracle: ctypes/numpy front end of ``liboracle.so``.
+
+TEST INFRASTRUCTURE ONLY.  Only ``tests/``, ``__graft_entry__.smoke()`` and the
+``cpu_baseline`` leg of ``bench.py`` import this package; the shipped library
+(``aidotnet.tensors_amd``) never does.  Each C function cites the reference
+file:line it restates in its own source comment.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboracle.so")
+_lib = None
+
+_f32p = ctypes.POINTER(ctypes.c_float)
+_f64p = ctypes.POINTER(ctypes.c_double)
+_u16p = ctypes.POINTER(ctypes.c_uint16)
+_u8p = ctypes.POINTER(ctypes.c_uint8)
+_i32p = ctypes.POINTER(ctypes.c_int)
+
+
+def build(force: bool = False) -> str:
+    """Compile ``liboracle.so`` with the Makefile beside this file."""
+    if force and os.path.exists(_LIB_PATH):
+        os.remove(_LIB_PATH)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.orc_bf16_from_float.argtypes = [ctypes.c_float]
+        L.orc_bf16_from_float.restype = ctypes.c_uint16
+        L.orc_bf16_to_float.argtypes = [ctypes.c_uint16]
+        L.orc_bf16_to_float.restype = ctypes.c_float
+        L.orc_f16_from_float.argtypes = [ctypes.c_float]
+        L.orc_f16_from_float.restype = ctypes.c_uint16
+        L.orc_f16_to_float.argtypes = [ctypes.c_uint16]
+        L.orc_f16_to_float.restype = ctypes.c_float
+        L.orc_hash_uniform.argtypes = [ctypes.c_uint32]
+        L.orc_hash_uniform.restype = ctypes.c_float
+        L.orc_max_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a: np.ndarray, typ):
+    return a.ctypes.data_as(typ)
+
+
+def _c(a, dtype) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=dtype)
+
+
+def max_threads() -> int:
+    return int(lib().orc_max_threads())
+
+
+# ----------------------------------------------------------------- conversions
+def f32_to_bf16(x) -> np.ndarray:
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_convert_f32_to_bf16(_p(x, _f32p), _p(out, _u16p), ctypes.c_long(x.size))
+    return out
+
+
+def bf16_to_f32(x) -> np.ndarray:
+    x = _c(x, np.uint16)
+    out = np.empty(x.shape, np.float32)
+    lib().orc_convert_bf16_to_f32(_p(x, _u16p), _p(out, _f32p), ctypes.c_long(x.size))
+    return out
+
+
+def f32_to_f16(x) -> np.ndarray:
+    """float32 -> IEEE binary16 bit patterns (uint16)."""
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    lib().orc_convert_f32_to_f16(_p(x, _f32p), _p(out, _u16p), ctypes.c_long(x.size))
+    return out
+
+
+def f16_to_f32(x) -> np.ndarray:
+    x = _c(x, np.uint16)
+    out = np.empty(x.shape, np.float32)
+    lib().orc_convert_f16_to_f32(_p(x, _u16p), _p(out, _f32p), ctypes.c_long(x.size))
+    return out
+
+
+def hash_uniform(n: int, seed: int = 0) -> np.ndarray:
+    """The reference test-suite's portable PCG-style hash generator, values in [-0.5, 0.5]."""
+    out = np.empty(int(n), np.float32)
+    lib().orc_fill_hash_uniform(_p(out, _f32p), ctypes.c_long(int(n)), ctypes.c_uint32(seed & 0xFFFFFFFF))
+    return out
+
+
+# ------------------------------------------------------------------------ GEMM
+def sgemm(a, b, m: int, k: int, n: int, threads: int = 1) -> np.ndarray:
+    """``SimdGemm.Sgemm(a, b, c, m, k, n)``: C[m,n] = A[m,k] * B[k,n], overwrite."""
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    assert a.size >= m * k and b.size >= k * n
+    c = np.full((max(m, 0), max(n, 0)), np.nan, np.float32)
+    lib().orc_sgemm(_p(a, _f32p), _p(b, _f32p), _p(c, _f32p), m, k, n, threads)
+    return c
+
+
+def sgemm_ex(a, lda, trans_a, b, ldb, trans_b, m, k, n, threads: int = 1) -> np.ndarray:
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    c = np.full((m, n), np.nan, np.float32)
+    lib().orc_sgemm_ex(_p(a, _f32p), lda, int(trans_a), _p(b, _f32p), ldb, int(trans_b),
+                       _p(c, _f32p), m, k, n, threads)
+    return c
+
+
+def gemm_alpha_beta(a, b, c, m, n, k, alpha=1.0, beta=0.0, trans_b=False, threads: int = 1) -> np.ndarray:
+    """Backend contract ``C = alpha*A*B + beta*C`` (argument order M, N, K). Returns the new C."""
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    c = np.array(c, dtype=np.float32, copy=True).reshape(m, n)
+    lib().orc_gemm_alpha_beta(_p(a, _f32p), _p(b, _f32p), _p(c, _f32p), m, n, k,
+                              ctypes.c_float(alpha), ctypes.c_float(beta), int(trans_b), threads)
+    return c
+
+
+def gemm_f64(a, b, m, k, n, trans_b=False, threads: int = 0) -> np.ndarray:
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    c = np.empty((m, n), np.float64)
+    lib().orc_gemm_f64(_p(a, _f32p), _p(b, _f32p), _p(c, _f64p), m, k, n, int(trans_b),
+                       threads or max_threads())
+    return c
+
+
+def _gemm16(fn, a, b, m, k, n, threads):
+    a = _c(a, np.uint16); b = _c(b, np.uint16)
+    assert a.size >= m * k and b.size >= k * n
+    o16 = np.empty((m, n), np.uint16)
+    o32 = np.empty((m, n), np.float32)
+    fn(_p(a, _u16p), k, _p(b, _u16p), n, _p(o16, _u16p), _p(o32, _f32p), n, m, k, n,
+       threads or max_threads())
+    return o16, o32
+
+
+def hgemm(a_bits, b_bits, m, k, n, threads: int = 0):
+    """``HalfKernels.Matmul`` on fp16 bit patterns: returns (rounded fp16 bits, fp32 accumulator)."""
+    return _gemm16(lib().orc_hgemm, a_bits, b_bits, m, k, n, threads)
+
+
+def bf16gemm(a_bits, b_bits, m, k, n, threads: int = 0):
+    """``BFloat16Kernels.Matmul`` on bf16 bit patterns: returns (rounded bf16 bits, fp32 accumulator)."""
+    return _gemm16(lib().orc_bf16gemm, a_bits, b_bits, m, k, n, threads)
+
+
+# ------------------------------------------------------------------- attention
+def attention_f32(q, k, v, scale, causal=False, query_offset=0, bias=None, keep=None,
+                  softcap=0.0, want_weights=False, threads: int = 0):
+    """fp32 attention as the reference CPU engine computes it.
+
+    q [B,H,Sq,D]; k, v [B,Hkv,Sk,D]; bias [B,H,Sq,Sk] or [H,Sq,Sk]; keep: bool array of
+    rank 4 broadcastable to [B,H,Sq,Sk].  Returns (out, lse, weights-or-None).
+    """
+    q = _c(q, np.float32); k = _c(k, np.float32); v = _c(v, np.float32)
+    B, H, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    out = np.full((B, H, Sq, D), np.nan, np.float32)
+    lse = np.full((B, H, Sq), np.nan, np.float32)
+    w = np.full((B, H, Sq, Sk), np.nan, np.float32) if want_weights else None
+    bias_p, bstride = None, 0
+    if bias is not None:
+        bias = _c(bias, np.float32)
+        bstride = H * Sq * Sk if bias.ndim == 4 else 0
+        bias_p = _p(bias, _f32p)
+    keep_p, shape_p = None, None
+    if keep is not None:
+        keep = _c(keep, np.uint8)
+        assert keep.ndim == 4
+        shape = np.array(keep.shape, np.int32)
+        keep_p, shape_p = _p(keep, _u8p), _p(shape, _i32p)
+    lib().orc_attention_f32(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), bias_p, ctypes.c_long(bstride),
+                            keep_p, shape_p, _p(out, _f32p), _p(lse, _f32p),
+                            _p(w, _f32p) if w is not None else None,
+                            B, H, Hkv, Sq, Sk, D, ctypes.c_float(scale), int(causal), int(query_offset),
+                            ctypes.c_float(softcap), threads or max_threads())
+    return out, lse, w
+
+
+def attention_f64(q, k, v, scale, causal=False, query_offset=0, bias=None, keep=None,
+                  softcap=0.0, threads: int = 0):
+    q = _c(q, np.float32); k = _c(k, np.float32); v = _c(v, np.float32)
+    B, H, Sq, D = q.shape
+    Hkv, Sk = k.shape[1], k.shape[2]
+    out = np.empty((B, H, Sq, D), np.float64)
+    lse = np.empty((B, H, Sq), np.float64)
+    bias_p, bstride = None, 0
+    if bias is not None:
+        bias = _c(bias, np.float32)
+        bstride = H * Sq * Sk if bias.ndim == 4 else 0
+        bias_p = _p(bias, _f32p)
+    keep_p, shape_p = None, None
+    if keep is not None:
+        keep = _c(keep, np.uint8)
+        shape = np.array(keep.shape, np.int32)
+        keep_p, shape_p = _p(keep, _u8p), _p(shape, _i32p)
+    lib().orc_attention_f64(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), bias_p, ctypes.c_long(bstride),
+                            keep_p, shape_p, _p(out, _f64p), _p(lse, _f64p),
+                            B, H, Hkv, Sq, Sk, D, ctypes.c_double(scale), int(causal), int(query_offset),
+                            ctypes.c_double(softcap), threads or max_threads())
+    return out, lse
+
+
+def decode_f32(q, k, v, heads, kv_heads, head_dim, seq_len, scale) -> np.ndarray:
+    """The reference decode test's oracle: q [heads, d], k/v [seqLen, kvHeads, d] -> [heads, d]."""
+    q = _c(q, np.float32); k = _c(k, np.float32); v = _c(v, np.float32)
+    out = np.empty((heads, head_dim), np.float32)
+    lib().orc_decode_f32(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), _p(out, _f32p),
+                         heads, kv_heads, head_dim, seq_len, ctypes.c_float(scale))
+    return out
