@@ -1,0 +1,268 @@
+// C ABI of libaidotnet_mi355.so (declared in include/aidotnet_mi355.h): argument validation,
+// status codes, the per-context workspace, and nothing else.  Validation mirrors what the
+// reference's managed backend checks before its native calls (non-positive dimensions,
+// grouped-query ratio, head-dim limit: src/AiDotNet.Tensors/Engines/DirectGpu/HIP/
+// HipBackend.HalfPrecision.cs:167-177, HipBackend.cs:6123-6141, GpuKernelGuards.cs:12-52).
+#include "../../../include/aidotnet_mi355.h"
+#include "launch.hpp"
+
+#include <mutex>
+#include <string>
+#include <cstdio>
+#include <cstring>
+
+namespace {
+
+struct Ctx {
+    int device = 0;
+    std::mutex mu;
+    std::string last_error;
+    void* ws = nullptr;          // library-owned workspace (decode split partials, LSE for weights)
+    size_t ws_bytes = 0;
+    int force_tile = 0;
+};
+
+int fail(Ctx* c, int code, const char* what)
+{
+    if (c) {
+        std::lock_guard<std::mutex> g(c->mu);
+        c->last_error = what;
+    }
+    return code;
+}
+
+int hip_status(Ctx* c, hipError_t e, const char* where)
+{
+    if (e == hipSuccess) return AIDN_OK;
+    char buf[256];
+    snprintf(buf, sizeof buf, "%s: %s", where, hipGetErrorString(e));
+    if (c) {
+        std::lock_guard<std::mutex> g(c->mu);
+        c->last_error = buf;
+    }
+    return (int)e;
+}
+
+// Grow-only workspace.  Replacing it first drains the device so no queued kernel still uses the old block.
+int ensure_ws(Ctx* c, size_t bytes)
+{
+    std::lock_guard<std::mutex> g(c->mu);
+    if (bytes <= c->ws_bytes) return AIDN_OK;
+    if (c->ws) {
+        hipError_t e = hipDeviceSynchronize();
+        if (e != hipSuccess) { c->last_error = "workspace: hipDeviceSynchronize failed"; return (int)e; }
+        (void)hipFree(c->ws);
+        c->ws = nullptr; c->ws_bytes = 0;
+    }
+    size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+    void* p = nullptr;
+    if (hipMalloc(&p, want) != hipSuccess) { c->last_error = "workspace: hipMalloc failed"; return AIDN_ERR_OUT_OF_MEMORY; }
+    c->ws = p; c->ws_bytes = want;
+    return AIDN_OK;
+}
+
+bool dense0(const int64_t* s) { return s[0] == 0 && s[1] == 0 && s[2] == 0; }
+
+int fill_params(Ctx* c, const aidn_attn_desc* d, aidn::AttnParams& p)
+{
+    if (!d) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: descriptor is null");
+    if (d->B <= 0 || d->H <= 0 || d->Sq <= 0 || d->Sk <= 0 || d->D <= 0)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: dimensions must be positive");
+    int hkv = d->Hkv > 0 ? d->Hkv : d->H;
+    if (hkv > d->H || d->H % hkv != 0)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: H must be an integer multiple of Hkv");
+    if (d->D > 256) return fail(c, AIDN_ERR_UNSUPPORTED, "attention: head dimension above 256");
+    if (d->mask_mode < 0 || d->mask_mode > 2) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: mask_mode must be 0, 1 or 2");
+    p.B = d->B; p.H = d->H; p.Hkv = hkv; p.Sq = d->Sq; p.Sk = d->Sk; p.D = d->D;
+    p.scale = d->scale; p.causal = d->causal != 0; p.qoff = d->causal_query_offset; p.softcap = d->softcap;
+    p.mask_mode = d->mask_mode; p.out16 = d->out_is_16bit != 0; p.bias_bs = d->bias_batch_stride;
+    auto set = [&](long long* dst, const int64_t* src, long long heads, long long rows) {
+        if (dense0(src)) { dst[0] = heads * rows * d->D; dst[1] = rows * d->D; dst[2] = d->D; }
+        else { dst[0] = src[0]; dst[1] = src[1]; dst[2] = src[2]; }
+    };
+    set(p.qs, d->q_strides, d->H, d->Sq);
+    set(p.ks, d->k_strides, hkv, d->Sk);
+    set(p.vs, d->v_strides, hkv, d->Sk);
+    set(p.os, d->o_strides, d->H, d->Sq);
+    return AIDN_OK;
+}
+
+int attn_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, const void* q, const void* k, const void* v,
+                void* o, float* lse, const float* bias, const float* mask, float* weights)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!q || !k || !v || !o) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: q, k, v and o must not be null");
+    aidn::AttnParams p;
+    int st = fill_params(c, d, p);
+    if (st) return st;
+    if (kind == 0 && p.out16) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: fp32 kernel has no 16-bit output");
+    if (p.mask_mode != 0 && !mask) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "attention: mask_mode set but mask is null");
+    p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.bias = bias; p.mask = p.mask_mode ? mask : nullptr; p.weights = weights;
+    if (weights && !lse) {
+        // the probabilities are rebuilt from the saved log-sum-exp: borrow the workspace for it
+        size_t need = (size_t)p.B * p.H * p.Sq * sizeof(float);
+        st = ensure_ws(c, need);
+        if (st) return st;
+        p.lse = (float*)c->ws;
+    }
+    return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "attn_fwd");
+}
+
+int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, const void* q, const void* k, const void* v,
+                  void* o, float* lse, int splits)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!q || !k || !v || !o) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "decode: q, k, v and o must not be null");
+    aidn::AttnParams p;
+    int st = fill_params(c, d, p);
+    if (st) return st;
+    if (p.Sq != 1) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "decode: Sq must be 1");
+    if (kind == 0 && p.out16) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "decode: fp32 kernel has no 16-bit output");
+    p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.bias = nullptr; p.mask = nullptr; p.weights = nullptr;
+    int eff = aidn::attn_decode_splits(p, splits);
+    size_t need = aidn::attn_decode_workspace_bytes(p, eff);
+    if (need) { st = ensure_ws(c, need); if (st) return st; }
+    return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, c->ws), "attn_decode");
+}
+
+int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32, int M, int N, int K)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: A, B and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: dimensions must be positive");
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile), "gemm_16");
+}
+
+int convert_common(void* ctx, void* stream, int kind, const void* in, void* out, int64_t n)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (n < 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "convert: negative element count");
+    if (n == 0) return AIDN_OK;
+    if (!in || !out) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "convert: in and out must not be null");
+    return hip_status(c, aidn::convert((hipStream_t)stream, kind, in, out, n), "convert");
+}
+
+}  // namespace
+
+extern "C" {
+
+AIDN_API int aidn_mi355_create(int device, void** ctx)
+{
+    if (!ctx) return AIDN_ERR_INVALID_ARGUMENT;
+    *ctx = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0 || device < 0 || device >= count) return AIDN_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return AIDN_ERR_NO_DEVICE;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return AIDN_ERR_NO_DEVICE;   // the code object holds gfx950 ISA only
+    hipError_t e = hipSetDevice(device);
+    if (e != hipSuccess) return (int)e;
+    Ctx* c = new Ctx();
+    c->device = device;
+    *ctx = c;
+    return AIDN_OK;
+}
+
+AIDN_API int aidn_mi355_destroy(void* ctx)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_OK;
+    if (c->ws) { (void)hipDeviceSynchronize(); (void)hipFree(c->ws); }
+    delete c;
+    return AIDN_OK;
+}
+
+AIDN_API const char* aidn_mi355_last_error(void* ctx)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return "";
+    std::lock_guard<std::mutex> g(c->mu);
+    static thread_local std::string copy;
+    copy = c->last_error;
+    return copy.c_str();
+}
+
+AIDN_API const char* aidn_mi355_version(void) { return "aidotnet-mi355 0.1 (gfx950)"; }
+
+AIDN_API int aidn_mi355_sync(void* ctx, void* stream)
+{
+    return hip_status((Ctx*)ctx, hipStreamSynchronize((hipStream_t)stream), "hipStreamSynchronize");
+}
+
+AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (tile != 0 && tile != 64 && tile != 128 && tile != 256) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "tile must be 0, 64, 128 or 256");
+    c->force_tile = tile;
+    return AIDN_OK;
+}
+
+AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
+                     int M, int N, int K, float alpha, float beta, int transB)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: A, B and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
+    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile), "gemm_f32");
+}
+
+AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, const float* B, float* C,
+                             int M, int N, int K, int batch, float alpha, float beta)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: A, B and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: dimensions must be positive");
+    if (batch <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: batch count must be positive");
+    if (batch > 65535) return fail(c, AIDN_ERR_UNSUPPORTED, "sgemm_batched: more than 65535 batches");
+    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, 0, batch,
+                                        (long long)M * K, (long long)K * N, (long long)M * N, tile), "gemm_f32 (batched)");
+}
+
+AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K)
+{ return gemm16_common(ctx, stream, 0, A, B, C, 1, M, N, K); }
+AIDN_API int aidn_mi355_hgemm_f16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K)
+{ return gemm16_common(ctx, stream, 0, A, B, C, 0, M, N, K); }
+AIDN_API int aidn_mi355_bf16gemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K)
+{ return gemm16_common(ctx, stream, 1, A, B, C, 1, M, N, K); }
+AIDN_API int aidn_mi355_bf16gemm_bf16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K)
+{ return gemm16_common(ctx, stream, 1, A, B, C, 0, M, N, K); }
+
+AIDN_API int aidn_mi355_convert_f32_to_f16(void* ctx, void* stream, const float* in, uint16_t* out, int64_t n)
+{ return convert_common(ctx, stream, 0, in, out, n); }
+AIDN_API int aidn_mi355_convert_f16_to_f32(void* ctx, void* stream, const uint16_t* in, float* out, int64_t n)
+{ return convert_common(ctx, stream, 1, in, out, n); }
+AIDN_API int aidn_mi355_convert_f32_to_bf16(void* ctx, void* stream, const float* in, uint16_t* out, int64_t n)
+{ return convert_common(ctx, stream, 2, in, out, n); }
+AIDN_API int aidn_mi355_convert_bf16_to_f32(void* ctx, void* stream, const uint16_t* in, float* out, int64_t n)
+{ return convert_common(ctx, stream, 3, in, out, n); }
+
+AIDN_API int aidn_mi355_attn_fwd_f32(void* ctx, void* stream, const aidn_attn_desc* desc, const float* q, const float* k, const float* v,
+                            float* o, float* lse, const float* bias, const float* mask, float* weights)
+{ return attn_common(ctx, stream, 0, desc, q, k, v, o, lse, bias, mask, weights); }
+AIDN_API int aidn_mi355_attn_fwd_f16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                            void* o, float* lse, const float* bias, const float* mask, float* weights)
+{ return attn_common(ctx, stream, 1, desc, q, k, v, o, lse, bias, mask, weights); }
+AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                             void* o, float* lse, const float* bias, const float* mask, float* weights)
+{ return attn_common(ctx, stream, 2, desc, q, k, v, o, lse, bias, mask, weights); }
+
+AIDN_API int aidn_mi355_attn_decode_f32(void* ctx, void* stream, const aidn_attn_desc* desc, const float* q, const float* k, const float* v,
+                               float* o, float* lse, int splits)
+{ return decode_common(ctx, stream, 0, desc, q, k, v, o, lse, splits); }
+AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                               void* o, float* lse, int splits)
+{ return decode_common(ctx, stream, 1, desc, q, k, v, o, lse, splits); }
+AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                void* o, float* lse, int splits)
+{ return decode_common(ctx, stream, 2, desc, q, k, v, o, lse, splits); }
+
+}  // extern "C"

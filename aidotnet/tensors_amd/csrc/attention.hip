@@ -1,0 +1,460 @@
+// Fused scaled-dot-product attention (forward) for gfx950: flash-style, one pass over K/V
+// tiles streamed through LDS, QK^T and PV on MFMA, online softmax in fp32 registers.
+//
+// Replaces, behind the reference's GPU-backend slot, FlashAttentionV2 / FlashAttention /
+// ScaledDotProductAttention (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/HipBackend.cs:6118-6302,
+// kernel strings Kernels/HipAttentionKernels.cs:33-232); value semantics are the CPU engine's
+// (src/AiDotNet.Tensors/Engines/CpuEngine.cs:29146-29288, 27695-27881).
+//
+// Formulation (per workgroup: 128 query rows of one (batch, head); per wave: 32 query rows):
+//   S^T = K_tile * Q^T    MFMA rows = keys, cols = queries.  Lane l then holds query (l % 32)
+//                          and 16 keys per 32-key sub-tile, so the row max / sum of a query are
+//                          an in-lane reduction plus ONE cross-lane exchange (lane ^ 32), and the
+//                          rescale factor of the output accumulator is a per-lane scalar.
+//   O^T += V_tile^T * P^T  MFMA rows = head-dim, cols = queries.  P^T in accumulator layout is
+//                          already the B-operand fragment (each lane owns the keys it needs), no
+//                          shuffles; V is transposed on its way into LDS ([d][key], keys of one
+//                          16-group stored in fragment order so a lane's 8 keys are 16 contiguous
+//                          bytes).
+// K/V tiles are double-buffered in LDS: global loads of tile j+1 are issued before the MFMAs of
+// tile j and stored after them, one barrier per tile.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace aidn {
+
+struct AttnArgs {
+    const void* q; const void* k; const void* v; void* o;
+    float* lse; const float* bias; const float* mask;
+    int B, H, Hkv, Sq, Sk, D;
+    float scale; int causal; int qoff; float softcap; int mask_mode;
+    long long bias_bs;
+    long long qs[3], ks[3], vs[3], os[3];
+    int qtiles;
+    int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
+    int vec_out;
+};
+
+template <typename T> struct Raw2;
+template <> struct Raw2<float> { typedef uint32_t type; };
+template <> struct Raw2<f16_t> { typedef uint16_t type; };
+template <> struct Raw2<bf16_t> { typedef uint16_t type; };
+
+// 16 bytes = PER16 consecutive elements from p; elements at index >= valid read as zero.
+template <typename T>
+__device__ __forceinline__ u32x4 ld16(const typename Raw2<T>::type* p, int valid, bool vec)
+{
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (valid <= 0) return v;
+    if (vec && valid >= Elem<T>::PER16) return *(const u32x4*)p;
+    if constexpr (Elem<T>::BYTES == 4) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) if (e < valid) v[e] = p[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) if (e < valid) v[e >> 1] |= ((uint32_t)p[e]) << (16 * (e & 1));
+    }
+    return v;
+}
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
+template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB>
+__global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
+{
+    typedef typename Raw2<T>::type raw_t;
+    constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
+    constexpr int NT = 256, BR = 128;
+    constexpr int KS = Mma32<T>::KS;
+    constexpr int DSTEPS = DP / KS;            // fragment steps over the head dim (QK^T)
+    constexpr int KPITCH = DP * EB + 16;       // K tile [key][d] row pitch, bytes
+    constexpr int VPITCH = BC * EB + 16;       // V^T tile [d][key] row pitch, bytes
+    constexpr int KBYTES = BC * KPITCH, VBYTES = DP * VPITCH;
+    constexpr int KT = BC / 32;                // 32-key sub-tiles per tile
+    constexpr int DT = DP / 32;                // 32-row tiles of O^T
+    constexpr int PSTEPS = 32 / KS;            // PV fragment steps per key sub-tile
+    constexpr int CPR = DP / E;                // 16-byte chunks per K row
+    constexpr int NKC = BC * CPR;              // K chunks per tile
+    constexpr int UK = (NKC + NT - 1) / NT;
+    constexpr int NVU = (BC / 4) * CPR;        // V units: 4 keys x E head-dim elements
+    constexpr int UV = (NVU + NT - 1) / NT;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    unsigned char* Ks = smem;                  // [2][KBYTES]
+    unsigned char* Vs = smem + 2 * KBYTES;     // [2][VBYTES]
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+
+    // workgroup -> (batch*head, query tile): XCD-contiguous so the q-tiles of one head share an L2;
+    // late (heavy, under a causal mask) query tiles first.
+    int bh, qt;
+    {
+        int nblk = gridDim.x, pid = blockIdx.x;
+        int per = nblk >> 3, rem = nblk & 7;
+        int xcd = pid & 7, idx = pid >> 3;
+        int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+        bh = logical / a.qtiles;
+        qt = a.qtiles - 1 - (logical - bh * a.qtiles);
+    }
+    const int b = bh / a.H, hd = bh - b * a.H;
+    const int kvh = hd / (a.H / a.Hkv);
+    const int q0 = qt * BR;
+    const int qi = q0 + wave * 32 + l32;       // this lane's query row
+    const bool vec = a.vec_in != 0;
+
+    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
+    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+
+    // ---- Q fragments (B operand of S^T): row qi, 16-byte chunk (2 s + h)
+    u32x4 qf[DSTEPS];
+#pragma unroll
+    for (int s = 0; s < DSTEPS; s++) {
+        int d0 = (2 * s + h) * E;
+        qf[s] = (qi < a.Sq) ? ld16<T>(Q + (long long)qi * a.qs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+    }
+
+    // ---- number of K/V tiles this query tile needs
+    int ntiles = (a.Sk + BC - 1) / BC;
+    if (a.causal) {
+        long long lastkey = (long long)q0 + BR - 1 + a.qoff;      // largest unmasked key of the tile's last row
+        if (lastkey < 0) ntiles = 0;
+        else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
+    }
+
+    u32x4 rk[UK];
+    u32x4 rv[UV * 4];
+
+    auto load_tile = [&](int kv0) {
+#pragma unroll
+        for (int i = 0; i < UK; i++) {
+            int u = t + i * NT;
+            int row = u / CPR, ch = u - row * CPR;
+            int key = kv0 + row, d0 = ch * E;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if ((NKC % NT == 0 || u < NKC) && key < a.Sk) v = ld16<T>(K + (long long)key * a.ks[2] + d0, a.D - d0, vec);
+            rk[i] = v;
+        }
+#pragma unroll
+        for (int i = 0; i < UV; i++) {
+            int u = t + i * NT;
+            int kb = u % (BC / 4), db = u / (BC / 4);
+            int d0 = db * E;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                int key = kv0 + kb * 4 + r;
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if ((NVU % NT == 0 || u < NVU) && key < a.Sk) v = ld16<T>(V + (long long)key * a.vs[2] + d0, a.D - d0, vec);
+                rv[i * 4 + r] = v;
+            }
+        }
+    };
+
+    auto store_tile = [&](int stage) {
+        unsigned char* ks = Ks + stage * KBYTES;
+        unsigned char* vs = Vs + stage * VBYTES;
+#pragma unroll
+        for (int i = 0; i < UK; i++) {
+            int u = t + i * NT;
+            int row = u / CPR, ch = u - row * CPR;
+            if (NKC % NT == 0 || u < NKC) *(u32x4*)(ks + row * KPITCH + ch * 16) = rk[i];
+        }
+#pragma unroll
+        for (int i = 0; i < UV; i++) {
+            int u = t + i * NT;
+            int kb = u % (BC / 4), db = u / (BC / 4);
+            if (NVU % NT == 0 || u < NVU) {
+                if constexpr (E == 8) {
+                    // 4 keys x 8 d  ->  8 rows (d) of 4 keys (8 bytes).  Keys of a 16-group are stored
+                    // in fragment order: 4-key blocks (0,1,2,3) at block positions (0,2,1,3).
+                    int blk = kb & 3;
+                    int pblk = ((blk & 1) << 1) | (blk >> 1);
+                    int kpos = (kb >> 2) * 16 + pblk * 4;              // in elements
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        uint32_t a0 = rv[i * 4 + 0][c >> 1], a1 = rv[i * 4 + 1][c >> 1];
+                        uint32_t a2 = rv[i * 4 + 2][c >> 1], a3 = rv[i * 4 + 3][c >> 1];
+                        u32x2 o;
+                        if (c & 1) { o[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302u); o[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302u); }
+                        else       { o[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100u); o[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100u); }
+                        *(u32x2*)(vs + (db * 8 + c) * VPITCH + kpos * 2) = o;
+                    }
+                } else {
+                    // 4 keys x 4 d -> 4 rows (d) of 4 keys (16 bytes), natural key order
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        u32x4 o = {rv[i * 4 + 0][c], rv[i * 4 + 1][c], rv[i * 4 + 2][c], rv[i * 4 + 3][c]};
+                        *(u32x4*)(vs + (db * 4 + c) * VPITCH + kb * 16) = o;
+                    }
+                }
+            }
+        }
+    };
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.0f;
+    float m_run = -INFINITY;     // running max of the log2-domain logits of query qi (same in lanes l and l^32)
+    float l_run = 0.0f;          // this lane's share of the running sum
+
+    const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
+    const float sl2 = a.scale * LOG2E;
+
+    if (ntiles > 0) {
+        load_tile(0);
+        store_tile(0);
+    }
+    __syncthreads();
+
+    for (int j = 0; j < ntiles; j++) {
+        const int stage = j & 1;
+        const int kv0 = j * BC;
+        if (j + 1 < ntiles) load_tile(kv0 + BC);
+
+        // a wave whose 32 rows are all above the causal diagonal of this tile only helps with the copies
+        const bool active = !(a.causal && (long long)kv0 > (long long)wq_max + a.qoff);
+        if (active) {
+            const unsigned char* ks = Ks + stage * KBYTES + l32 * KPITCH + h * 16;
+            const unsigned char* vs = Vs + stage * VBYTES + l32 * VPITCH + h * 16;
+
+            f32x16 st[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) st[kt][r] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < DSTEPS; s++) {
+#pragma unroll
+                for (int kt = 0; kt < KT; kt++) {
+                    u32x4 kf = *(const u32x4*)(ks + kt * 32 * KPITCH + s * 32);
+                    Mma32<T>::run(st[kt], kf, qf[s]);
+                }
+            }
+
+            // ---- logits in the log2 domain, masks
+            const bool need_mask = (kv0 + BC > a.Sk) || (a.causal && (long long)kv0 + BC - 1 > (long long)wq_min + a.qoff);
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float x;
+                    const int key = kv0 + kt * 32 + acc_row(r, h);
+                    if constexpr (FULL) {
+                        x = st[kt][r] * a.scale;
+                        if (a.softcap > 0.0f) x = a.softcap * tanhf(x / a.softcap);
+                        const bool inb = qi < a.Sq && key < a.Sk;
+                        if (a.bias && inb) x += a.bias[b * a.bias_bs + ((long long)hd * a.Sq + qi) * a.Sk + key];
+                        if (a.mask_mode != 0 && inb) {
+                            long long mi = (a.mask_mode == 2 ? ((long long)bh * a.Sq + qi) : (long long)qi) * a.Sk + key;
+                            if (a.mask[mi] == 0.0f) x = -INFINITY;
+                        }
+                        x *= LOG2E;
+                    } else {
+                        x = st[kt][r] * sl2;
+                    }
+                    if (need_mask) {
+                        if (key >= a.Sk || (a.causal && (long long)key > (long long)qi + a.qoff)) x = -INFINITY;
+                    }
+                    st[kt][r] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+            }
+            mloc = fmaxf(mloc, shfl_xor_f(mloc, 32));
+            const float m_new = fmaxf(m_run, mloc);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+            m_run = m_new;
+
+            float psum = 0.0f;
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float p = __builtin_amdgcn_exp2f(st[kt][r] - m_use);
+                    st[kt][r] = p;
+                    psum += p;
+                }
+            l_run = l_run * alpha + psum;
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+
+            // ---- O^T += V^T * P^T
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++) {
+#pragma unroll
+                for (int ps = 0; ps < PSTEPS; ps++) {
+                    u32x4 pf;
+                    if constexpr (E == 8) {
+#pragma unroll
+                        for (int w = 0; w < 4; w++)
+                            pf[w] = Elem<T>::narrow(st[kt][8 * ps + 2 * w]) | (Elem<T>::narrow(st[kt][8 * ps + 2 * w + 1]) << 16);
+                    } else {
+#pragma unroll
+                        for (int w = 0; w < 4; w++) pf[w] = __builtin_bit_cast(uint32_t, st[kt][4 * ps + w]);
+                    }
+#pragma unroll
+                    for (int i = 0; i < DT; i++) {
+                        u32x4 vf = *(const u32x4*)(vs + i * 32 * VPITCH + kt * 32 * EB + ps * 32);
+                        Mma32<T>::run(oacc[i], vf, pf);
+                    }
+                }
+            }
+        }
+        if (j + 1 < ntiles) store_tile(stage ^ 1);
+        __syncthreads();
+    }
+
+    // ---- normalise and store: lane holds query qi, head-dim elements i*32 + 8 g + 4 h + (0..3)
+    const float l_tot = l_run + shfl_xor_f(l_run, 32);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (qi < a.Sq) {
+        typedef typename Raw2<OutT>::type out_t;
+        out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
+#pragma unroll
+        for (int i = 0; i < DT; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = i * 32 + 8 * g + 4 * h;
+                float v0 = oacc[i][4 * g + 0] * inv, v1 = oacc[i][4 * g + 1] * inv;
+                float v2 = oacc[i][4 * g + 2] * inv, v3 = oacc[i][4 * g + 3] * inv;
+                if constexpr (Elem<OutT>::BYTES == 4) {
+                    if (a.vec_out && d0 + 4 <= a.D) {
+                        *(f32x4*)(O + d0) = f32x4{v0, v1, v2, v3};
+                    } else {
+                        if (d0 + 0 < a.D) O[d0 + 0] = __builtin_bit_cast(uint32_t, v0);
+                        if (d0 + 1 < a.D) O[d0 + 1] = __builtin_bit_cast(uint32_t, v1);
+                        if (d0 + 2 < a.D) O[d0 + 2] = __builtin_bit_cast(uint32_t, v2);
+                        if (d0 + 3 < a.D) O[d0 + 3] = __builtin_bit_cast(uint32_t, v3);
+                    }
+                } else {
+                    uint32_t w0 = Elem<OutT>::narrow(v0) | (Elem<OutT>::narrow(v1) << 16);
+                    uint32_t w1 = Elem<OutT>::narrow(v2) | (Elem<OutT>::narrow(v3) << 16);
+                    if (a.vec_out && d0 + 4 <= a.D) {
+                        *(u32x2*)(O + d0) = u32x2{w0, w1};
+                    } else {
+                        if (d0 + 0 < a.D) O[d0 + 0] = (out_t)(w0 & 0xFFFFu);
+                        if (d0 + 1 < a.D) O[d0 + 1] = (out_t)(w0 >> 16);
+                        if (d0 + 2 < a.D) O[d0 + 2] = (out_t)(w1 & 0xFFFFu);
+                        if (d0 + 3 < a.D) O[d0 + 3] = (out_t)(w1 >> 16);
+                    }
+                }
+            }
+        }
+        if (a.lse && h == 0)
+            a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+    }
+}
+
+// Normalised probabilities P[b,h,i,j] = exp(logit - LSE[b,h,i]) for callers that ask for the
+// attention-weights tensor (the optional output of ScaledDotProductAttention,
+// src/AiDotNet.Tensors/Engines/DirectGpu/IDirectGpuBackend.cs:1421-1424).  Not on the hot path:
+// one thread per (row, key), fp32 dot product.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_weights_kernel(const AttnArgs a, float* __restrict__ w)
+{
+    typedef typename Raw2<T>::type raw_t;
+    long long total = (long long)a.B * a.H * a.Sq * a.Sk;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (long long)gridDim.x * blockDim.x) {
+        int key = (int)(idx % a.Sk);
+        long long row = idx / a.Sk;
+        int qi = (int)(row % a.Sq);
+        int bh = (int)(row / a.Sq);
+        int b = bh / a.H, hd = bh - b * a.H;
+        int kvh = hd / (a.H / a.Hkv);
+        const raw_t* q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1] + (long long)qi * a.qs[2];
+        const raw_t* k = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1] + (long long)key * a.ks[2];
+        float s = 0.0f;
+        for (int d = 0; d < a.D; d++) {
+            float qv, kv;
+            if constexpr (Elem<T>::BYTES == 4) { qv = __builtin_bit_cast(float, q[d]); kv = __builtin_bit_cast(float, k[d]); }
+            else { qv = Elem<T>::widen(q[d]); kv = Elem<T>::widen(k[d]); }
+            s += qv * kv;
+        }
+        float x = s * a.scale;
+        if (a.softcap > 0.0f) x = a.softcap * tanhf(x / a.softcap);
+        if (a.bias) x += a.bias[b * a.bias_bs + ((long long)hd * a.Sq + qi) * a.Sk + key];
+        bool masked = false;
+        if (a.mask_mode != 0) {
+            long long mi = (a.mask_mode == 2 ? ((long long)bh * a.Sq + qi) : (long long)qi) * a.Sk + key;
+            masked = a.mask[mi] == 0.0f;
+        }
+        if (a.causal && (long long)key > (long long)qi + a.qoff) masked = true;
+        float lse = a.lse[row];
+        w[idx] = (masked || lse == -INFINITY) ? 0.0f : __expf(x - lse);
+    }
+}
+
+// ------------------------------------------------------------------ host side
+template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB>
+static hipError_t launch_attn(AttnArgs a, hipStream_t stream)
+{
+    auto kern = attn_fwd_kernel<T, OutT, DP, BC, FULL, MINB>;
+    constexpr int EB = Elem<T>::BYTES;
+    constexpr int smem = 2 * (BC * (DP * EB + 16) + DP * (BC * EB + 16));
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    a.qtiles = (a.Sq + 127) / 128;
+    long long nblk = (long long)a.qtiles * a.B * a.H;
+    if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
+    return hipGetLastError();
+}
+
+template <typename T, typename OutT, int BC>
+static hipError_t dispatch_attn_d(const AttnArgs& a, bool full, hipStream_t stream)
+{
+    const int D = a.D;
+    if (D <= 32)  return full ? launch_attn<T, OutT, 32, BC, true, 2>(a, stream)  : launch_attn<T, OutT, 32, BC, false, 2>(a, stream);
+    if (D <= 64)  return full ? launch_attn<T, OutT, 64, BC, true, 2>(a, stream)  : launch_attn<T, OutT, 64, BC, false, 2>(a, stream);
+    if (D <= 128) return full ? launch_attn<T, OutT, 128, BC, true, 2>(a, stream) : launch_attn<T, OutT, 128, BC, false, 2>(a, stream);
+    if (D <= 256) return full ? launch_attn<T, OutT, 256, BC, true, 1>(a, stream) : launch_attn<T, OutT, 256, BC, false, 1>(a, stream);
+    return hipErrorInvalidValue;
+}
+
+// kind: 0 fp32, 1 fp16, 2 bf16
+hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
+{
+    AttnArgs a;
+    a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
+    a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
+    a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;
+    a.bias_bs = p.bias_bs;
+    for (int i = 0; i < 3; i++) { a.qs[i] = p.qs[i]; a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; a.os[i] = p.os[i]; }
+    a.qtiles = 0;
+    const int eb = kind == 0 ? 4 : 2, e = 16 / eb;
+    const int oeb = (kind == 0 || !p.out16) ? 4 : 2;
+    auto al = [](const void* ptr, const long long* s, int bytes) {
+        return ((uintptr_t)ptr & 15u) == 0 && (s[0] * bytes) % 16 == 0 && (s[1] * bytes) % 16 == 0 && (s[2] * bytes) % 16 == 0;
+    };
+    a.vec_in = (p.D % e == 0) && al(p.q, p.qs, eb) && al(p.k, p.ks, eb) && al(p.v, p.vs, eb);
+    a.vec_out = (p.D % 4 == 0) && al(p.o, p.os, oeb);
+    const bool full = p.bias != nullptr || a.mask_mode != 0 || p.softcap > 0.0f;
+    hipError_t err;
+    if (kind == 0) err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    else if (kind == 1) err = p.out16 ? dispatch_attn_d<f16_t, f16_t, 64>(a, full, stream) : dispatch_attn_d<f16_t, float, 64>(a, full, stream);
+    else err = p.out16 ? dispatch_attn_d<bf16_t, bf16_t, 64>(a, full, stream) : dispatch_attn_d<bf16_t, float, 64>(a, full, stream);
+    if (err != hipSuccess) return err;
+    if (p.weights) {
+        long long total = (long long)a.B * a.H * a.Sq * a.Sk;
+        unsigned grid = (unsigned)((total + 255) / 256 > 65535 ? 65535 : (total + 255) / 256);
+        a.lse = p.lse;
+        if (kind == 0) hipLaunchKernelGGL(attn_weights_kernel<float>, dim3(grid), dim3(256), 0, stream, a, p.weights);
+        else if (kind == 1) hipLaunchKernelGGL(attn_weights_kernel<f16_t>, dim3(grid), dim3(256), 0, stream, a, p.weights);
+        else hipLaunchKernelGGL(attn_weights_kernel<bf16_t>, dim3(grid), dim3(256), 0, stream, a, p.weights);
+        err = hipGetLastError();
+    }
+    return err;
+}
+
+}  // namespace aidn

@@ -1,0 +1,317 @@
+// Decode attention (one query row per (batch, head)) for gfx950.  HBM-bound: each K and V row is
+// read exactly once with 128-bit loads, LPK lanes per row so one wave load covers 64/LPK whole
+// consecutive rows (1 KiB contiguous when the cache is dense); no MFMA.
+//
+// Replaces FlashDecode (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/HipBackend.cs:919-965, kernel
+// strings Kernels/HipFlashDecodeKernels.cs:21-83: one THREAD per (head, split)) and the Sq == 1 use
+// of ScaledDotProductAttention (Kernels/HipAttentionKernels.cs:33-125).  Value semantics: the
+// reference decode test's oracle (tests/AiDotNet.Tensors.Tests/Engines/DirectGpu/
+// FlashDecodeHipTests.cs:43-69), i.e. softmax(scale * q.K^T) V over all cached keys.
+//
+// grid = (splits, B*H), 256 threads.  Wave w of the workgroup walks its split in blocks of
+// U * KPW keys (KPW = 64 / LPK keys per load, U loads in flight for K and U for V).  Every lane
+// keeps an online-softmax state (m, l, acc[E]) for its key slot and its 16-byte slice of the head
+// dim; slots and waves are merged through LDS, splits through a workspace and a second kernel.
+#include "common.hpp"
+#include "launch.hpp"
+
+namespace aidn {
+
+struct DecodeArgs {
+    const void* q; const void* k; const void* v; void* o; float* lse;
+    float* ws;               // [B*H][splits][2 + DPAD] : m, l, acc[DPAD]   (splits > 1)
+    int B, H, Hkv, Sk, D;
+    float scale;
+    int splits, chunk;       // keys per split
+    long long qs[2], ks[3], vs[3], os[2];   // q/o: batch, head; k/v: batch, head, row
+    int vec_in;
+};
+
+template <typename T> struct Raw3;
+template <> struct Raw3<float> { typedef uint32_t type; };
+template <> struct Raw3<f16_t> { typedef uint16_t type; };
+template <> struct Raw3<bf16_t> { typedef uint16_t type; };
+
+template <typename T>
+__device__ __forceinline__ u32x4 ld16d(const typename Raw3<T>::type* p, int valid, bool vec)
+{
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (valid <= 0) return v;
+    if (vec && valid >= Elem<T>::PER16) return *(const u32x4*)p;
+    if constexpr (Elem<T>::BYTES == 4) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) if (e < valid) v[e] = p[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; e++) if (e < valid) v[e >> 1] |= ((uint32_t)p[e]) << (16 * (e & 1));
+    }
+    return v;
+}
+
+// widen one 16-byte fragment to E floats
+template <typename T>
+__device__ __forceinline__ void widen16(const u32x4& x, float (&f)[Elem<T>::PER16])
+{
+    if constexpr (Elem<T>::BYTES == 4) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) f[e] = __builtin_bit_cast(float, x[e]);
+    } else {
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            f[2 * w] = Elem<T>::widen(x[w] & 0xFFFFu);
+            f[2 * w + 1] = Elem<T>::widen(x[w] >> 16);
+        }
+    }
+}
+
+constexpr float D_LOG2E = 1.4426950408889634f;
+constexpr float D_LN2 = 0.6931471805599453f;
+
+template <typename T, typename OutT, int LPK, int U>
+__global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
+{
+    typedef typename Raw3<T>::type raw_t;
+    constexpr int E = Elem<T>::PER16;
+    constexpr int KPW = 64 / LPK;          // keys per wave load
+    constexpr int NWV = 4;
+    constexpr int DPAD = LPK * E;          // padded head dim
+    constexpr int SLOTS = NWV * KPW;
+
+    __shared__ float s_m[SLOTS], s_l[SLOTS];
+    __shared__ float s_acc[SLOTS][DPAD + 4];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int dl = lane % LPK, sk = lane / LPK;
+    const int split = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / a.H, hd = bh - b * a.H;
+    const int kvh = hd / (a.H / a.Hkv);
+    const bool vec = a.vec_in != 0;
+    const int d0 = dl * E;
+
+    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
+
+    float qf[E];
+    {
+        u32x4 qx = ld16d<T>(Q + d0, a.D - d0, vec);
+        widen16<T>(qx, qf);
+        const float sl2 = a.scale * D_LOG2E;
+#pragma unroll
+        for (int e = 0; e < E; e++) qf[e] *= sl2;      // scores come out in the log2 domain
+    }
+
+    const int kbeg = split * a.chunk;
+    const int kend = min(a.Sk, kbeg + a.chunk);
+
+    float m_run = -INFINITY, l_run = 0.0f;
+    float acc[E];
+#pragma unroll
+    for (int e = 0; e < E; e++) acc[e] = 0.0f;
+
+    for (int base = kbeg + wave * (U * KPW); base < kend; base += NWV * U * KPW) {
+        u32x4 kx[U], vx[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            int key = base + u * KPW + sk;
+            bool ok = key < kend;
+            kx[u] = ok ? ld16d<T>(K + (long long)key * a.ks[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+            vx[u] = ok ? ld16d<T>(V + (long long)key * a.vs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+        }
+        float s[U];
+        float mloc = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float kf[E];
+            widen16<T>(kx[u], kf);
+            float p = 0.0f;
+#pragma unroll
+            for (int e = 0; e < E; e++) p = fmaf(qf[e], kf[e], p);
+#pragma unroll
+            for (int off = 1; off < LPK; off <<= 1) p += shfl_xor_f(p, off);
+            int key = base + u * KPW + sk;
+            s[u] = key < kend ? p : -INFINITY;
+            mloc = fmaxf(mloc, s[u]);
+        }
+        const float m_new = fmaxf(m_run, mloc);
+        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        m_run = m_new;
+        l_run *= alpha;
+#pragma unroll
+        for (int e = 0; e < E; e++) acc[e] *= alpha;
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float p = __builtin_amdgcn_exp2f(s[u] - m_use);
+            l_run += p;
+            float vf[E];
+            widen16<T>(vx[u], vf);
+#pragma unroll
+            for (int e = 0; e < E; e++) acc[e] = fmaf(p, vf[e], acc[e]);
+        }
+    }
+
+    // ---- merge the key slots of all waves
+    const int slot = wave * KPW + sk;
+    if (dl == 0) { s_m[slot] = m_run; s_l[slot] = l_run; }
+#pragma unroll
+    for (int e = 0; e < E; e++) s_acc[slot][d0 + e] = acc[e];
+    __syncthreads();
+
+    float M = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < SLOTS; i++) M = fmaxf(M, s_m[i]);
+    const float Muse = (M == -INFINITY) ? 0.0f : M;
+    for (int d = t; d < DPAD; d += 256) {
+        float L = 0.0f, A = 0.0f;
+#pragma unroll
+        for (int i = 0; i < SLOTS; i++) {
+            float w = __builtin_amdgcn_exp2f(s_m[i] - Muse);
+            L += s_l[i] * w;
+            A += s_acc[i][d] * w;
+        }
+        if (a.splits > 1) {
+            float* ws = a.ws + ((long long)bh * a.splits + split) * (2 + DPAD);
+            if (d == 0) { ws[0] = M; ws[1] = L; }
+            ws[2 + d] = A;
+        } else if (d < a.D) {
+            typedef typename Raw3<OutT>::type out_t;
+            out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
+            float r = L > 0.0f ? A / L : 0.0f;
+            if constexpr (Elem<OutT>::BYTES == 4) O[d] = __builtin_bit_cast(uint32_t, r);
+            else O[d] = (out_t)Elem<OutT>::narrow(r);
+            if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
+        }
+    }
+}
+
+// Merge the per-split (m, l, acc) triples: grid = B*H, one thread per head-dim element.
+template <typename OutT>
+__global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a, int dpad)
+{
+    const int bh = blockIdx.x;
+    const int b = bh / a.H, hd = bh - b * a.H;
+    const float* ws = a.ws + (long long)bh * a.splits * (2 + dpad);
+    float M = -INFINITY;
+    for (int s = 0; s < a.splits; s++) M = fmaxf(M, ws[(long long)s * (2 + dpad)]);
+    const float Muse = (M == -INFINITY) ? 0.0f : M;
+    for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
+        float L = 0.0f, A = 0.0f;
+        for (int s = 0; s < a.splits; s++) {
+            const float* p = ws + (long long)s * (2 + dpad);
+            float w = __builtin_amdgcn_exp2f(p[0] - Muse);
+            L += p[1] * w;
+            A += p[2 + d] * w;
+        }
+        typedef typename Raw3<OutT>::type out_t;
+        out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
+        float r = L > 0.0f ? A / L : 0.0f;
+        if constexpr (Elem<OutT>::BYTES == 4) O[d] = __builtin_bit_cast(uint32_t, r);
+        else O[d] = (out_t)Elem<OutT>::narrow(r);
+        if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
+    }
+}
+
+// ------------------------------------------------------------------ host side
+static int lanes_per_key(int D, int eb)
+{
+    int chunks = (D * eb + 15) / 16;
+    int lpk = 1;
+    while (lpk < chunks) lpk <<= 1;
+    return lpk;
+}
+
+static int effective_sk(const AttnParams& p)
+{
+    // Sq == 1: key j is masked iff j > 0 + qoff
+    if (!p.causal) return p.Sk;
+    long long lim = (long long)p.qoff + 1;
+    if (lim < 0) lim = 0;
+    return (int)(lim < p.Sk ? lim : p.Sk);
+}
+
+int attn_decode_splits(const AttnParams& p, int splits)
+{
+    const int sk = effective_sk(p);
+    int maxs = (sk + 255) / 256;            // at least 256 keys per split
+    if (maxs < 1) maxs = 1;
+    if (splits <= 0) {
+        long long bh = (long long)p.B * p.H;
+        splits = (int)((2048 + bh - 1) / bh);   // ~8 workgroups per CU
+    }
+    if (splits > maxs) splits = maxs;
+    if (splits > 64) splits = 64;
+    if (splits < 1) splits = 1;
+    return splits;
+}
+
+size_t attn_decode_workspace_bytes(const AttnParams& p, int eff_splits)
+{
+    if (eff_splits <= 1) return 0;
+    // padded head dim of whichever element size is used: take the larger of the two
+    int l4 = lanes_per_key(p.D, 4), l2 = lanes_per_key(p.D, 2);
+    if (l4 < 4) l4 = 4;
+    if (l2 < 4) l2 = 4;
+    int dpad = l4 * 4 > l2 * 8 ? l4 * 4 : l2 * 8;
+    return (size_t)p.B * p.H * eff_splits * (2 + dpad) * sizeof(float);
+}
+
+template <typename T, typename OutT, int LPK, int U>
+static hipError_t launch_decode(DecodeArgs a, hipStream_t stream)
+{
+    constexpr int DPAD = LPK * Elem<T>::PER16;
+    dim3 grid((unsigned)a.splits, (unsigned)(a.B * a.H));
+    hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U>), grid, dim3(256), 0, stream, a);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    if (a.splits > 1) {
+        int threads = a.D <= 64 ? 64 : (a.D <= 128 ? 128 : 256);
+        hipLaunchKernelGGL((decode_reduce_kernel<OutT>), dim3((unsigned)(a.B * a.H)), dim3(threads), 0, stream, a, DPAD);
+        e = hipGetLastError();
+    }
+    return e;
+}
+
+template <typename T, typename OutT>
+static hipError_t dispatch_decode(const DecodeArgs& a, hipStream_t stream)
+{
+    const int lpk = lanes_per_key(a.D, Elem<T>::BYTES);
+    switch (lpk) {
+    case 1: case 2: case 4: return launch_decode<T, OutT, 4, 4>(a, stream);
+    case 8: return launch_decode<T, OutT, 8, 4>(a, stream);
+    case 16: return launch_decode<T, OutT, 16, 4>(a, stream);
+    case 32: return launch_decode<T, OutT, 32, 4>(a, stream);
+    case 64: return launch_decode<T, OutT, 64, 4>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t attn_decode(hipStream_t stream, int kind, const AttnParams& p, int eff_splits, void* workspace)
+{
+    DecodeArgs a;
+    a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.ws = (float*)workspace;
+    a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sk = effective_sk(p); a.D = p.D;
+    a.scale = p.scale;
+    a.splits = eff_splits;
+    a.qs[0] = p.qs[0]; a.qs[1] = p.qs[1]; a.os[0] = p.os[0]; a.os[1] = p.os[1];
+    for (int i = 0; i < 3; i++) { a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; }
+    const int eb = kind == 0 ? 4 : 2, e = 16 / eb;
+    const int lpk = lanes_per_key(p.D, eb) < 4 ? 4 : lanes_per_key(p.D, eb);
+    // keys per split: a multiple of the keys one workgroup iteration covers
+    const int step = 4 * 4 * (64 / lpk);
+    int chunk = (a.Sk + eff_splits - 1) / eff_splits;
+    chunk = ((chunk + step - 1) / step) * step;
+    if (chunk < step) chunk = step;
+    a.chunk = chunk;
+    auto al = [](const void* ptr, const long long* s, int n, int bytes) {
+        bool ok = ((uintptr_t)ptr & 15u) == 0;
+        for (int i = 0; i < n; i++) ok = ok && (s[i] * bytes) % 16 == 0;
+        return ok;
+    };
+    a.vec_in = (p.D % e == 0) && al(p.q, p.qs, 2, eb) && al(p.k, p.ks, 3, eb) && al(p.v, p.vs, 3, eb);
+    if (kind == 0) return dispatch_decode<float, float>(a, stream);
+    if (kind == 1) return p.out16 ? dispatch_decode<f16_t, f16_t>(a, stream) : dispatch_decode<f16_t, float>(a, stream);
+    return p.out16 ? dispatch_decode<bf16_t, bf16_t>(a, stream) : dispatch_decode<bf16_t, float>(a, stream);
+}
+
+}  // namespace aidn

@@ -1,0 +1,35 @@
+// Host-side launchers shared between the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace aidn {
+
+hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
+                    float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
+                    int force_tile);
+hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                   int M, int N, int K, int force_tile);
+
+// kind: 0 f32->f16, 1 f16->f32, 2 f32->bf16, 3 bf16->f32
+hipError_t convert(hipStream_t stream, int kind, const void* in, void* out, long long n);
+
+// Attention problem description shared by the prefill and decode launchers (host side).
+struct AttnParams {
+    const void* q; const void* k; const void* v; void* o;
+    float* lse; const float* bias; const float* mask; float* weights;
+    int B, H, Hkv, Sq, Sk, D;
+    float scale; int causal; int qoff; float softcap; int mask_mode; int out16;
+    long long bias_bs;
+    long long qs[3], ks[3], vs[3], os[3];   // batch, head, row strides in elements
+};
+
+// kind: 0 fp32, 1 fp16, 2 bf16
+hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p);
+
+// Decode (Sq == 1).  eff_splits: the split count actually used for `splits` requested (<= 0 = auto).
+int attn_decode_splits(const AttnParams& p, int splits);
+size_t attn_decode_workspace_bytes(const AttnParams& p, int eff_splits);
+hipError_t attn_decode(hipStream_t stream, int kind, const AttnParams& p, int eff_splits, void* workspace);
+
+}  // namespace aidn

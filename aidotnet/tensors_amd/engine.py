@@ -1,0 +1,150 @@
+"""Operator-level mirror of the reference's GPU tensor engine for the hot path.
+
+``Mi355Engine`` keeps the operator names and shape rules of ``IEngine`` /
+``DirectGpuTensorEngine`` for the members on the path
+(src/AiDotNet.Tensors/Engines/IEngine.cs:3186 TensorMatMul, :4133-4140 ScaledDotProductAttention,
+:4587-4594 FlashAttention; routing src/AiDotNet.Tensors/Engines/DirectGpuTensorEngine.cs:19660-19857,
+19987-20019, 10966-11089, 11436-11548) on device-resident ``torch`` tensors, and calls the backend
+members of :class:`Mi355Backend`.  Unlike the reference there is no CPU fallback: a failure raises
+(the behaviour of ``ThrowOnGpuKernelFallback = true``, DirectGpuTensorEngine.cs:19850-19856).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from .backend import ArgumentException, ArgumentNullException, Mi355Backend, NotSupportedException
+
+_KIND = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}
+
+
+class Mi355Engine:
+    def __init__(self, backend: Optional[Mi355Backend] = None):
+        self.backend = backend or Mi355Backend()
+
+    # ------------------------------------------------------------------ MatMul
+    def TensorMatMul(self, a: torch.Tensor, b: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """rank-2 x rank-2, ND x 2D (leading dims collapse into M) and ND x ND of equal rank
+        (batched), as CpuEngine.TensorMatMul (CpuEngine.cs:12458-12575).  fp16 / bf16 inputs use
+        fp32 accumulation; out_dtype float32 selects the fp32-output route (GemmFp16In32fOut)."""
+        if a is None or b is None:
+            raise ArgumentNullException("a" if a is None else "b")
+        if a.dim() < 2 or b.dim() < 2:
+            raise ArgumentException("TensorMatMul requires tensors of rank >= 2")
+        if a.dtype != b.dtype or a.dtype not in _KIND:
+            raise NotSupportedException("TensorMatMul: unsupported dtype combination %s x %s" % (a.dtype, b.dtype))
+        if a.shape[-1] != b.shape[-2]:
+            raise ArgumentException("inner dimensions do not match: %s x %s" % (tuple(a.shape), tuple(b.shape)))
+        be = self.backend
+        a = a.contiguous(); b = b.contiguous()
+        K, N = b.shape[-2], b.shape[-1]
+        out_dtype = out_dtype or a.dtype
+        if b.dim() == 2:
+            M = a.numel() // K
+            out = torch.empty(*a.shape[:-1], N, dtype=out_dtype, device=a.device)
+            A, B, C = be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(out)
+            if a.dtype == torch.float32:
+                be.Gemm(A, B, C, M, N, K)
+            elif a.dtype == torch.float16:
+                (be.GemmFp16In32fOut if out_dtype == torch.float32 else be.Hgemm)(A, B, C, M, N, K)
+            else:
+                (be.GemmBf16In32fOut if out_dtype == torch.float32 else be.Bf16Gemm)(A, B, C, M, N, K)
+            return out
+        if a.dim() != b.dim() or a.shape[:-2] != b.shape[:-2]:
+            raise ArgumentException("batched TensorMatMul needs equal leading dimensions")
+        return self.BatchMatMul(a, b)
+
+    def BatchMatMul(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+        """[..., M, K] x [..., K, N], fp32 (DirectGpuTensorEngine.cs:19987-20019 -> BatchedGemm)."""
+        if a.dtype != torch.float32 or b.dtype != torch.float32:
+            raise NotSupportedException("BatchMatMul is fp32 only (as the reference's batched route)")
+        a = a.contiguous(); b = b.contiguous()
+        M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
+        batch = a.numel() // (M * K)
+        out = torch.empty(*a.shape[:-2], M, N, dtype=torch.float32, device=a.device)
+        be = self.backend
+        be.BatchedGemm(be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(out), M, N, K, batch)
+        return out
+
+    # ------------------------------------------------------------------ attention
+    def FlashAttention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, scale: Optional[float] = None,
+                       isCausal: bool = False, attentionBias: Optional[torch.Tensor] = None,
+                       queryOffset: int = 0) -> Tuple[torch.Tensor, torch.Tensor]:
+        """[B,H,Sq,d] x [B,H,Sk,d] -> (O [B,H,Sq,d], LSE [B,H,Sq]); top-left causal rule shifted by
+        queryOffset (IEngine.cs:4587-4594; CpuEngine.cs:28748, 29146-29288).  16-bit inputs give an
+        fp32 O and LSE."""
+        for t, n in ((query, "query"), (key, "key"), (value, "value")):
+            if t is None:
+                raise ArgumentNullException(n)
+            if t.dim() != 4:
+                raise ArgumentException("%s must be rank 4 [B,H,S,d]" % n)
+        B, H, Sq, D = query.shape
+        Sk = key.shape[2]
+        if key.shape != value.shape or key.shape[0] != B or key.shape[3] != D:
+            raise ArgumentException("key/value shapes do not match the query")
+        if isCausal and queryOffset + Sq > Sk:
+            raise ArgumentException("queryOffset + Sq exceeds Sk")       # FusedAttentionAuditTests.cs:81-92
+        if scale is None:
+            scale = 1.0 / math.sqrt(D)
+        be = self.backend
+        q = query.contiguous(); k = key.contiguous(); v = value.contiguous()
+        out = torch.empty(B, H, Sq, D, dtype=torch.float32, device=q.device)
+        lse = torch.empty(B, H, Sq, dtype=torch.float32, device=q.device)
+        kind = _KIND.get(q.dtype)
+        if kind is None:
+            raise NotSupportedException("unsupported dtype %s" % q.dtype)
+        if kind == "f32" and queryOffset == 0 and key.shape[1] == H:
+            bias = None
+            bstride = 0
+            if attentionBias is not None:
+                bias = be.WrapTensor(attentionBias.contiguous().float())
+                bstride = H * Sq * Sk if attentionBias.dim() == 4 else 0
+            be.FlashAttentionV2(be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), be.WrapTensor(lse),
+                                B, H, Sq, Sk, D, scale, isCausal, bias, bstride)
+        else:
+            if attentionBias is not None:
+                raise NotSupportedException("attention bias is available on the fp32 route only")
+            if kind == "f32":
+                from ._lib import AttnDesc
+                d = AttnDesc(B=B, H=H, Hkv=key.shape[1], Sq=Sq, Sk=Sk, D=D, scale=scale, causal=int(isCausal),
+                             causal_query_offset=queryOffset)
+                be._attn("f32", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), be.WrapTensor(lse),
+                         None, None, None, d)
+            else:
+                be.FlashAttentionHalf(kind, be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out),
+                                      be.WrapTensor(lse), B, H, Sq, Sk, D, scale, isCausal, queryOffset, key.shape[1])
+        return out, lse
+
+    def ScaledDotProductAttention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                  mask: Optional[torch.Tensor] = None, scale: Optional[float] = None,
+                                  softcap: float = 0.0, isCausal: bool = False,
+                                  returnWeights: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """fp32 SDPA with an optional boolean keep-mask broadcastable to [B,H,Sq,Sk] (true = keep) and
+        soft-cap; returns (O, weights) (IEngine.cs:4133-4140; CpuEngine.cs:27376, 27695-27881; GPU
+        route DirectGpuTensorEngine.MissingKernels.cs:6085-6140).  GQA is inferred from key.shape[1];
+        the causal rule is bottom-right (DirectGpuTensorEngine.cs:11501)."""
+        if query is None or key is None or value is None:
+            raise ArgumentNullException("query/key/value")
+        if query.dim() != 4 or query.dtype != torch.float32:
+            raise NotSupportedException("ScaledDotProductAttention GPU route is float + rank 4 only")
+        B, H, Sq, D = query.shape
+        Hkv, Sk = key.shape[1], key.shape[2]
+        if scale is None:
+            scale = 1.0 / math.sqrt(D)
+        be = self.backend
+        q = query.contiguous(); k = key.contiguous(); v = value.contiguous()
+        out = torch.empty(B, H, Sq, D, dtype=torch.float32, device=q.device)
+        w = torch.empty(B, H, Sq, Sk, dtype=torch.float32, device=q.device) if returnWeights else None
+        m = None
+        if mask is not None:
+            if mask.dim() != 4:
+                raise ArgumentException("mask must be rank 4, broadcastable to [B,H,Sq,Sk]")
+            shared = mask.shape[0] == 1 and mask.shape[1] == 1
+            full = mask.expand(1 if shared else B, 1 if shared else H, Sq, Sk)
+            m = be.WrapTensor(full.to(torch.float32).contiguous().reshape(-1))
+        be.ScaledDotProductAttention(be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out),
+                                     be.WrapTensor(w) if w is not None else None, m, B, H, Sq, Sk, D, scale,
+                                     isCausal, softcap, Hkv)
+        return out, w

@@ -1,0 +1,178 @@
+/*
+ * aidotnet_mi355.h -- C ABI of libaidotnet_mi355.so: hand-written gfx950 (MI355X) kernels for the
+ * GEMM and fused-attention members of AiDotNet.Tensors' GPU-backend slot.
+ *
+ * These are the entry points a P/Invoke binding in the reference's HIP backend would bind in
+ * place of its hipBLAS calls and run-time compiled kernel strings.  Paths below are relative to
+ * the reference checkout (src/AiDotNet.Tensors/...).
+ *
+ * Conventions (mirroring Engines/DirectGpu/HIP/HipNativeBindings.cs:13-87, 342-641 and
+ * HipBlasNative.cs:16-27, 82-157): cdecl, blittable arguments only, every function returns an int
+ * status (0 = success); all pointers are raw device pointers (IGpuBuffer.Handle,
+ * Engines/DirectGpu/IDirectGpuBackend.cs:3776-3803) owned by the caller and never retained;
+ * matrices are dense row-major; `stream` is a hipStream_t (NULL = the default stream).  Work is
+ * enqueued on `stream` and the call returns without waiting: a caller that keeps the reference's
+ * "result ready on return" contract (HipBackend.cs:1444-1446) calls aidn_mi355_sync afterwards.
+ * fp16 / bf16 values travel as raw 16-bit patterns (uint16_t).  Every output element is
+ * overwritten (pooled buffers may hold stale data; beta == 0 never reads C).
+ */
+#ifndef AIDOTNET_MI355_H
+#define AIDOTNET_MI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Exported with default visibility; everything else in the library is hidden. */
+#if defined(__GNUC__)
+#define AIDN_API __attribute__((visibility("default")))
+#else
+#define AIDN_API
+#endif
+
+/* Status codes. Values 1000+ are this library's; any other non-zero value is a hipError_t. */
+enum {
+    AIDN_OK = 0,
+    AIDN_ERR_INVALID_ARGUMENT = 1001,   /* null pointer, non-positive dimension, bad ratio */
+    AIDN_ERR_UNSUPPORTED = 1002,        /* e.g. head dimension the kernels do not cover */
+    AIDN_ERR_NO_DEVICE = 1003,          /* no gfx950 device */
+    AIDN_ERR_OUT_OF_MEMORY = 1004       /* library-owned workspace could not be allocated */
+};
+
+/* ---- lifetime ------------------------------------------------------------------------------
+ * One context per backend instance (the reference creates one stream + one hipBLAS handle per
+ * HipBackend, HipBackend.cs:246, 288, 371).  The context owns only the library's private
+ * workspace (split-KV partials); it is released by aidn_mi355_destroy. */
+AIDN_API int aidn_mi355_create(int device, void** ctx);
+AIDN_API int aidn_mi355_destroy(void* ctx);
+/* Text of the last failure on this context (never NULL; empty when none). */
+AIDN_API const char* aidn_mi355_last_error(void* ctx);
+AIDN_API const char* aidn_mi355_version(void);
+/* hipStreamSynchronize(stream): replaces HipBackend.Synchronize (HipBackend.cs:1444-1446). */
+AIDN_API int aidn_mi355_sync(void* ctx, void* stream);
+
+/* ---- fp32 GEMM -------------------------------------------------------------------------------
+ * C[M,N] = alpha * A[M,K] * op(B) + beta * C.  transB == 0: B is [K,N]; transB != 0: B is stored
+ * [N,K] (C = A * B^T).  Replaces IDirectGpuBackend.Gemm (IDirectGpuBackend.cs:160-172; host
+ * HipBackend.cs:1370-1447, hipblasSgemm :1502-1545) and MatMulTransposed (:184-203; host
+ * HipBackend.cs:1450-1490).  Argument order (M, N, K) as at that layer.  True fp32 MFMA, fp32
+ * accumulation (no TF32-style truncation). */
+AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
+                     int M, int N, int K, float alpha, float beta, int transB);
+
+/* batch independent products on concatenated matrices: A[i] is M x K at A + i*M*K, B[i] K x N,
+ * C[i] M x N.  Replaces IDirectGpuBackend.BatchedGemm (IDirectGpuBackend.cs:205-222; host
+ * HipBackend.cs:1599-1631). */
+AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, const float* B, float* C,
+                             int M, int N, int K, int batch, float alpha, float beta);
+
+/* ---- 16-bit GEMM, fp32 accumulation ------------------------------------------------------------
+ * C[M,N] = A[M,K] * B[K,N].  *_f32out replaces IGpuHalfPrecisionBackend.GemmFp16In32fOut
+ * (Engines/Gpu/IGpuHalfPrecisionBackend.cs:39-48; host HipBackend.HalfPrecision.cs:125-150,
+ * hipblasGemmEx); *_f16out replaces Hgemm (:27-37; host :97-122) with fp32 accumulation and one
+ * round-to-nearest-even narrow, the arithmetic of the CPU kernel (Engines/Simd/HalfKernels.cs:35-99).
+ * The bf16 pair has no member in the reference's backend interface today (its planner widens
+ * bf16 tensors to fp32, Engines/Gpu/GpuPrecisionPolicy.cs:497-532); it follows the CPU kernel
+ * Engines/Simd/BFloat16Kernels.cs:144-211 and NumericOperations/BFloat16.cs:64-90. */
+AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K);
+AIDN_API int aidn_mi355_hgemm_f16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K);
+AIDN_API int aidn_mi355_bf16gemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K);
+AIDN_API int aidn_mi355_bf16gemm_bf16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K);
+
+/* ---- storage conversions ------------------------------------------------------------------------
+ * Replace IDirectGpuBackend.ConvertToFp16 / ConvertToFp32 (IDirectGpuBackend.cs:1876-1911; host
+ * HipBackend.cs:11942-11981).  n = element count.  Narrowing is round-to-nearest-even; the bf16
+ * rule is BFloat16.FromFloat (NumericOperations/BFloat16.cs:64-82), NaN keeps a quiet bit. */
+AIDN_API int aidn_mi355_convert_f32_to_f16(void* ctx, void* stream, const float* in, uint16_t* out, int64_t n);
+AIDN_API int aidn_mi355_convert_f16_to_f32(void* ctx, void* stream, const uint16_t* in, float* out, int64_t n);
+AIDN_API int aidn_mi355_convert_f32_to_bf16(void* ctx, void* stream, const float* in, uint16_t* out, int64_t n);
+AIDN_API int aidn_mi355_convert_bf16_to_f32(void* ctx, void* stream, const uint16_t* in, float* out, int64_t n);
+
+/* ---- fused scaled-dot-product attention (forward) -------------------------------------------------
+ * O = softmax(scale * Q K^T (+ soft-cap, + bias, masks)) V per (batch, head), computed in tiles with
+ * an online softmax: the [Sq,Sk] score matrix is never written unless `weights` is requested.
+ *
+ * One descriptor covers IDirectGpuBackend.FlashAttentionV2 (IDirectGpuBackend.cs:1451-1471; host
+ * HipBackend.cs:6261-6302), FlashAttention (:1448-1449) and ScaledDotProductAttention
+ * (:1395-1424; host HipBackend.cs:6118-6175); the value semantics are the CPU engine's
+ * (Engines/CpuEngine.cs:29146-29288 and 27695-27881).
+ *
+ *   q [B,H,Sq,D], k and v [B,Hkv,Sk,D], o [B,H,Sq,D]; the head dimension is unit stride; the
+ *   batch / head / row strides are given in ELEMENTS (0 in every stride of a tensor = dense).
+ *   H % Hkv == 0; query head h reads kv head h / (H / Hkv)  (HipAttentionKernels.cs:60-66).
+ *   lse      [B,H,Sq] fp32 or NULL: max + log(sum) per row (CpuEngine.cs:29262-29263); -inf for a
+ *            row with every key masked, whose output row is all zeros (CpuEngine.cs:29243-29249).
+ *   causal   != 0: key j is masked iff j > i + causal_query_offset.  Offset 0 is the top-left rule
+ *            of FlashAttention / FlashAttentionV2 (CpuEngine.cs:29235, HipAttentionKernels.cs:199);
+ *            offset Sk - Sq is the bottom-right rule of ScaledDotProductAttention
+ *            (HipAttentionKernels.cs:69-71); same parameter as FlashAttentionConfig.QueryOffset
+ *            (Engines/Autodiff/FlashAttention2.cs:58-60, 123, 144-145).
+ *   bias     additive fp32 [B,H,Sq,Sk] (bias_batch_stride = H*Sq*Sk) or [H,Sq,Sk]
+ *            (bias_batch_stride = 0), added after the scale, or NULL (IDirectGpuBackend.cs:1465-1466).
+ *   mask     fp32, 0.0f = masked, anything else = keep (HipAttentionKernels.cs:78); mask_mode 0 none,
+ *            1 one [Sq,Sk] plane shared by all (batch, head), 2 full [B,H,Sq,Sk]
+ *            (HipBackend.cs:6150-6151).
+ *   softcap  > 0: logit = softcap * tanh(scale * qk / softcap) before bias / masks
+ *            (CpuEngine.cs:27806-27807); 0 disables.
+ *   weights  fp32 [B,H,Sq,Sk] normalised probabilities or NULL (the optional attentionWeights of
+ *            ScaledDotProductAttention); written by a second pass from the saved LSE.
+ * 16-bit variants: q, k, v are fp16 / bf16 patterns, softmax and accumulation are fp32, the output
+ * is fp32 (out_is_16bit == 0; the reference's only reduced-precision attention contract: fp16 in,
+ * fp32 O and LSE out, Engines/DirectGpuTensorEngine.cs:11143-11167) or the input type
+ * (out_is_16bit != 0).  D must be a multiple of 16 (16-bit) / 8 (fp32) and at most 256
+ * (GpuKernelGuards.MaxHeadDim, Engines/DirectGpu/GpuKernelGuards.cs:12), else AIDN_ERR_UNSUPPORTED.
+ */
+typedef struct aidn_attn_desc {
+    int32_t B, H, Hkv, Sq, Sk, D;
+    float scale;
+    int32_t causal;
+    int32_t causal_query_offset;
+    float softcap;
+    int32_t mask_mode;
+    int32_t out_is_16bit;
+    int64_t bias_batch_stride;
+    int64_t q_strides[3];   /* batch, head, row (elements); all zero = dense [B,H,Sq,D] */
+    int64_t k_strides[3];
+    int64_t v_strides[3];
+    int64_t o_strides[3];
+} aidn_attn_desc;
+
+AIDN_API int aidn_mi355_attn_fwd_f32(void* ctx, void* stream, const aidn_attn_desc* desc,
+                            const float* q, const float* k, const float* v, float* o,
+                            float* lse, const float* bias, const float* mask, float* weights);
+AIDN_API int aidn_mi355_attn_fwd_f16(void* ctx, void* stream, const aidn_attn_desc* desc,
+                            const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o,
+                            float* lse, const float* bias, const float* mask, float* weights);
+AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_desc* desc,
+                             const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o,
+                             float* lse, const float* bias, const float* mask, float* weights);
+
+/* ---- decode attention (Sq == 1) ---------------------------------------------------------------------
+ * One query row per (batch, head) against a KV cache of Sk rows: HBM-bound, the keys are split over
+ * workgroups (coalesced 128-bit loads), partial (max, sum, acc) triples are merged by a second
+ * kernel from a library-owned workspace.  Same descriptor (Sq must be 1; with causal != 0 keys
+ * j > causal_query_offset are masked, so offset Sk - 1, the bottom-right rule, attends to the whole
+ * cache; bias, mask and soft-cap are not available here); strides select the cache
+ * layout: [B,Hkv,Sk,D] (dense), the reference's decode layout [Sk,Hkv,D]
+ * (HipFlashDecodeKernels.cs:9-10; host FlashDecode HipBackend.cs:919-965) or its dense KVCache
+ * [B,Sk,Hkv,D] (Engines/Autodiff/KVCache.cs:5-8).  splits <= 0 picks the split count
+ * (the reference default is min(Sk, 8), HipBackend.cs:936); results do not depend on it beyond
+ * rounding.  o is fp32 or the input type per desc->out_is_16bit. */
+AIDN_API int aidn_mi355_attn_decode_f32(void* ctx, void* stream, const aidn_attn_desc* desc,
+                               const float* q, const float* k, const float* v, float* o, float* lse, int splits);
+AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn_desc* desc,
+                               const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
+AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc,
+                                const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
+
+/* ---- test / tuning hook --------------------------------------------------------------------------------
+ * Forces the GEMM tile edge (64, 128 or 256; 0 = automatic choice) for subsequent calls on this
+ * context, so the parity suite can exercise every kernel instance.  No counterpart in the reference. */
+AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AIDOTNET_MI355_H */

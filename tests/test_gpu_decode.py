@@ -1,0 +1,129 @@
+"""GPU parity of decode attention (one query row per head) through the C ABI against the CPU oracle.
+
+Reference precedent: FlashDecodeHipTests.cs:43-130 (tests/AiDotNet.Tensors.Tests/Engines/DirectGpu): in-test
+DecodeOracle, tolerance 2e-3 + 2e-3 * |e|, split-count independence, grouped-query heads.  The task's bar
+is tighter and is what is asserted: 1e-4 (fp32), 2e-2 (bf16 / fp16) in the mixed metric.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import TORCH16, dev, from_bits16, mixed_err, round_to
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def be():
+    from aidotnet.tensors_amd import Mi355Backend
+    b = Mi355Backend()
+    yield b
+    b.Dispose()
+
+
+def _run_flash_decode(be, heads, kv, d, seq, splits, seed):
+    rng = np.random.default_rng(seed)
+    k = rng.uniform(-1, 1, (seq, kv, d)).astype(np.float32)
+    v = rng.uniform(-1, 1, (seq, kv, d)).astype(np.float32)
+    q = rng.uniform(-1, 1, (heads, d)).astype(np.float32)
+    scale = 1.0 / math.sqrt(d)
+    out = be.FlashDecode(be.AllocateBuffer(q), be.AllocateBuffer(k), be.AllocateBuffer(v), heads, kv, d, seq, scale, splits)
+    got = be.DownloadBuffer(out).numpy().reshape(heads, d)
+    want = oracle.decode_f32(q, k, v, heads, kv, d, seq, scale)
+    return got, want
+
+
+@pytest.mark.parametrize("heads,d,seq,splits", [(4, 64, 40, 8), (8, 32, 100, 8), (4, 64, 7, 8), (4, 64, 64, 1), (6, 48, 77, 0),
+                                                (2, 128, 3000, 0), (2, 128, 3000, 5), (3, 20, 513, 2), (1, 256, 700, 3)])
+def test_mha_decode_matches_oracle(be, heads, d, seq, splits):
+    got, want = _run_flash_decode(be, heads, heads, d, seq, splits, 0xFDE + heads + seq + splits)
+    assert np.all(np.abs(got - want) <= 2e-3 + 2e-3 * np.abs(want))        # the reference's tolerance
+    assert mixed_err(got, want) <= 1e-4                                     # the task's
+
+
+@pytest.mark.parametrize("heads,kv,d,seq,splits", [(8, 2, 64, 50, 8), (8, 1, 32, 300, 4), (12, 4, 128, 1025, 0)])
+def test_gqa_decode_matches_oracle(be, heads, kv, d, seq, splits):
+    got, want = _run_flash_decode(be, heads, kv, d, seq, splits, 0xABC + heads + kv + seq)
+    assert mixed_err(got, want) <= 1e-4
+
+
+def test_split_count_independence(be):
+    # FlashDecodeHipTests.cs:107-117
+    base, _ = _run_flash_decode(be, 4, 4, 64, 2000, 1, 99)
+    for s in (2, 3, 7, 8):
+        other, _ = _run_flash_decode(be, 4, 4, 64, 2000, s, 99)
+        assert np.max(np.abs(other - base)) <= 2e-6
+
+
+def test_decode_guards(be):
+    from aidotnet.tensors_amd import ArgumentException, ArgumentOutOfRangeException
+    b = be.AllocateBuffer(1024)
+    for bad in ((0, 1, 8, 4), (4, 3, 8, 4), (4, 4, 512, 4), (4, 4, 8, 0)):   # GpuKernelGuards.cs:41-52
+        with pytest.raises(ArgumentOutOfRangeException):
+            be.FlashDecode(b, b, b, bad[0], bad[1], bad[2], bad[3], 1.0)
+    with pytest.raises(ArgumentException):
+        be.FlashDecode(b, b, b, 8, 8, 64, 100, 1.0)                          # undersized K/V
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+@pytest.mark.parametrize("B,H,Hkv,S,D", [(3, 4, 4, 333, 64), (2, 8, 2, 1000, 128), (1, 2, 2, 65, 32)])
+def test_batched_decode_all_types_and_layouts(be, kind, layout, B, H, Hkv, S, D):
+    rng = np.random.default_rng(B + H + S + D)
+    q = rng.standard_normal((B, H, 1, D)).astype(np.float32)
+    k = rng.standard_normal((B, Hkv, S, D)).astype(np.float32)
+    v = rng.standard_normal((B, Hkv, S, D)).astype(np.float32)
+    scale = 1.0 / math.sqrt(D)
+    if kind == "f32":
+        qw, kw, vw = q, k, v
+        tq, tk, tv = dev(q), dev(k), dev(v)
+        tol = 1e-4
+    else:
+        (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+        dt = TORCH16[kind]
+        tq, tk, tv = from_bits16(qb, dt), from_bits16(kb, dt), from_bits16(vb, dt)
+        tol = 2e-2
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale)
+    if layout == "bshd":
+        tk = tk.transpose(1, 2).contiguous(); tv = tv.transpose(1, 2).contiguous()
+    out = torch.full((B, H, 1, D), float("nan"), device="cuda")
+    lse = torch.empty(B, H, 1, device="cuda")
+    be.DecodeAttention(kind, be.WrapTensor(tq), be.WrapTensor(tk), be.WrapTensor(tv), be.WrapTensor(out), B, H, S, D, scale,
+                       Hkv, 0, False, be.WrapTensor(lse), layout)
+    assert mixed_err(out.cpu().numpy(), o64) <= tol
+    assert mixed_err(lse.cpu().numpy(), lse64) <= (1e-4 if kind == "f32" else 1e-3)
+    if kind != "f32":
+        out16 = torch.zeros((B, H, 1, D), dtype=TORCH16[kind], device="cuda")
+        be.DecodeAttention(kind, be.WrapTensor(tq), be.WrapTensor(tk), be.WrapTensor(tv), be.WrapTensor(out16), B, H, S, D, scale,
+                           Hkv, 3, True, None, layout)
+        assert mixed_err(out16.float().cpu().numpy(), o64) <= tol
+
+
+def test_config5_decode_bf16_b32_h32_s4096_d128(be):
+    # B=32, H=32, q_len=1, KV length 4096, d=128, contiguous [32,32,4096,128] bf16 cache.  Sampled (batch, head)
+    # slices against the fp64 oracle; every slice against the prefill kernel run at Sq = 1 on the same cache.
+    B, H, S, D = 32, 32, 4096, 128
+    g = torch.Generator(device="cuda"); g.manual_seed(4096)
+    q = torch.randn(B, H, 1, D, device="cuda", generator=g).to(torch.bfloat16)
+    k = torch.randn(B, H, S, D, device="cuda", generator=g).to(torch.bfloat16)
+    v = torch.randn(B, H, S, D, device="cuda", generator=g).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((B, H, 1, D), float("nan"), device="cuda")
+    lse = torch.empty(B, H, 1, device="cuda")
+    be.DecodeAttention("bf16", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), B, H, S, D, scale,
+                       0, 0, False, be.WrapTensor(lse))
+    ref = torch.full((B, H, 1, D), float("nan"), device="cuda")
+    ref_lse = torch.empty(B, H, 1, device="cuda")
+    be.FlashAttentionHalf("bf16", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(ref), be.WrapTensor(ref_lse),
+                          B, H, 1, S, D, scale, True, S - 1)
+    assert torch.isfinite(out).all()
+    assert mixed_err(out.cpu().numpy(), ref.cpu().numpy()) <= 2e-2
+    assert mixed_err(lse.cpu().numpy(), ref_lse.cpu().numpy()) <= 1e-3
+    for (b, h) in [(0, 0), (13, 7), (31, 31)]:
+        qs, ks, vs = (t[b:b + 1, h:h + 1].float().cpu().numpy() for t in (q, k, v))
+        o64, lse64 = oracle.attention_f64(qs, ks, vs, scale)
+        assert mixed_err(out[b, h].cpu().numpy(), o64[0, 0]) <= 2e-2
+        assert mixed_err(lse[b, h].cpu().numpy(), lse64[0, 0]) <= 1e-3

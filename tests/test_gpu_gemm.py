@@ -1,0 +1,310 @@
+"""GPU parity of the GEMM entry points (through the C ABI) against the CPU oracle.
+
+Bars: bit-exact on dyadic inputs (every summation order is exact there, so GPU, oracle and integer
+arithmetic must agree bit for bit); |a - e| <= 1e-4 * (1 + |e|) for fp32 and 2e-2 for fp16 / bf16
+against the fp64 truth of the same (already rounded) inputs -- the tolerances the task states.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from _util import TORCH16, bits16, dev, dyadic, from_bits16, mixed_err, rel_frobenius, round_to
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-4
+HALF_TOL = 2e-2
+
+# (M, N, K): the reference's edge shapes (TensorMatMulSimdFallbackTests.cs:69-73, HipHalfPrecisionGemmTests.cs:119-122,
+# Fp16Bf16GemmTests.cs:23-62, SgemmCachedBTests.cs:10-41) plus tile-boundary cases for the 64/128/256 tiles.
+SHAPES = [(1, 1, 1), (7, 13, 11), (96, 130, 80), (37, 53, 71), (13, 10, 17), (4, 32, 8), (16, 24, 20), (3, 5, 7),
+          (1, 64, 1), (64, 64, 32), (65, 63, 33), (128, 128, 64), (129, 127, 65), (256, 256, 64), (200, 300, 100),
+          (32, 4096, 128), (8, 512, 1030), (512, 512, 512)]
+
+
+@pytest.fixture(scope="module")
+def be():
+    from aidotnet.tensors_amd import Mi355Backend
+    b = Mi355Backend()
+    yield b
+    b.SetGemmTile(0)
+    b.Dispose()
+
+
+def _gemm(be, a, b, M, N, K, alpha=1.0, beta=0.0, c0=None, transB=False):
+    A, B = be.WrapTensor(dev(a)), be.WrapTensor(dev(b))
+    c = dev(c0) if c0 is not None else torch.full((M, N), float("nan"), device="cuda")
+    C = be.WrapTensor(c)
+    (be.MatMulTransposed if transB else be.Gemm)(A, B, C, M, N, K, alpha, beta)
+    return c.cpu().numpy()
+
+
+@pytest.mark.parametrize("tile", [0, 64, 128])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_sgemm_bit_exact_on_dyadic_inputs(be, tile, M, N, K):
+    be.SetGemmTile(tile)
+    rng = np.random.default_rng(M * 7919 + N * 31 + K)
+    a = dyadic(rng, (M, K)); b = dyadic(rng, (K, N))
+    want = oracle.sgemm(a, b, M, K, N, threads=4)
+    got = _gemm(be, a, b, M, N, K)
+    assert np.array_equal(got, want)
+    gotT = _gemm(be, a, np.ascontiguousarray(b.T), M, N, K, transB=True)
+    assert np.array_equal(gotT, want)
+    be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_sgemm_random_within_tolerance_of_fp64_truth(be, M, N, K):
+    rng = np.random.default_rng(M + 3 * N + 5 * K)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32)
+    b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    truth = oracle.gemm_f64(a, b, M, K, N)
+    cpu = oracle.sgemm(a, b, M, K, N, threads=4)
+    got = _gemm(be, a, b, M, N, K)
+    assert mixed_err(got, truth) <= FP32_TOL
+    # GpuCpuConsistencyTests.cs:1213-1287: GPU error vs fp64 <= 4 x CPU fp32 error + 1e-6
+    assert np.max(np.abs(got - truth)) <= 4 * np.max(np.abs(cpu - truth)) + 1e-6
+    assert mixed_err(got, cpu) <= FP32_TOL
+
+
+def test_sgemm_alpha_beta_and_poisoned_output(be):
+    rng = np.random.default_rng(17)
+    M, N, K = 45, 70, 33
+    a = dyadic(rng, (M, K)); b = dyadic(rng, (K, N)); c0 = dyadic(rng, (M, N))
+    want = oracle.gemm_alpha_beta(a, b, c0, M, N, K, alpha=0.5, beta=2.0)
+    assert np.array_equal(_gemm(be, a, b, M, N, K, 0.5, 2.0, c0), want)
+    wantT = oracle.gemm_alpha_beta(a, np.ascontiguousarray(b.T), c0, M, N, K, alpha=-1.5, beta=0.25, trans_b=True)
+    assert np.array_equal(_gemm(be, a, np.ascontiguousarray(b.T), M, N, K, -1.5, 0.25, c0, transB=True), wantT)
+    # beta == 0 must overwrite NaN-poisoned storage and never touch memory past M*N (GemmBeta0BitExactTests.cs:24-34, 88-140)
+    big = torch.full((M * N + 4096,), float("nan"), device="cuda")
+    be.Gemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(big), M, N, K, 1.0, 0.0)
+    host = big.cpu().numpy()
+    assert np.array_equal(host[:M * N].reshape(M, N), oracle.sgemm(a, b, M, K, N))
+    assert np.isnan(host[M * N:]).all()
+
+
+def test_sgemm_identity_known_answer(be):
+    # BatchMatMulAndAttentionTests.cs:17-56
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((19, 23)).astype(np.float32)
+    assert np.array_equal(_gemm(be, a, np.eye(23, dtype=np.float32), 19, 23, 23), a)
+    a2 = np.array([[1, 2, 3], [4, 5, 6]], np.float32); b2 = np.array([[7, 8], [9, 10], [11, 12]], np.float32)
+    assert np.array_equal(_gemm(be, a2, b2, 2, 2, 3), np.array([[58, 64], [139, 154]], np.float32))
+
+
+@pytest.mark.parametrize("batch,M,N,K", [(1, 5, 7, 3), (6, 33, 65, 40), (96, 64, 64, 64), (3, 130, 100, 70)])
+def test_batched_gemm_matches_per_matrix_oracle(be, batch, M, N, K):
+    rng = np.random.default_rng(batch + M + N + K)
+    a = dyadic(rng, (batch, M, K)); b = dyadic(rng, (batch, K, N)); c0 = dyadic(rng, (batch, M, N))
+    c = dev(c0)
+    be.BatchedGemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), M, N, K, batch, 1.0, 0.5)
+    got = c.cpu().numpy()
+    for i in range(batch):
+        assert np.array_equal(got[i], oracle.gemm_alpha_beta(a[i], b[i], c0[i], M, N, K, 1.0, 0.5))
+
+
+def test_engine_matmul_shape_rules(be):
+    from aidotnet.tensors_amd import ArgumentException, Mi355Engine
+    eng = Mi355Engine(be)
+    rng = np.random.default_rng(5)
+    a = dyadic(rng, (2, 3, 9, 11)); b = dyadic(rng, (11, 6))
+    got = eng.TensorMatMul(dev(a), dev(b)).cpu().numpy()        # ND x 2D = collapse (BatchMatMulAndAttentionTests.cs:127-151)
+    assert np.array_equal(got.reshape(-1, 6), oracle.sgemm(a.reshape(-1, 11), b, 54, 11, 6))
+    bb = dyadic(rng, (2, 3, 11, 4))
+    got2 = eng.TensorMatMul(dev(a), dev(bb)).cpu().numpy()      # ND x ND batched
+    for i in range(2):
+        for j in range(3):
+            assert np.array_equal(got2[i, j], oracle.sgemm(a[i, j], bb[i, j], 9, 11, 4))
+    with pytest.raises(ArgumentException):
+        eng.TensorMatMul(dev(a), dev(dyadic(rng, (12, 6))))
+
+
+def test_argument_errors_match_reference_behaviour(be):
+    from aidotnet.tensors_amd import ArgumentException, ArgumentNullException, ArgumentOutOfRangeException
+    buf = be.AllocateBuffer(64)
+    h = be.AllocateByteBuffer(128)
+    for bad in ((0, 4, 4), (4, 0, 4), (4, 4, -1)):            # HipHalfPrecisionGemmTests.cs:147-159
+        with pytest.raises(ArgumentOutOfRangeException):
+            be.Hgemm(h, h, h, *bad)
+        with pytest.raises(ArgumentOutOfRangeException):
+            be.Gemm(buf, buf, buf, *bad)
+    with pytest.raises(ArgumentNullException):
+        be.GemmFp16In32fOut(None, h, buf, 2, 2, 2)
+    with pytest.raises(ArgumentException):
+        be.Gemm(buf, buf, buf, 64, 64, 64)                      # undersized buffers (GpuKernelGuards.cs:61-68)
+    with pytest.raises(ArgumentException):
+        be.BatchedGemm(buf, buf, buf, 2, 2, 2, 0)               # HipBackend.cs:1601-1602
+    # the native layer rejects the same conditions by status code
+    import ctypes
+    st = be._lib.aidn_mi355_sgemm(be._ctx, None, buf.Handle, buf.Handle, buf.Handle, 0, 4, 4, 1.0, 0.0, 0)
+    assert st == 1001 and b"positive" in be._lib.aidn_mi355_last_error(be._ctx)
+    assert be._lib.aidn_mi355_sgemm(be._ctx, None, None, buf.Handle, buf.Handle, 4, 4, 4, 1.0, 0.0, 0) == 1001
+
+
+# ------------------------------------------------------------------------------------------- 16-bit
+HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7, 13, 11), (96, 130, 80), (37, 53, 71),
+               (128, 128, 64), (256, 256, 128), (512, 256, 192), (130, 260, 70), (32, 512, 4096)]
+
+
+def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
+    A = be.WrapTensor(from_bits16(abits, TORCH16[kind])); B = be.WrapTensor(from_bits16(bbits, TORCH16[kind]))
+    if out32:
+        c = torch.full((M, N), float("nan"), device="cuda")
+        (be.GemmFp16In32fOut if kind == "f16" else be.GemmBf16In32fOut)(A, B, be.WrapTensor(c), M, N, K)
+        return c.cpu().numpy()
+    c = torch.zeros((M, N), dtype=TORCH16[kind], device="cuda")
+    (be.Hgemm if kind == "f16" else be.Bf16Gemm)(A, B, be.WrapTensor(c), M, N, K)
+    return bits16(c)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("tile", [0, 64, 128])
+@pytest.mark.parametrize("M,N,K", HALF_SHAPES)
+def test_half_gemm_bit_exact_on_dyadic_inputs(be, kind, tile, M, N, K):
+    be.SetGemmTile(tile)
+    rng = np.random.default_rng(M * 131 + N * 17 + K)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+    ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+    fn = oracle.hgemm if kind == "f16" else oracle.bf16gemm
+    want16, want32 = fn(ab, bb, M, K, N)
+    assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, True), want32)
+    assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, False), want16)
+    be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", HALF_SHAPES)
+def test_half_gemm_random_within_tolerance(be, kind, M, N, K):
+    rng = np.random.default_rng(M + N + K + (1 if kind == "f16" else 2))
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+    truth = oracle.gemm_f64(aw, bw, M, K, N)                     # fp64 over the SAME rounded inputs
+    fn = oracle.hgemm if kind == "f16" else oracle.bf16gemm
+    want16, want32 = fn(ab, bb, M, K, N)
+    got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
+    assert mixed_err(got32, truth) <= 1e-4                       # fp32 accumulation: far inside the 2e-2 gate
+    assert np.all(np.abs(got32 - want32) <= 1e-2 + 1e-2 * np.abs(want32))    # HipHalfPrecisionGemmTests.cs:137
+    got16 = _half_gemm(be, kind, ab, bb, M, N, K, False)
+    back = oracle.f16_to_f32(got16) if kind == "f16" else oracle.bf16_to_f32(got16)
+    assert mixed_err(back, truth) <= HALF_TOL
+    rel = 6e-3 if kind == "f16" else 2e-2                        # Fp16Bf16GemmTests.cs:108-121
+    assert np.all(np.abs(back - truth) <= rel * np.maximum(1.0, np.abs(truth)))
+    # the 16-bit output is exactly the RNE narrowing of the kernel's own fp32 result
+    narrow = oracle.f32_to_f16(got32) if kind == "f16" else oracle.f32_to_bf16(got32)
+    assert np.array_equal(got16, narrow)
+    if K >= 64:
+        # a reduced-precision result must differ from the fp32 product of the unrounded inputs
+        # (GotoGemmBf16FusionTests.cs:81-82): guards against silently running the wrong kernel
+        assert np.max(np.abs(got32 - oracle.gemm_f64(a, b, M, K, N))) > 1e-6
+
+
+def test_bf16_literal_known_answer(be):
+    # BFloat16KernelsTests.cs:55-68
+    ab, _ = round_to(np.array([[1, 2, 3], [4, 5, 6]], np.float32), "bf16")
+    bb, _ = round_to(np.array([[7, 8], [9, 10], [11, 12]], np.float32), "bf16")
+    got = _half_gemm(be, "bf16", ab, bb, 2, 2, 3, False)
+    assert np.array_equal(oracle.bf16_to_f32(got), np.array([[58, 64], [139, 154]], np.float32))
+
+
+# ------------------------------------------------------------------------------------ full-size configs
+def test_config1_fp32_1024_cubed_against_oracle(be):
+    # fp32 GEMM M=N=K=1024, A,B ~ U[-1,1]
+    rng = np.random.default_rng(1024)
+    a = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32); b = rng.uniform(-1, 1, (1024, 1024)).astype(np.float32)
+    truth = oracle.gemm_f64(a, b, 1024, 1024, 1024)
+    cpu = oracle.sgemm(a, b, 1024, 1024, 1024, threads=oracle.max_threads())
+    got = _gemm(be, a, b, 1024, 1024, 1024)
+    assert mixed_err(got, truth) <= FP32_TOL and mixed_err(got, cpu) <= FP32_TOL
+    assert rel_frobenius(got, truth) < 1e-6
+    assert np.max(np.abs(got - truth)) <= 4 * np.max(np.abs(cpu - truth)) + 1e-6
+
+
+@pytest.mark.parametrize("kind", ["f32", "f16", "bf16"])
+def test_config2_projection_gemm_sampled_rows(be, kind):
+    # M=4096 (8 x 512), K=768, N=3072; activations N(0,1), weights N(0, 0.02^2)
+    M, K, N = 4096, 768, 3072
+    rng = np.random.default_rng(4096)
+    a = rng.standard_normal((M, K)).astype(np.float32); b = (0.02 * rng.standard_normal((K, N))).astype(np.float32)
+    rows = np.sort(rng.choice(M, 96, replace=False))
+    if kind == "f32":
+        got = _gemm(be, a, b, M, N, K)
+        truth = a[rows].astype(np.float64) @ b.astype(np.float64)
+        assert mixed_err(got[rows], truth) <= FP32_TOL
+        cpu = oracle.sgemm(a, b, M, K, N, threads=oracle.max_threads())
+        assert mixed_err(got, cpu) <= FP32_TOL
+    else:
+        ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+        got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
+        truth = aw[rows].astype(np.float64) @ bw.astype(np.float64)
+        assert mixed_err(got32[rows], truth) <= 1e-4
+        got16 = _half_gemm(be, kind, ab, bb, M, N, K, False)
+        back = oracle.f16_to_f32(got16[rows]) if kind == "f16" else oracle.bf16_to_f32(got16[rows])
+        assert mixed_err(back, truth) <= HALF_TOL
+        narrow = oracle.f32_to_f16(got32) if kind == "f16" else oracle.f32_to_bf16(got32)
+        assert np.array_equal(got16, narrow)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_config2_square_8192_checksums_and_samples(be, kind):
+    # 8192^3: too large for the CPU oracle, so use size-independent properties.  Inputs are dyadic
+    # (integers in [-4, 4] / 8), so every fp32 partial sum is exact and the result must equal integer
+    # arithmetic: (1) row / column checksums C.1 = A.(B.1), 1^T.C = (1^T.A).B in float64 on the device,
+    # (2) sampled rows against numpy int64 matmul, (3) 16-bit output == RNE(fp32 output).
+    n = 8192
+    g = torch.Generator(device="cuda"); g.manual_seed(8192)
+    ai = torch.randint(-4, 5, (n, n), device="cuda", generator=g, dtype=torch.int32)
+    bi = torch.randint(-4, 5, (n, n), device="cuda", generator=g, dtype=torch.int32)
+    a = (ai.float() / 8).to(TORCH16[kind]); b = (bi.float() / 8).to(TORCH16[kind])
+    c = torch.full((n, n), float("nan"), device="cuda")
+    (be.GemmFp16In32fOut if kind == "f16" else be.GemmBf16In32fOut)(be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(c), n, n, n)
+    cd = c.double()
+    rows_want = (ai.double() @ bi.double().sum(1, keepdim=True)).squeeze(1) / 64
+    cols_want = (ai.double().sum(0, keepdim=True) @ bi.double()).squeeze(0) / 64
+    assert torch.equal(cd.sum(1), rows_want) and torch.equal(cd.sum(0), cols_want)
+    rng = np.random.default_rng(7)
+    rows = np.sort(rng.choice(n, 16, replace=False))
+    want = (ai[rows].cpu().numpy().astype(np.int64) @ bi.cpu().numpy().astype(np.int64)).astype(np.float64) / 64
+    assert np.array_equal(c[rows].cpu().numpy().astype(np.float64), want)
+    c16 = torch.zeros((n, n), dtype=TORCH16[kind], device="cuda")
+    (be.Hgemm if kind == "f16" else be.Bf16Gemm)(be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(c16), n, n, n)
+    assert torch.equal(c16, c.to(TORCH16[kind]))
+
+
+def test_config5_decode_projection_gemm_bf16(be):
+    # M=32, K=4096, N=4096 bf16
+    M, K, N = 32, 4096, 4096
+    rng = np.random.default_rng(32)
+    a = rng.standard_normal((M, K)).astype(np.float32); b = (0.02 * rng.standard_normal((K, N))).astype(np.float32)
+    ab, aw = round_to(a, "bf16"); bb, bw = round_to(b, "bf16")
+    truth = oracle.gemm_f64(aw, bw, M, K, N)
+    got32 = _half_gemm(be, "bf16", ab, bb, M, N, K, True)
+    assert mixed_err(got32, truth) <= 1e-4
+    got16 = _half_gemm(be, "bf16", ab, bb, M, N, K, False)
+    assert mixed_err(oracle.bf16_to_f32(got16), truth) <= HALF_TOL
+    assert np.array_equal(got16, oracle.f32_to_bf16(got32))
+
+
+# --------------------------------------------------------------------------------------- conversions
+@pytest.mark.parametrize("n", [1, 7, 8, 1000, 4099, 1 << 20])
+def test_conversions_bit_exact(be, n):
+    rng = np.random.default_rng(n)
+    bits = rng.integers(0, 2 ** 32, size=n, dtype=np.uint64).astype(np.uint32)
+    x = bits.view(np.float32).copy()
+    x[: min(n, 6)] = np.array([0.0, -0.0, np.inf, -np.inf, 65520.0, 2.0 ** -25], np.float32)[: min(n, 6)]
+    xin = dev(x)
+    h = torch.zeros(n, dtype=torch.float16, device="cuda"); bf = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+    be.ConvertToFp16(be.WrapTensor(xin), be.WrapTensor(h), n)
+    be.ConvertToBf16(be.WrapTensor(xin), be.WrapTensor(bf), n)
+    nan = np.isnan(x)
+    got_h, got_b = bits16(h), bits16(bf)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got_h[~nan], oracle.f32_to_f16(x)[~nan])
+    assert np.array_equal(got_b, oracle.f32_to_bf16(x))          # bf16 rule is integer arithmetic: NaNs included
+    assert np.isnan(oracle.f16_to_f32(got_h[nan])).all()
+    back_h = torch.zeros(n, device="cuda"); back_b = torch.zeros(n, device="cuda")
+    be.ConvertToFp32(be.WrapTensor(h), be.WrapTensor(back_h), n)
+    be.ConvertBf16ToFp32(be.WrapTensor(bf), be.WrapTensor(back_b), n)
+    assert np.array_equal(back_b.cpu().numpy().view(np.uint32), oracle.bf16_to_f32(got_b).view(np.uint32))
+    ok = ~np.isnan(oracle.f16_to_f32(got_h))
+    assert np.array_equal(back_h.cpu().numpy()[ok], oracle.f16_to_f32(got_h)[ok])
