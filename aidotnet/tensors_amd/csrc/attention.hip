@@ -297,7 +297,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                             pf[w] = Elem<T>::narrow(st[kt][8 * ps + 2 * w]) | (Elem<T>::narrow(st[kt][8 * ps + 2 * w + 1]) << 16);
                     } else {
 #pragma unroll
-                        for (int w = 0; w < 4; w++) pf[w] = __builtin_bit_cast(uint32_t, st[kt][4 * ps + w]);
+                        for (int w = 0; w < 4; w++) pf[w] = as_u32(st[kt][4 * ps + w]);
                     }
 #pragma unroll
                     for (int i = 0; i < DT; i++) {
@@ -328,10 +328,10 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     if (a.vec_out && d0 + 4 <= a.D) {
                         *(f32x4*)(O + d0) = f32x4{v0, v1, v2, v3};
                     } else {
-                        if (d0 + 0 < a.D) O[d0 + 0] = __builtin_bit_cast(uint32_t, v0);
-                        if (d0 + 1 < a.D) O[d0 + 1] = __builtin_bit_cast(uint32_t, v1);
-                        if (d0 + 2 < a.D) O[d0 + 2] = __builtin_bit_cast(uint32_t, v2);
-                        if (d0 + 3 < a.D) O[d0 + 3] = __builtin_bit_cast(uint32_t, v3);
+                        if (d0 + 0 < a.D) O[d0 + 0] = as_u32(v0);
+                        if (d0 + 1 < a.D) O[d0 + 1] = as_u32(v1);
+                        if (d0 + 2 < a.D) O[d0 + 2] = as_u32(v2);
+                        if (d0 + 3 < a.D) O[d0 + 3] = as_u32(v3);
                     }
                 } else {
                     uint32_t w0 = Elem<OutT>::narrow(v0) | (Elem<OutT>::narrow(v1) << 16);
@@ -373,7 +373,7 @@ __global__ __launch_bounds__(256) void attn_weights_kernel(const AttnArgs a, flo
         float s = 0.0f;
         for (int d = 0; d < a.D; d++) {
             float qv, kv;
-            if constexpr (Elem<T>::BYTES == 4) { qv = __builtin_bit_cast(float, q[d]); kv = __builtin_bit_cast(float, k[d]); }
+            if constexpr (Elem<T>::BYTES == 4) { qv = as_f32(q[d]); kv = as_f32(k[d]); }
             else { qv = Elem<T>::widen(q[d]); kv = Elem<T>::widen(k[d]); }
             s += qv * kv;
         }

@@ -20,8 +20,13 @@ struct bf16_t { uint16_t bits; };
 
 constexpr int WAVE = 64;
 
+// Bit reinterpretation through by-value scalars.  (Applying __builtin_bit_cast directly to an element
+// of an ext_vector lvalue, e.g. v[i], reads element 0 for every i with this compiler.)
+__device__ __forceinline__ float as_f32(uint32_t v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ uint32_t as_u32(float v) { return __builtin_bit_cast(uint32_t, v); }
+
 // ------------------------------------------------------------------ conversions
-__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __builtin_bit_cast(float, b << 16); }
+__device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return as_f32(b << 16); }
 
 // float -> bf16 bits, round-to-nearest-even; NaN keeps sign/payload top bits with the
 // quiet bit forced (the rule of the reference's BFloat16.FromFloat,
@@ -29,7 +34,7 @@ __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __built
 // result is bit-identical to the host rule for every input.
 __device__ __forceinline__ uint32_t float_to_bf16_bits(float f)
 {
-    uint32_t u = __builtin_bit_cast(uint32_t, f);
+    uint32_t u = as_u32(f);
     if ((u & 0x7F800000u) == 0x7F800000u && (u & 0x007FFFFFu) != 0u) return (u >> 16) | 0x0040u;
     return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
@@ -96,7 +101,7 @@ template <> struct Mma32<float> {
     {
 #pragma unroll
         for (int s = 0; s < 4; s++)
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[s]), __builtin_bit_cast(float, b[s]), acc, 0, 0, 0);
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(as_f32(a[s]), as_f32(b[s]), acc, 0, 0, 0);
     }
 };
 

@@ -19,8 +19,8 @@ __global__ __launch_bounds__(256) void narrow_kernel(const float* __restrict__ i
         u32x4 o;
 #pragma unroll
         for (int w = 0; w < 2; w++) {
-            o[w] = Elem<T>::narrow(__builtin_bit_cast(float, a[2 * w])) | (Elem<T>::narrow(__builtin_bit_cast(float, a[2 * w + 1])) << 16);
-            o[w + 2] = Elem<T>::narrow(__builtin_bit_cast(float, b[2 * w])) | (Elem<T>::narrow(__builtin_bit_cast(float, b[2 * w + 1])) << 16);
+            o[w] = Elem<T>::narrow(as_f32(a[2 * w])) | (Elem<T>::narrow(as_f32(a[2 * w + 1])) << 16);
+            o[w + 2] = Elem<T>::narrow(as_f32(b[2 * w])) | (Elem<T>::narrow(as_f32(b[2 * w + 1])) << 16);
         }
         ((u32x4*)out)[i] = o;
     }
@@ -38,10 +38,10 @@ __global__ __launch_bounds__(256) void widen_kernel(const uint16_t* __restrict__
         u32x4 a, b;
 #pragma unroll
         for (int w = 0; w < 2; w++) {
-            a[2 * w] = __builtin_bit_cast(uint32_t, Elem<T>::widen(v[w] & 0xFFFFu));
-            a[2 * w + 1] = __builtin_bit_cast(uint32_t, Elem<T>::widen(v[w] >> 16));
-            b[2 * w] = __builtin_bit_cast(uint32_t, Elem<T>::widen(v[w + 2] & 0xFFFFu));
-            b[2 * w + 1] = __builtin_bit_cast(uint32_t, Elem<T>::widen(v[w + 2] >> 16));
+            a[2 * w] = as_u32(Elem<T>::widen(v[w] & 0xFFFFu));
+            a[2 * w + 1] = as_u32(Elem<T>::widen(v[w] >> 16));
+            b[2 * w] = as_u32(Elem<T>::widen(v[w + 2] & 0xFFFFu));
+            b[2 * w + 1] = as_u32(Elem<T>::widen(v[w + 2] >> 16));
         }
         ((u32x4*)out)[2 * i] = a;
         ((u32x4*)out)[2 * i + 1] = b;

@@ -54,7 +54,7 @@ __device__ __forceinline__ void widen16(const u32x4& x, float (&f)[Elem<T>::PER1
 {
     if constexpr (Elem<T>::BYTES == 4) {
 #pragma unroll
-        for (int e = 0; e < 4; e++) f[e] = __builtin_bit_cast(float, x[e]);
+        for (int e = 0; e < 4; e++) f[e] = as_f32(x[e]);
     } else {
 #pragma unroll
         for (int w = 0; w < 4; w++) {
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
             typedef typename Raw3<OutT>::type out_t;
             out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
             float r = L > 0.0f ? A / L : 0.0f;
-            if constexpr (Elem<OutT>::BYTES == 4) O[d] = __builtin_bit_cast(uint32_t, r);
+            if constexpr (Elem<OutT>::BYTES == 4) O[d] = as_u32(r);
             else O[d] = (out_t)Elem<OutT>::narrow(r);
             if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
         }
@@ -206,7 +206,7 @@ __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a, 
         typedef typename Raw3<OutT>::type out_t;
         out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
         float r = L > 0.0f ? A / L : 0.0f;
-        if constexpr (Elem<OutT>::BYTES == 4) O[d] = __builtin_bit_cast(uint32_t, r);
+        if constexpr (Elem<OutT>::BYTES == 4) O[d] = as_u32(r);
         else O[d] = (out_t)Elem<OutT>::narrow(r);
         if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
     }

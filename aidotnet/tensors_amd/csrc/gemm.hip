@@ -252,8 +252,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
                     out_t* p = C + (long long)row * g.ldc + col;
                     float v = g.alpha * acc[i][j][r];
                     if constexpr (Elem<OutT>::BYTES == 4) {
-                        if (use_beta) v += g.beta * __builtin_bit_cast(float, *p);
-                        *p = __builtin_bit_cast(uint32_t, v);
+                        if (use_beta) v += g.beta * as_f32(*p);
+                        *p = as_u32(v);
                     } else {
                         if (use_beta) v += g.beta * Elem<OutT>::widen(*p);
                         *p = (out_t)Elem<OutT>::narrow(v);

@@ -84,8 +84,10 @@ class Mi355Engine:
         Sk = key.shape[2]
         if key.shape != value.shape or key.shape[0] != B or key.shape[3] != D:
             raise ArgumentException("key/value shapes do not match the query")
-        if isCausal and queryOffset + Sq > Sk:
-            raise ArgumentException("queryOffset + Sq exceeds Sk")       # FusedAttentionAuditTests.cs:81-92
+        if isCausal and queryOffset != 0 and queryOffset + Sq > Sk:
+            # the offset form is rejected when it runs past the keys (FusedAttentionAuditTests.cs:81-92);
+            # plain top-left causal with Sq > Sk is legal for IEngine.FlashAttention (CpuEngine.cs:29235)
+            raise ArgumentException("queryOffset + Sq exceeds Sk")
         if scale is None:
             scale = 1.0 / math.sqrt(D)
         be = self.backend
