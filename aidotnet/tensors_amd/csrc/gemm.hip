@@ -220,17 +220,25 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
         if (kt + 1 < KT) load_tile((kt + 1) * BK);
         const unsigned char* as = As + stage * BM * ROWB + (wm * WTM + l32) * ROWB + h * 16;
         const unsigned char* bs = Bs + stage * BN * ROWB + (wn * WTN + l32) * ROWB + h * 16;
+        // fragments are double-buffered in registers: the LDS reads of step s+1 are in flight during the
+        // MFMAs of step s
+        u32x4 fa[2][TM], fb[2][TN];
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[0][i] = *(const u32x4*)(as + i * 32 * ROWB);
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[0][j] = *(const u32x4*)(bs + j * 32 * ROWB);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            u32x4 fa[TM], fb[TN];
+            if (s < 3) {
 #pragma unroll
-            for (int i = 0; i < TM; i++) fa[i] = *(const u32x4*)(as + i * 32 * ROWB + s * 32);
+                for (int i = 0; i < TM; i++) fa[(s + 1) & 1][i] = *(const u32x4*)(as + i * 32 * ROWB + (s + 1) * 32);
 #pragma unroll
-            for (int j = 0; j < TN; j++) fb[j] = *(const u32x4*)(bs + j * 32 * ROWB + s * 32);
+                for (int j = 0; j < TN; j++) fb[(s + 1) & 1][j] = *(const u32x4*)(bs + j * 32 * ROWB + (s + 1) * 32);
+            }
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
-                for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[i], fb[j]);
+                for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
         }
         if (kt + 1 < KT) store_tile(stage ^ 1);
         __syncthreads();
@@ -262,6 +270,177 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
             }
         }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Large-tile fast path for 16-bit inputs, B stored [K,N]: 256 x 256 x 64 tile, 8 waves (2 x 4, wave tile
+// 128 x 64).  Requires M % 256 == 0, N % 256 == 0, K % 64 == 0 and 16-byte aligned rows.
+//   * global -> LDS by the gfx950 direct load (global_load_lds_dwordx4): no staging registers, no
+//     ds_write, no register transposes.  One wave-load moves 64 lanes x 16 B into 1 KiB of contiguous LDS,
+//     so bank-conflict avoidance is done by choosing WHICH global chunk a lane fetches (XOR swizzle):
+//       A tile [256 rows][128 B]: 16-byte chunk c of row r lives at chunk position c ^ ((r >> 1) & 7)
+//       B tile [64 k][512 B]    : 16-byte chunk c of row k lives at chunk position c ^ ((k & 3) << 2)
+//   * B fragments come out of the [k][n] tile with the transposing LDS read ds_read_b64_tr_b16: within
+//     a 16-lane group, lane i receives element (i % 4) of the 8 bytes addressed by lane 4 m + i / 4,
+//     for m = 0..3; lanes address B[k0 + j/4][n0 + 4 (j%4)] and receive B[k0 .. k0+3][n0 + i].
+//   * the DMA is issued through inline asm: with the builtin the compiler orders every later LDS read
+//     that may alias the destination behind s_waitcnt vmcnt(0), which serialises load latency and MFMA.
+//     Completion is waited for explicitly (vmcnt(0) + workgroup barrier) before a stage is read.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void dma16_to_lds(const void* gptr, void* lds_dst_wave_uniform)
+{
+    uint32_t l = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds_dst_wave_uniform);
+    l = __builtin_amdgcn_readfirstlane(l);
+    // M0 carries the LDS base of the wave's 1 KiB destination; nothing else in these kernels uses M0
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(l), "v"(gptr));
+}
+
+template <typename T, typename OutT>
+__global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
+{
+    typedef uint16_t raw_t;
+    constexpr int WM = 2, WN = 4;
+    constexpr int BM = 256, BN = 256, BK = 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int ABYTES = BM * 128, BBYTES = BK * 512, STAGE = ABYTES + BBYTES;
+    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (32 + 32 per workgroup)
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const raw_t* __restrict__ A = (const raw_t*)g.A;
+    const raw_t* __restrict__ B = (const raw_t*)g.B;
+
+    // per-lane global sources of this wave's loads at k0 = 0
+    const raw_t* pa[LA];
+    const raw_t* pb[LB];
+#pragma unroll
+    for (int i = 0; i < LA; i++) {
+        int w = wave * LA + i;                                // A wave-load w: rows 8w .. 8w+7
+        int row = 8 * w + (lane >> 3), pos = lane & 7;
+        pa[i] = A + (long long)(m0 + row) * g.lda + (pos ^ ((row >> 1) & 7)) * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+        int w = wave * LB + i;                                // B wave-load w: k-rows 2w, 2w+1
+        int row = 2 * w + (lane >> 5), pos = lane & 31;
+        pb[i] = B + (long long)row * g.ldb + n0 + (pos ^ ((row & 3) << 2)) * 8;
+    }
+    auto issue_loads = [&](int kt, int stage) {
+        unsigned char* as = smem + stage * STAGE;
+        unsigned char* bs = as + ABYTES;
+#pragma unroll
+        for (int i = 0; i < LA; i++) dma16_to_lds(pa[i] + kt * BK, as + (wave * LA + i) * 1024);
+#pragma unroll
+        for (int i = 0; i < LB; i++) dma16_to_lds(pb[i] + (long long)kt * BK * g.ldb, bs + (wave * LB + i) * 1024);
+    };
+
+    // per-lane LDS read offsets
+    int a_off[TM], a_sw[TM];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+        int row = wm * WTM + i * 32 + l32;
+        a_off[i] = row * 128;
+        a_sw[i] = (row >> 1) & 7;
+    }
+    const int jl = lane & 15;
+    const int b_rowl = 8 * h + (jl >> 2);                     // + 16 s + 4 q
+    const int b_half = (jl & 1) * 8;
+    int b_chunk[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) b_chunk[j] = (wn * WTN + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;
+
+    auto read_frags = [&](const unsigned char* as, const unsigned char* bs, int s, u32x4 (&fa)[TM], u32x4 (&fb)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[i] = *(const u32x4*)(as + a_off[i] + (((2 * s + h) ^ a_sw[i]) << 4));
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                int row = 16 * s + 4 * q + b_rowl;
+                int pos = b_chunk[j] ^ ((row & 3) << 2);
+                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4*)(bs + row * 512 + pos * 16 + b_half));
+                u32x2 w = __builtin_bit_cast(u32x2, v);
+                fb[j][2 * q] = w[0];
+                fb[j][2 * q + 1] = w[1];
+            }
+        }
+    };
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    const int KT = g.K / BK;
+    issue_loads(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int stage = kt & 1;
+        const unsigned char* as = smem + stage * STAGE;
+        const unsigned char* bs = as + ABYTES;
+        // the other stage was last read before the barrier that ended the previous iteration
+        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+        u32x4 fa[2][TM], fb[2][TN];
+        read_frags(as, bs, 0, fa[0], fb[0]);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if (s < 3) read_frags(as, bs, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
+        }
+        __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed ...
+        __syncthreads();                    // ... and so has everyone else's
+    }
+
+    typedef typename Raw<OutT>::type out_t;
+    out_t* __restrict__ C = (out_t*)g.C;
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            const int col = n0 + wn * WTN + j * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                out_t* p = C + (long long)row * g.ldc + col;
+                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(acc[i][j][r]);
+                else *p = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
+            }
+        }
+}
+
+template <typename T, typename OutT>
+static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
+{
+    auto kern = gemm_dl_kernel<T, OutT>;
+    constexpr int smem = 2 * (256 * 128 + 64 * 512);
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    g.tiles_m = g.M / 256;
+    g.tiles_n = g.N / 256;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), smem, stream, g);
+    return hipGetLastError();
 }
 
 // ------------------------------------------------------------------ host side
@@ -297,14 +476,16 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     int tile = force_tile;
     if (tile == 0) {
         if constexpr (E == 8 && !TRANSB) {
-            if (vec && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 && tiles(256, 256) >= 128) tile = 256;
+            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 &&
+                tiles(256, 256) >= 128) tile = 256;
         }
         if (tile == 0) tile = tiles(128, 128) >= 192 ? 128 : 64;
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 256) {
             if (!(vec && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0)) return hipErrorInvalidValue;
-            return launch_gemm<T, OutT, 256, 256, 2, 4, TRANSB, true, false>(g, batch, stream);
+            if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
+            return launch_gemm_dl<T, OutT>(g, stream);
         }
     }
     if (tile == 128) {

@@ -199,6 +199,32 @@ def test_half_gemm_random_within_tolerance(be, kind, M, N, K):
         assert np.max(np.abs(got32 - oracle.gemm_f64(a, b, M, K, N))) > 1e-6
 
 
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (512, 256, 192), (768, 1024, 320), (256, 512, 4096)])
+def test_half_gemm_large_tile_direct_to_lds_path(be, kind, M, N, K):
+    # the 256 x 256 tile kernel (direct global->LDS loads, transposing LDS reads) forced on small shapes
+    be.SetGemmTile(256)
+    try:
+        rng = np.random.default_rng(M + 2 * N + 3 * K)
+        a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+        ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+        fn = oracle.hgemm if kind == "f16" else oracle.bf16gemm
+        want16, want32 = fn(ab, bb, M, K, N)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, True), want32)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, False), want16)
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+        truth = oracle.gemm_f64(aw, bw, M, K, N)
+        got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
+        assert mixed_err(got32, truth) <= 1e-4
+        # a shape the large tile does not divide is refused rather than mis-computed
+        from aidotnet.tensors_amd import HipException
+        with pytest.raises(HipException):
+            _half_gemm(be, kind, ab[:M * K - K].copy(), bb, M - 1, N, K, True)
+    finally:
+        be.SetGemmTile(0)
+
+
 def test_bf16_literal_known_answer(be):
     # BFloat16KernelsTests.cs:55-68
     ab, _ = round_to(np.array([[1, 2, 3], [4, 5, 6]], np.float32), "bf16")
