@@ -68,6 +68,7 @@ SIGNATURES = {
     "aidn_mi355_attn_decode_f16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_attn_decode_bf16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_set_gemm_tile": (_i, [_vp, _i]),
+    "aidn_mi355_set_attention_fast_path": (_i, [_vp, _i]),
 }
 
 _lib = None

@@ -138,6 +138,10 @@ class Mi355Backend:
         """Test hook: force the GEMM tile edge (0 = automatic)."""
         self._check(self._lib.aidn_mi355_set_gemm_tile(self._ctx, tile))
 
+    def SetAttentionFastPath(self, enabled: bool) -> None:
+        """Test hook: False routes every attention shape through the general kernel."""
+        self._check(self._lib.aidn_mi355_set_attention_fast_path(self._ctx, 1 if enabled else 0))
+
     # buffers -- AllocateBuffer zero-fills (HipBackend.cs:1251-1273)
     def AllocateBuffer(self, data_or_size) -> GpuBuffer:
         if isinstance(data_or_size, int):

@@ -202,6 +202,13 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
     return AIDN_OK;
 }
 
+AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
+{
+    if (!ctx) return AIDN_ERR_INVALID_ARGUMENT;
+    aidn::attn_set_fast_path(enabled);
+    return AIDN_OK;
+}
+
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
                      int M, int N, int K, float alpha, float beta, int transB)
 {

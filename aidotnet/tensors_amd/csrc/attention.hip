@@ -352,6 +352,265 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Fast path: 16-bit inputs, head dim 128, 16-byte aligned rows, no bias / mask / soft-cap.
+// Same formulation as above (S^T = K Q^T, O^T += V^T P^T), but K and V tiles go global -> LDS with the
+// gfx950 direct load (no staging registers, no ds_write, no register transposes) and V^T fragments are
+// produced by the transposing LDS read:
+//   K tile [64 keys][256 B]: 16-byte chunk c of key k at chunk position c ^ (k & 15)        (b128 reads)
+//   V tile [64 keys][256 B]: 16-byte chunk c of key k at chunk position c ^ ((k & 3) << 2)  (tr16 reads)
+// Softmax: the scale is folded into one FMA per logit (p = exp2(s * c - m)); the running max used for
+// the exponent is only raised when the true max has grown by more than 8 (log2 units), so the O
+// accumulator is rescaled rarely and P never exceeds 2^8 -- exact mathematics, LSE = m + log2(l) holds
+// for any reference point m.
+typedef short s16x4a __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void attn_dma16(const void* gptr, void* lds_dst_wave_uniform)
+{
+    uint32_t l = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds_dst_wave_uniform);
+    l = __builtin_amdgcn_readfirstlane(l);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(l), "v"(gptr));
+}
+
+template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
+{
+    return float_to_f16_bits(a) | (float_to_f16_bits(b) << 16);
+}
+template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b)
+{
+    // probabilities are finite and non-negative: the hardware round-to-nearest-even convert equals the
+    // integer rule of float_to_bf16_bits on them
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+template <typename T, typename OutT>
+__global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
+{
+    typedef uint16_t raw_t;
+    constexpr int D = 128, BC = 64, BR = 128;
+    constexpr int KBYTES = BC * 256, VBYTES = BC * 256, STAGE = KBYTES + VBYTES;
+    constexpr int DSTEPS = D / 16, KT = BC / 32, DT = D / 32;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    int bh, qt;
+    {
+        int nblk = gridDim.x, pid = blockIdx.x;
+        int per = nblk >> 3, rem = nblk & 7;
+        int xcd = pid & 7, idx = pid >> 3;
+        int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
+        bh = logical / a.qtiles;
+        qt = a.qtiles - 1 - (logical - bh * a.qtiles);
+    }
+    const int b = bh / a.H, hd = bh - b * a.H;
+    const int kvh = hd / (a.H / a.Hkv);
+    const int q0 = qt * BR;
+    const int qi = q0 + wave * 32 + l32;
+
+    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
+    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+
+    u32x4 qf[DSTEPS];
+#pragma unroll
+    for (int s = 0; s < DSTEPS; s++) {
+        u32x4 z = {0u, 0u, 0u, 0u};
+        qf[s] = (qi < a.Sq) ? *(const u32x4*)(Q + (long long)qi * a.qs[2] + (2 * s + h) * 8) : z;
+    }
+
+    int ntiles = (a.Sk + BC - 1) / BC;
+    if (a.causal) {
+        long long lastkey = (long long)q0 + BR - 1 + a.qoff;
+        if (lastkey < 0) ntiles = 0;
+        else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
+    }
+
+    // this wave's DMA: K wave-loads 4w..4w+3 and V wave-loads 4w..4w+3, each 4 keys x 256 B.
+    // lane -> (key = 4 * load + lane / 16, chunk position = lane % 16)
+    const int ld_key = lane >> 4, ld_pos = lane & 15;
+    auto issue_loads = [&](int kv0, int stage) {
+        unsigned char* ks = smem + stage * STAGE;
+        unsigned char* vs = ks + KBYTES;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int key = 4 * (wave * 4 + i) + ld_key;               // key inside the tile
+            int gkey = min(kv0 + key, a.Sk - 1);                 // clamp: rows past the end are masked later
+            attn_dma16(K + (long long)gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 8, ks + (wave * 4 + i) * 1024);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            int key = 4 * (wave * 4 + i) + ld_key;
+            int gkey = min(kv0 + key, a.Sk - 1);
+            attn_dma16(V + (long long)gkey * a.vs[2] + (ld_pos ^ ((key & 3) << 2)) * 8, vs + (wave * 4 + i) * 1024);
+        }
+    };
+
+    f32x16 oacc[DT];
+#pragma unroll
+    for (int i = 0; i < DT; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[i][r] = 0.0f;
+    float m_ref = -INFINITY;     // reference point of the exponent (log2 domain); same in lanes l and l ^ 32
+    float l_run = 0.0f;
+
+    const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
+    const float sl2 = a.scale * LOG2E;
+
+    // V^T fragment addressing (transposing read): 16-lane group, lane j addresses key (base + j/4), 8 bytes at
+    // head-dim 4 (j % 4) of the 16-wide block
+    const int jl = lane & 15;
+    const int v_rowl = 4 * h + (jl >> 2);                        // + 32 kt + 16 ps + 8 q
+    const int v_half = (jl & 1) * 8;
+    const int v_chunk0 = (16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;   // + 4 dt
+
+    if (ntiles > 0) issue_loads(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    for (int j = 0; j < ntiles; j++) {
+        const int stage = j & 1;
+        const int kv0 = j * BC;
+        if (j + 1 < ntiles) issue_loads(kv0 + BC, stage ^ 1);
+
+        const bool active = !(a.causal && (long long)kv0 > (long long)wq_max + a.qoff);
+        if (active) {
+            const unsigned char* ks = smem + stage * STAGE;
+            const unsigned char* vs = ks + KBYTES;
+
+            f32x16 st[KT];
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) st[kt][r] = 0.0f;
+#pragma unroll
+            for (int s = 0; s < DSTEPS; s++) {
+#pragma unroll
+                for (int kt = 0; kt < KT; kt++) {
+                    const int key = kt * 32 + l32;
+                    u32x4 kf = *(const u32x4*)(ks + key * 256 + (((2 * s + h) ^ (key & 15)) << 4));
+                    Mma32<T>::run(st[kt], kf, qf[s]);
+                }
+            }
+
+            const bool need_mask = (kv0 + BC > a.Sk) || (a.causal && (long long)kv0 + BC - 1 > (long long)wq_min + a.qoff);
+            float mloc = -INFINITY;
+            if (need_mask) {
+#pragma unroll
+                for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = kv0 + kt * 32 + acc_row(r, h);
+                        if (key >= a.Sk || (a.causal && (long long)key > (long long)qi + a.qoff)) st[kt][r] = -INFINITY;
+                    }
+            }
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, st[kt][r]);
+            mloc = fmaxf(mloc, shfl_xor_f(mloc, 32)) * sl2;       // scale > 0: max commutes with the scaling
+            // raise the reference only when the row max has moved by more than 8 (or on first use)
+            if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
+                const float m_new = (mloc > m_ref + 8.0f) ? mloc : m_ref;
+                const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
+                m_ref = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int i = 0; i < DT; i++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            }
+            const float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
+            float psum = 0.0f;
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float p = __builtin_amdgcn_exp2f(fmaf(st[kt][r], sl2, -m_use));
+                    st[kt][r] = p;
+                    psum += p;
+                }
+            l_run += psum;
+
+#pragma unroll
+            for (int kt = 0; kt < KT; kt++) {
+#pragma unroll
+                for (int ps = 0; ps < 2; ps++) {
+                    u32x4 pf;
+#pragma unroll
+                    for (int w = 0; w < 4; w++) pf[w] = pack2_p<T>(st[kt][8 * ps + 2 * w], st[kt][8 * ps + 2 * w + 1]);
+#pragma unroll
+                    for (int i = 0; i < DT; i++) {
+                        u32x4 vf;
+#pragma unroll
+                        for (int q = 0; q < 2; q++) {
+                            const int key = 32 * kt + 16 * ps + 8 * q + v_rowl;
+                            const int pos = (v_chunk0 + 4 * i) ^ ((key & 3) << 2);
+                            s16x4a v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                (__attribute__((address_space(3))) s16x4a*)(vs + key * 256 + pos * 16 + v_half));
+                            u32x2 w2 = __builtin_bit_cast(u32x2, v);
+                            vf[2 * q] = w2[0];
+                            vf[2 * q + 1] = w2[1];
+                        }
+                        Mma32<T>::run(oacc[i], vf, pf);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+
+    const float l_tot = l_run + shfl_xor_f(l_run, 32);
+    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (qi < a.Sq) {
+        typedef typename Raw2<OutT>::type out_t;
+        out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
+#pragma unroll
+        for (int i = 0; i < DT; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int d0 = i * 32 + 8 * g + 4 * h;
+                float v0 = oacc[i][4 * g + 0] * inv, v1 = oacc[i][4 * g + 1] * inv;
+                float v2 = oacc[i][4 * g + 2] * inv, v3 = oacc[i][4 * g + 3] * inv;
+                if constexpr (Elem<OutT>::BYTES == 4) {
+                    if (a.vec_out) *(f32x4*)(O + d0) = f32x4{v0, v1, v2, v3};
+                    else { O[d0] = as_u32(v0); O[d0 + 1] = as_u32(v1); O[d0 + 2] = as_u32(v2); O[d0 + 3] = as_u32(v3); }
+                } else {
+                    uint32_t w0 = Elem<OutT>::narrow(v0) | (Elem<OutT>::narrow(v1) << 16);
+                    uint32_t w1 = Elem<OutT>::narrow(v2) | (Elem<OutT>::narrow(v3) << 16);
+                    if (a.vec_out) *(u32x2*)(O + d0) = u32x2{w0, w1};
+                    else { O[d0] = (out_t)(w0 & 0xFFFFu); O[d0 + 1] = (out_t)(w0 >> 16); O[d0 + 2] = (out_t)(w1 & 0xFFFFu); O[d0 + 3] = (out_t)(w1 >> 16); }
+                }
+            }
+        }
+        if (a.lse && h == 0)
+            a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+    }
+}
+
+template <typename T, typename OutT>
+static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
+{
+    auto kern = attn_fwd_dl_kernel<T, OutT>;
+    constexpr int smem = 2 * (64 * 256 + 64 * 256);
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    a.qtiles = (a.Sq + 127) / 128;
+    long long nblk = (long long)a.qtiles * a.B * a.H;
+    if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
+    return hipGetLastError();
+}
+
 // Normalised probabilities P[b,h,i,j] = exp(logit - LSE[b,h,i]) for callers that ask for the
 // attention-weights tensor (the optional output of ScaledDotProductAttention,
 // src/AiDotNet.Tensors/Engines/DirectGpu/IDirectGpuBackend.cs:1421-1424).  Not on the hot path:
@@ -422,6 +681,10 @@ static hipError_t dispatch_attn_d(const AttnArgs& a, bool full, hipStream_t stre
     return hipErrorInvalidValue;
 }
 
+// Test hook: 0 routes every shape through the general kernel.
+bool g_attn_allow_dl = true;
+void attn_set_fast_path(int enabled) { g_attn_allow_dl = enabled != 0; }
+
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
 {
@@ -441,6 +704,12 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     a.vec_out = (p.D % 4 == 0) && al(p.o, p.os, oeb);
     const bool full = p.bias != nullptr || a.mask_mode != 0 || p.softcap > 0.0f;
     hipError_t err;
+    // fast path: 16-bit, head dim 128, aligned rows, plain (optionally causal) attention
+    const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && g_attn_allow_dl;
+    if (dl) {
+        if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
+        else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);
+    } else
     if (kind == 0) err = dispatch_attn_d<float, float, 32>(a, full, stream);
     else if (kind == 1) err = p.out16 ? dispatch_attn_d<f16_t, f16_t, 64>(a, full, stream) : dispatch_attn_d<f16_t, float, 64>(a, full, stream);
     else err = p.out16 ? dispatch_attn_d<bf16_t, bf16_t, 64>(a, full, stream) : dispatch_attn_d<bf16_t, float, 64>(a, full, stream);

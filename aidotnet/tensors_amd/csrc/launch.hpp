@@ -26,6 +26,7 @@ struct AttnParams {
 
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p);
+void attn_set_fast_path(int enabled);
 
 // Decode (Sq == 1).  eff_splits: the split count actually used for `splits` requested (<= 0 = auto).
 int attn_decode_splits(const AttnParams& p, int splits);

@@ -171,6 +171,10 @@ AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_att
  * Forces the GEMM tile edge (64, 128 or 256; 0 = automatic choice) for subsequent calls on this
  * context, so the parity suite can exercise every kernel instance.  No counterpart in the reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
+/* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast
+ * path is then not taken), so the parity suite can hold the two kernels against each other.  Process-wide.
+ * No counterpart in the reference. */
+AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled);
 
 #ifdef __cplusplus
 }

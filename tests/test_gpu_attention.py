@@ -265,3 +265,65 @@ def test_config4_half_causal_b4_h32_s2048_d128(be, kind):
         o64, lse64 = oracle.attention_f64(qs, ks, vs, scale, True)
         assert mixed_err(out[b, h].cpu().numpy(), o64[0, 0]) <= HALF_TOL
         assert mixed_err(lse[b, h].cpu().numpy(), lse64[0, 0]) <= 1e-3
+
+
+# --------------------------------------------------------------- head-dim-128 fast path (direct-to-LDS kernel)
+FAST_CASES = [
+    (1, 1, 1, 1, 1, False, 0),
+    (1, 2, 2, 5, 9, False, 0),
+    (2, 3, 3, 128, 128, True, 0),
+    (1, 2, 1, 130, 200, True, 70),        # GQA, bottom-right causal, ragged tiles
+    (1, 4, 4, 257, 63, True, 0),          # Sq > Sk top-left causal: one partial K/V tile
+    (2, 2, 2, 64, 1000, False, 0),
+    (1, 2, 2, 1, 4097, True, 4096),       # decode shape through the prefill kernel
+    (1, 1, 1, 300, 300, True, 0),
+]
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES)
+def test_fast_path_d128_matches_oracle_and_general_kernel(be, kind, B, H, Hkv, Sq, Sk, causal, offset):
+    D = 128
+    rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + len(kind))
+    q, k, v = _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+    scale = 1.0 / math.sqrt(D)
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale, causal, offset)
+    dt = TORCH16[kind]
+    args = (be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)))
+    outs = {}
+    try:
+        for fast in (True, False):
+            be.SetAttentionFastPath(fast)
+            out = torch.full((B, H, Sq, D), float("nan"), device="cuda")
+            lse = torch.full((B, H, Sq), float("nan"), device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out), be.WrapTensor(lse), B, H, Sq, Sk, D, scale, causal, offset, Hkv)
+            outs[fast] = (out.cpu().numpy(), lse.cpu().numpy())
+            assert mixed_err(outs[fast][0], o64) <= HALF_TOL
+            assert mixed_err(outs[fast][1], lse64) <= 1e-3
+        # the two kernels agree far inside the 16-bit tolerance (both round P to 16 bits, at different scalings)
+        assert mixed_err(outs[True][0], outs[False][0]) <= 1e-2
+        be.SetAttentionFastPath(True)
+        out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
+        be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
+        assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
+    finally:
+        be.SetAttentionFastPath(True)
+
+
+def test_fast_path_all_masked_rows_and_large_logits(be):
+    # rows above the diagonal with a negative offset see no key: O = 0, LSE = -inf (CpuEngine.cs:29243-29249);
+    # logits of magnitude ~60 exercise the lazily raised exponent reference
+    B, H, S, D = 1, 2, 200, 128
+    rng = np.random.default_rng(77)
+    q, k, v = 3 * _rand(rng, B, H, S, D), 3 * _rand(rng, B, H, S, D), _rand(rng, B, H, S, D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, "bf16"), round_to(k, "bf16"), round_to(v, "bf16")
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, 0.5, True, -3)
+    dt = torch.bfloat16
+    out = torch.full((B, H, S, D), float("nan"), device="cuda"); lse = torch.full((B, H, S), float("nan"), device="cuda")
+    be.FlashAttentionHalf("bf16", be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)),
+                          be.WrapTensor(out), be.WrapTensor(lse), B, H, S, S, D, 0.5, True, -3)
+    o = out.cpu().numpy(); l = lse.cpu().numpy()
+    assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
+    assert mixed_err(o, o64) <= HALF_TOL
+    assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
