@@ -26,6 +26,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what the
+# same counter reads for a 1 GiB device copy; the runs and factors are in profiles/ (one summary per kernel).  None = not
+# measured yet.
+TRAFFIC_BYTES = {
+    "gemm_f16_8192": None,
+    "decode_bf16": None,
+    "attn_f16_prefill": None,
+    "attn_bf16_prefill": None,
+}
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
@@ -66,6 +75,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--only", default="", help="comma list of workloads to time besides the headline (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 1 GiB device copies (a plain copy kernel of known size) so that FETCH_SIZE / "
+                         "WRITE_SIZE counters collected over this command can be scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards without "
@@ -103,7 +115,7 @@ def main() -> int:
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "fp16 GEMM C=A*B, M=N=K=8192, fp32 accumulate, fp16 out (A~N(0,1), B~N(0,0.02^2), seeded)",
                    "wall_ms_per_step": round(wall_ms, 5)},
-        "roofline": _roof_flops("f16", flops, ms),
+        "roofline": _roof_flops("f16", flops, ms, TRAFFIC_BYTES.get("gemm_f16_8192")),
     }
     del a, b, c
 
@@ -161,7 +173,7 @@ def main() -> int:
             fn = lambda: be.FlashAttentionHalf(kind, W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, sc, True)
         ms_, _ = _events_time(torch, fn, steps, warmup)
         exact = 4.0 * Bn * H * D * (S * (S + 1) / 2)
-        roof = _roof_flops(kind, exact, ms_)
+        roof = _roof_flops(kind, exact, ms_, TRAFFIC_BYTES.get(name))
         roof["tflops_full_matrix_convention"] = round(4.0 * Bn * H * S * S * D / (ms_ * 1e-3) / 1e12, 3)
         add(name, kind, "causal attention B=%d H=%d S=%d d=%d (fp32 softmax/accumulate, fp32 O + LSE)" % (Bn, H, S, D), ms_, roof)
 
@@ -174,7 +186,7 @@ def main() -> int:
         fn = lambda: be.DecodeAttention(kind, W(q), W(k), W(v), W(o), Bn, H, S, D, sc)
         ms_, _ = _events_time(torch, fn, steps, warmup)
         nbytes = 2.0 * Bn * H * S * D * q.element_size()
-        add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_))
+        add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)))
 
     gemm_case("gemm_f32_1024", "f32", 1024, 1024, 1024, wstd=1.0)
     gemm_case("gemm_f32_proj", "f32", 4096, 3072, 768)
@@ -188,28 +200,36 @@ def main() -> int:
     gemm_case("gemm_bf16_decode_proj", "bf16", 32, 4096, 4096, hbm=True, rotate=12)
     out["others"] = others
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_(generator=g)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
     if not args.no_cpu:
         try:
             import numpy as np
             import oracle      # test infrastructure: used here only as the reported CPU baseline
             threads = min(oracle.max_threads(), os.cpu_count() or 1)
-            ms_rows = 1024     # a 1024-row slab of the 8192^3 product, fp32 path on widened inputs
+            ms_rows = 8192     # the whole 8192^3 product, fp32 path on widened inputs (about 2 s per pass on 16 cores)
             rng = np.random.default_rng(0)
             ah = rng.standard_normal((ms_rows, n)).astype(np.float16).astype(np.float32)
             bh = (0.02 * rng.standard_normal((n, n))).astype(np.float16).astype(np.float32)
-            oracle.sgemm(ah[:64], bh, 64, n, n, threads=threads)      # warm-up
+            oracle.sgemm(ah[:256], bh, 256, n, n, threads=threads)    # warm-up
             times = []
-            for _ in range(3):
+            for _ in range(5):
                 t0 = time.perf_counter()
                 oracle.sgemm(ah, bh, ms_rows, n, n, threads=threads)
                 times.append(time.perf_counter() - t0)
-            tsec = sorted(times)[1]
+            tsec = sorted(times)[len(times) // 2]
             out["cpu_baseline"] = {
                 "value": round(2.0 * ms_rows * n * n / tsec / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
                 "sample": "C restatement of the reference SimdGemm (6x16 AVX2 FMA tile, Kc=512, 2-D tile parallelism) on a "
                           "%d-row slab of the 8192^3 product (%d x 8192 x 8192, fp32 path on fp16-rounded inputs), "
-                          "median of 3, %.2f s each" % (ms_rows, ms_rows, tsec),
+                          "median of 5, %.2f s each" % (ms_rows, ms_rows, tsec),
             }
         except Exception as ex:     # the baseline is a reported extra, never the product path
             out["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": 0, "kind": "port", "sample": "failed: %r" % (ex,)}
