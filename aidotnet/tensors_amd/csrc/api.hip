@@ -133,7 +133,14 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: dimensions must be positive");
-    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile), "gemm_16");
+    void* ws = nullptr;
+    size_t need = c->force_tile == 0 ? aidn::gemm_16_workspace_bytes(M, N, K) : 0;
+    if (need) {
+        int st = ensure_ws(c, need);
+        if (st) return st;
+        ws = c->ws;
+    }
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws), "gemm_16");
 }
 
 int convert_common(void* ctx, void* stream, int kind, const void* in, void* out, int64_t n)

@@ -443,6 +443,145 @@ static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny-M path (decode projections): M <= 32, 16-bit, B stored [K,N], N % 128 == 0, K % 64 == 0.
+// HBM-bound: B (K x N) is read exactly once.  grid = (N / 128, KS): each workgroup streams a 128-column
+// slab of B over its K range with the direct global->LDS load (two 20 KB stages, several workgroups per
+// CU so many loads are in flight), computes a 32 x 128 partial product on MFMA (A rows beyond M are
+// clamped duplicates that are never stored) and writes it either to C (KS == 1) or to an fp32 workspace
+// that skinny_reduce_kernel sums in split order (deterministic) and narrows.
+//   B tile [64 k][256 B]: chunk c of row k at position c ^ ((k & 3) << 2)   (transposing reads)
+//   A tile [32 m][128 B]: chunk c of row m at position c ^ ((m >> 1) & 7)   (b128 reads)
+template <typename T>
+__global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
+{
+    typedef uint16_t raw_t;
+    constexpr int BK = 64;
+    constexpr int ABYTES = 32 * 128, BBYTES = BK * 256, STAGE = ABYTES + BBYTES;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGE];
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * 128;
+    const int ks = blockIdx.y;
+    const int kbeg = ks * kper;
+    const int KT = kper / BK;
+    const raw_t* __restrict__ A = (const raw_t*)g.A;
+    const raw_t* __restrict__ B = (const raw_t*)g.B;
+
+    // this wave's DMA per K-tile: 4 B wave-loads (k-rows 4w'..4w'+3, w' = 4*wave+i) and A wave-load `wave` (rows 8*wave..)
+    const raw_t* pb[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int row = 4 * (wave * 4 + i) + (lane >> 4), pos = lane & 15;
+        pb[i] = B + (long long)(kbeg + row) * g.ldb + n0 + (pos ^ ((row & 3) << 2)) * 8;
+    }
+    const raw_t* pa;
+    {
+        int row = 8 * wave + (lane >> 3), pos = lane & 7;
+        int grow = min(row, g.M - 1);
+        pa = A + (long long)grow * g.lda + kbeg + (pos ^ ((row >> 1) & 7)) * 8;
+    }
+    auto issue_loads = [&](int kt, int stage) {
+        unsigned char* as = smem + stage * STAGE;
+        unsigned char* bs = as + ABYTES;
+        dma16_to_lds(pa + kt * BK, as + wave * 1024);
+#pragma unroll
+        for (int i = 0; i < 4; i++) dma16_to_lds(pb[i] + (long long)kt * BK * g.ldb, bs + (wave * 4 + i) * 1024);
+    };
+
+    const int a_off = l32 * 128, a_sw = (l32 >> 1) & 7;
+    const int jl = lane & 15;
+    const int b_rowl = 8 * h + (jl >> 2);
+    const int b_half = (jl & 1) * 8;
+    const int b_chunk = (wave * 32 + 16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    issue_loads(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; kt++) {
+        const int stage = kt & 1;
+        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+        const unsigned char* as = smem + stage * STAGE;
+        const unsigned char* bs = as + ABYTES;
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            u32x4 fa = *(const u32x4*)(as + a_off + (((2 * s + h) ^ a_sw) << 4));
+            u32x4 fb;
+#pragma unroll
+            for (int q = 0; q < 2; q++) {
+                int row = 16 * s + 4 * q + b_rowl;
+                int pos = b_chunk ^ ((row & 3) << 2);
+                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (__attribute__((address_space(3))) s16x4*)(bs + row * 256 + pos * 16 + b_half));
+                u32x2 w = __builtin_bit_cast(u32x2, v);
+                fb[2 * q] = w[0];
+                fb[2 * q + 1] = w[1];
+            }
+            Mma32<T>::run(acc, fa, fb);
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
+
+    const int col = n0 + wave * 32 + l32;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = acc_row(r, h);
+        if (row < g.M) ws[((long long)ks * g.M + row) * g.N + col] = acc[r];
+    }
+}
+
+template <typename OutT>
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv, int M, int N, int ksplit)
+{
+    typedef typename Raw<OutT>::type out_t;
+    out_t* C = (out_t*)Cv;
+    const long long total = (long long)M * N;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
+        float s = 0.0f;
+        for (int k = 0; k < ksplit; k++) s += ws[(long long)k * total + i];
+        if constexpr (Elem<OutT>::BYTES == 4) C[i] = as_u32(s);
+        else C[i] = (out_t)Elem<OutT>::narrow(s);
+    }
+}
+
+static bool skinny_applies(int M, int N, int K) { return M <= 32 && N % 128 == 0 && K % 64 == 0 && N >= 128; }
+
+static int skinny_ksplit(int N, int K)
+{
+    int slabs = N / 128, tiles = K / 64;
+    int ks = (768 + slabs - 1) / slabs;          // about three workgroups per CU
+    if (ks > tiles) ks = tiles;
+    if (ks < 1) ks = 1;
+    while (tiles % ks != 0) ks--;                // equal K ranges, each a multiple of 64
+    return ks;
+}
+
+size_t gemm_16_workspace_bytes(int M, int N, int K)
+{
+    if (!skinny_applies(M, N, K)) return 0;
+    return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
+}
+
+template <typename T, typename OutT>
+static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
+{
+    const int ks = skinny_ksplit(g.N, g.K);
+    const int kper = g.K / ks;
+    hipLaunchKernelGGL((gemm_skinny_kernel<T>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), 0, stream, g, ws, ks, kper);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    long long total = (long long)g.M * g.N;
+    unsigned grid = (unsigned)((total + 255) / 256);
+    hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks);
+    return hipGetLastError();
+}
+
 // ------------------------------------------------------------------ host side
 template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK>
 static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
@@ -510,9 +649,14 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
 
 // kind: 0 = fp16, 1 = bf16; out32: C is fp32 (else the same 16-bit type as the inputs)
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile)
+                   int M, int N, int K, int force_tile, void* workspace)
 {
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0};
+    if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
+        float* ws = (float*)workspace;
+        if (kind == 0) return out32 ? launch_skinny<f16_t, float>(g, stream, ws) : launch_skinny<f16_t, f16_t>(g, stream, ws);
+        return out32 ? launch_skinny<bf16_t, float>(g, stream, ws) : launch_skinny<bf16_t, bf16_t>(g, stream, ws);
+    }
     if (kind == 0) {
         if (out32) return dispatch_gemm<f16_t, float, false>(g, 1, stream, force_tile);
         return dispatch_gemm<f16_t, f16_t, false>(g, 1, stream, force_tile);

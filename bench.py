@@ -30,10 +30,11 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # same counter reads for a 1 GiB device copy; the runs and factors are in profiles/ (one summary per kernel).  None = not
 # measured yet.
 TRAFFIC_BYTES = {
-    "gemm_f16_8192": None,
-    "decode_bf16": None,
-    "attn_f16_prefill": None,
-    "attn_bf16_prefill": None,
+    # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes)
+    "gemm_f16_8192": int((792204 * 2.0 + 134918) * 1024),
+    "decode_bf16": int((1048959 * 2.0 + 1088) * 1024),
+    "attn_f16_prefill": int((98762 * 2.0 + 132098) * 1024),
+    "attn_bf16_prefill": int((98443 * 2.0 + 132096) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
