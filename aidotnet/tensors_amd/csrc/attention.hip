@@ -365,11 +365,17 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 // for any reference point m.
 typedef short s16x4a __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void attn_dma16(const void* gptr, void* lds_dst_wave_uniform)
+// Direct global -> LDS load of 16 bytes per lane: lane i's data lands at LDS address lds_dst + 16 i (lds_dst wave
+// uniform).  Issued from inline asm so the compiler does not order later LDS reads behind it; completion is
+// awaited explicitly (s_waitcnt vmcnt(0) + barrier) before the tile is read.
+__device__ __forceinline__ void attn_dma16(const void* gptr, uint32_t lds_dst)
 {
-    uint32_t l = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)lds_dst_wave_uniform);
-    l = __builtin_amdgcn_readfirstlane(l);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(l), "v"(gptr));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_dst), "v"(gptr) : "memory");
+}
+// same, source = wave-uniform base (SGPR pair) + per-lane unsigned 32-bit byte offset
+__device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
 }
 
 template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
@@ -391,8 +397,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 {
     typedef uint16_t raw_t;
     constexpr int D = 128, BC = 64, BR = 128;
-    constexpr int KBYTES = BC * 256, VBYTES = BC * 256, STAGE = KBYTES + VBYTES;
-    constexpr int DSTEPS = D / 16, KT = BC / 32, DT = D / 32;
+    constexpr int KBYTES = BC * 256, VBYTES = BC * 256;
+    constexpr int DSTEPS = D / 16, DT = D / 32;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -430,23 +436,46 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
     }
 
-    // this wave's DMA: K wave-loads 4w..4w+3 and V wave-loads 4w..4w+3, each 4 keys x 256 B.
-    // lane -> (key = 4 * load + lane / 16, chunk position = lane % 16)
+    // LDS: K ring [2][KBYTES] then V ring [2][VBYTES].  This wave's DMA per tile: K wave-loads 4w..4w+3 and V
+    // wave-loads 4w..4w+3, each 4 keys x 256 B; lane -> (key = 4 * load + lane / 16, chunk position = lane % 16).
+    // For a tile that lies fully inside the sequence the source address is a scalar base (tile, wave, load) plus
+    // a per-lane byte offset fixed for the whole kernel, so issuing a load costs no vector arithmetic.
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const int ld_key = lane >> 4, ld_pos = lane & 15;
-    auto issue_loads = [&](int kv0, int stage) {
-        unsigned char* ks = smem + stage * STAGE;
-        unsigned char* vs = ks + KBYTES;
+    const long long k_row_bytes = a.ks[2] * 2, v_row_bytes = a.vs[2] * 2;
+    uint32_t k_lane_off[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int key = 4 * (wave * 4 + i) + ld_key;               // key inside the tile
-            int gkey = min(kv0 + key, a.Sk - 1);                 // clamp: rows past the end are masked later
-            attn_dma16(K + (long long)gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 8, ks + (wave * 4 + i) * 1024);
+    for (int i = 0; i < 4; i++) k_lane_off[i] = (uint32_t)(ld_key * k_row_bytes) + ((ld_pos ^ (4 * i + ld_key)) << 4);
+    const uint32_t v_lane_off = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (ld_key << 2)) << 4);
+    auto issue_k = [&](int tile) {
+        const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * 4096;
+        if (tile * BC + BC <= a.Sk) {
+            const unsigned char* src = (const unsigned char*)K + (long long)(tile * BC + 16 * wave_s) * k_row_bytes;
+#pragma unroll
+            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                int key = 4 * (wave * 4 + i) + ld_key;               // key inside the tile
+                int gkey = min(tile * BC + key, a.Sk - 1);           // clamp: rows past the end are masked later
+                attn_dma16(K + (long long)gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 8, dst + i * 1024);
+            }
         }
+    };
+    auto issue_v = [&](int tile) {
+        const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * 4096;
+        if (tile * BC + BC <= a.Sk) {
+            const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            int key = 4 * (wave * 4 + i) + ld_key;
-            int gkey = min(kv0 + key, a.Sk - 1);
-            attn_dma16(V + (long long)gkey * a.vs[2] + (ld_pos ^ ((key & 3) << 2)) * 8, vs + (wave * 4 + i) * 1024);
+            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                int key = 4 * (wave * 4 + i) + ld_key;
+                int gkey = min(tile * BC + key, a.Sk - 1);
+                attn_dma16(V + (long long)gkey * a.vs[2] + (ld_pos ^ ((key & 3) << 2)) * 8, dst + i * 1024);
+            }
         }
     };
 
@@ -460,112 +489,167 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
     const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
     const float sl2 = a.scale * LOG2E;
+    // tiles this wave computes: under a causal mask a prefix of the workgroup's tiles
+    int nact = ntiles;
+    if (a.causal) {
+        long long lk = (long long)wq_max + a.qoff;
+        if (lk < 0) nact = 0;
+        else { long long nt = lk / BC + 1; if (nt < nact) nact = (int)nt; }
+    }
 
-    // V^T fragment addressing (transposing read): 16-lane group, lane j addresses key (base + j/4), 8 bytes at
-    // head-dim 4 (j % 4) of the 16-wide block
+    // Fragment addressing.  K (b128 reads): lane reads key l32 (+ 32 per sub-tile), chunk (2 s + h) ^ (key & 15).
+    // V^T (transposing reads): in a 16-lane group lane j addresses key (base + j / 4), 8 bytes at head-dim
+    // 4 (j % 4) of the 16-wide block; chunk position (c + 4 dt) ^ ((key & 3) << 2).
     const int jl = lane & 15;
-    const int v_rowl = 4 * h + (jl >> 2);                        // + 32 kt + 16 ps + 8 q
-    const int v_half = (jl & 1) * 8;
-    const int v_chunk0 = (16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;   // + 4 dt
+    const uint32_t k_lane = l32 * 256 + ((h ^ (l32 & 15)) << 4);
+    const uint32_t v_lane = (4 * h + (jl >> 2)) * 256 + ((16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3) * 16 + (jl & 1) * 8
+                          + ((jl >> 2) << 6);
 
-    if (ntiles > 0) issue_loads(0, 0);
+    // last key a query may see (sequence end and causal diagonal folded into one 32-bit bound); klim carries the
+    // lane's accumulator row offset 4 h so that the per-element test is against a constant
+    auto key_limit = [&](int q) -> int {
+        long long lim = a.Sk - 1;
+        if (a.causal) { long long c = (long long)q + a.qoff; if (c < lim) lim = c; }
+        return (int)(lim < -1 ? -1 : lim);
+    };
+    const int klim = key_limit(qi) - 4 * h;
+    const int wave_klim = __builtin_amdgcn_readfirstlane(key_limit(wq_min));
+
+    if (ntiles > 0) { issue_k(0); issue_v(0); }
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
+    // raise the exponent reference only when a row max has moved by more than 8 (or on first use)
+    auto lazy_rescale = [&](float mloc) {
+        if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
+            const float m_new = (mloc > m_ref + 8.0f) ? mloc : m_ref;
+            const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
+            m_ref = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+        }
+    };
+    // p = exp2(s * c - m) of two scores, packed; returns their sum
+    auto exp_pair = [&](float s0, float s1, float m_use, uint32_t& packed) -> float {
+        float p0 = __builtin_amdgcn_exp2f(fmaf(s0, sl2, -m_use));
+        float p1 = __builtin_amdgcn_exp2f(fmaf(s1, sl2, -m_use));
+        packed = pack2_p<T>(p0, p1);
+        return p0 + p1;
+    };
+
+    // Per tile (64 keys = two 32-key sub-tiles) the work of a wave is pipelined so that the exponentials sit in
+    // the shadow of the matrix pipe:   S0 = QK(sub 0) | S1 = QK(sub 1) with exp(S0) | PV(sub 0) with exp(S1) | PV(sub 1)
     for (int j = 0; j < ntiles; j++) {
         const int stage = j & 1;
-        const int kv0 = j * BC;
-        if (j + 1 < ntiles) issue_loads(kv0 + BC, stage ^ 1);
-
-        const bool active = !(a.causal && (long long)kv0 > (long long)wq_max + a.qoff);
-        if (active) {
-            const unsigned char* ks = smem + stage * STAGE;
-            const unsigned char* vs = ks + KBYTES;
-
-            f32x16 st[KT];
+        if (j + 1 < ntiles) { issue_k(j + 1); issue_v(j + 1); }
+        if (j < nact) {
+            const int kv0 = j * BC;
+            const bool need_mask = kv0 + BC - 1 > wave_klim;
+            const int rel_lim = klim - kv0;                   // keys of this tile with index > rel_lim are masked
+            auto mask_sub = [&](int kt, f32x16& st) {
 #pragma unroll
-            for (int kt = 0; kt < KT; kt++)
+                for (int r = 0; r < 16; r++)
+                    if (kt * 32 + 8 * (r >> 2) + (r & 3) > rel_lim) st[r] = -INFINITY;
+            };
+            auto sub_max = [&](const f32x16& st) -> float {
+                float m = -INFINITY;
 #pragma unroll
-                for (int r = 0; r < 16; r++) st[kt][r] = 0.0f;
+                for (int r = 0; r < 16; r++) m = fmaxf(m, st[r]);
+                return max_with_partner32(m) * sl2;            // scale > 0: max commutes with the scaling
+            };
+
+            // Fragment addresses: the swizzle is an XOR on address bits that only the lane's chunk index occupies,
+            // so one base per tile and lane serves every step (XOR with a constant, then an immediate offset).
+            const uint32_t kA = lds0 + stage * KBYTES + k_lane;
+            const uint32_t vA = lds0 + 2 * KBYTES + stage * VBYTES + v_lane;
+            auto k_frag = [&](int kt, int s) -> u32x4 {
+                return *(const __attribute__((address_space(3))) u32x4*)((kA ^ (uint32_t)(s << 5)) + kt * 32 * 256);
+            };
+            auto v_frag8 = [&](int kt, int s) -> u32x4 {          // s = 4 * (16-key half) + head-dim block
+                const uint32_t ad = (vA ^ (uint32_t)((s & 3) << 6)) + (32 * kt + 16 * (s >> 2)) * 256;
+                u32x2 w0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)ad));
+                u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 8 * 256)));
+                return u32x4{w0[0], w0[1], w1[0], w1[1]};
+            };
+
+            // LDS fragment reads run four ahead of the MFMAs that consume them (fr[] is a 4-deep ring);
+            // sched_barrier pins that order and the MFMA / exp interleave.
+            // ---- S0 = K[0:32] Q^T
+            f32x16 s0, s1;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
+            u32x4 fr[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++) fr[s] = k_frag(0, s);
 #pragma unroll
             for (int s = 0; s < DSTEPS; s++) {
-#pragma unroll
-                for (int kt = 0; kt < KT; kt++) {
-                    const int key = kt * 32 + l32;
-                    u32x4 kf = *(const u32x4*)(ks + key * 256 + (((2 * s + h) ^ (key & 15)) << 4));
-                    Mma32<T>::run(st[kt], kf, qf[s]);
-                }
+                Mma32<T>::run(s0, fr[s & 3], qf[s]);
+                fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
+                __builtin_amdgcn_sched_barrier(0);
             }
+            if (need_mask) mask_sub(0, s0);
+            lazy_rescale(sub_max(s0));
+            float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
 
-            const bool need_mask = (kv0 + BC > a.Sk) || (a.causal && (long long)kv0 + BC - 1 > (long long)wq_min + a.qoff);
-            float mloc = -INFINITY;
-            if (need_mask) {
-#pragma unroll
-                for (int kt = 0; kt < KT; kt++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int key = kv0 + kt * 32 + acc_row(r, h);
-                        if (key >= a.Sk || (a.causal && (long long)key > (long long)qi + a.qoff)) st[kt][r] = -INFINITY;
-                    }
-            }
-#pragma unroll
-            for (int kt = 0; kt < KT; kt++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mloc = fmaxf(mloc, st[kt][r]);
-            mloc = fmaxf(mloc, shfl_xor_f(mloc, 32)) * sl2;       // scale > 0: max commutes with the scaling
-            // raise the reference only when the row max has moved by more than 8 (or on first use)
-            if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
-                const float m_new = (mloc > m_ref + 8.0f) ? mloc : m_ref;
-                const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
-                m_ref = m_new;
-                l_run *= alpha;
-#pragma unroll
-                for (int i = 0; i < DT; i++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
-            }
-            const float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
+            // ---- S1 = K[32:64] Q^T interleaved with P0 = exp(S0)
+            u32x4 p0f[2], p1f[2];
             float psum = 0.0f;
 #pragma unroll
-            for (int kt = 0; kt < KT; kt++)
+            for (int s = 0; s < DSTEPS; s++) {
+                Mma32<T>::run(s1, fr[s & 3], qf[s]);
+                fr[s & 3] = s + 4 < DSTEPS ? k_frag(1, s + 4) : v_frag8(0, s + 4 - DSTEPS);
+                uint32_t pk;
+                psum += exp_pair(s0[2 * s], s0[2 * s + 1], m_use, pk);
+                asm volatile("" : "+v"(pk), "+v"(psum));       // keeps the exponentials here, between the MFMAs
+                p0f[s >> 2][s & 3] = pk;
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (need_mask) mask_sub(1, s1);
+            const float mloc1 = sub_max(s1);
+            // ---- O^T += V[0:32]^T P0^T interleaved with P1 = exp(S1) against the standing reference
+            float psum1 = 0.0f;
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    float p = __builtin_amdgcn_exp2f(fmaf(st[kt][r], sl2, -m_use));
-                    st[kt][r] = p;
-                    psum += p;
-                }
+            for (int s = 0; s < 8; s++) {
+                Mma32<T>::run(oacc[s & 3], fr[s & 3], p0f[s >> 2]);
+                fr[s & 3] = s + 4 < 8 ? v_frag8(0, s + 4) : v_frag8(1, s + 4 - 8);
+                uint32_t pk;
+                psum1 += exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk);
+                asm volatile("" : "+v"(pk), "+v"(psum1));
+                p1f[s >> 2][s & 3] = pk;
+                __builtin_amdgcn_sched_barrier(0);
+            }
             l_run += psum;
-
+            if (__builtin_amdgcn_ballot_w64(mloc1 > m_ref + 8.0f) != 0ull) {
+                // rare: the second sub-tile raises the reference.  P0 (formed against the old one) is already
+                // accumulated; O and l are rescaled and P1 is formed again against the new reference (the
+                // values computed above may have overflowed and are dropped).
+                lazy_rescale(mloc1);
+                m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
+                psum1 = 0.0f;
 #pragma unroll
-            for (int kt = 0; kt < KT; kt++) {
-#pragma unroll
-                for (int ps = 0; ps < 2; ps++) {
-                    u32x4 pf;
-#pragma unroll
-                    for (int w = 0; w < 4; w++) pf[w] = pack2_p<T>(st[kt][8 * ps + 2 * w], st[kt][8 * ps + 2 * w + 1]);
-#pragma unroll
-                    for (int i = 0; i < DT; i++) {
-                        u32x4 vf;
-#pragma unroll
-                        for (int q = 0; q < 2; q++) {
-                            const int key = 32 * kt + 16 * ps + 8 * q + v_rowl;
-                            const int pos = (v_chunk0 + 4 * i) ^ ((key & 3) << 2);
-                            s16x4a v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                (__attribute__((address_space(3))) s16x4a*)(vs + key * 256 + pos * 16 + v_half));
-                            u32x2 w2 = __builtin_bit_cast(u32x2, v);
-                            vf[2 * q] = w2[0];
-                            vf[2 * q + 1] = w2[1];
-                        }
-                        Mma32<T>::run(oacc[i], vf, pf);
-                    }
+                for (int s = 0; s < 8; s++) {
+                    uint32_t pk;
+                    psum1 += exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk);
+                    p1f[s >> 2][s & 3] = pk;
                 }
             }
+            l_run += psum1;
+
+            // ---- O^T += V[32:64]^T P1^T
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                Mma32<T>::run(oacc[s & 3], fr[s & 3], p1f[s >> 2]);
+                if (s + 4 < 8) fr[s & 3] = v_frag8(1, s + 4);
+            }
         }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
+        __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA of tile j+1 has landed ...
+        __syncthreads();                    // ... everyone's has, and everyone is done with tile j
     }
 
-    const float l_tot = l_run + shfl_xor_f(l_run, 32);
+    const float l_tot = sum_with_partner32(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
@@ -705,7 +789,9 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     const bool full = p.bias != nullptr || a.mask_mode != 0 || p.softcap > 0.0f;
     hipError_t err;
     // fast path: 16-bit, head dim 128, aligned rows, plain (optionally causal) attention
-    const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && g_attn_allow_dl;
+    // the fast kernel addresses K/V rows of a 4-key load group with unsigned 32-bit byte offsets
+    const bool rows32 = p.ks[2] > 0 && p.ks[2] < (1LL << 28) && p.vs[2] > 0 && p.vs[2] < (1LL << 28);
+    const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && rows32 && g_attn_allow_dl;
     if (dl) {
         if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
         else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);

@@ -135,4 +135,18 @@ __device__ __forceinline__ void transpose4x4_b32(const u32x4 (&in)[4], u32x4 (&o
 // ---------------------------------------------------------------- wave helpers
 __device__ __forceinline__ float shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, WAVE); }
 
+// Value held by lane (l ^ 32), through the gfx950 half-wave swap (a VALU operation, no LDS round trip):
+// after v_permlane32_swap(a = v, b = v) register a holds the low half's values in both halves and b the
+// high half's, so lane l < 32 finds its partner in b and lane l >= 32 in a.
+__device__ __forceinline__ void half_swap(float v, float& lo_half, float& hi_half)
+{
+    uint32_t u = as_u32(v);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    uint32_t a = r[0], b = r[1];
+    lo_half = as_f32(a);
+    hi_half = as_f32(b);
+}
+__device__ __forceinline__ float max_with_partner32(float v) { float a, b; half_swap(v, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float sum_with_partner32(float v) { float a, b; half_swap(v, a, b); return a + b; }
+
 }  // namespace aidn
