@@ -20,6 +20,7 @@
 // tile j and stored after them, one barrier per tile.
 #include "common.hpp"
 #include "launch.hpp"
+#include <type_traits>
 
 namespace aidn {
 
@@ -381,7 +382,26 @@ __device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32
 template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
 {
-    return float_to_f16_bits(a) | (float_to_f16_bits(b) << 16);
+    // one packed round-to-nearest-even convert (v_cvt_pk_f16_f32)
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    f2 x = {a, b};
+    h2 v = __builtin_convertvector(x, h2);
+    return __builtin_bit_cast(uint32_t, v);
+}
+// acc + lo + hi of a packed pair (one VALU operation)
+template <typename T> __device__ __forceinline__ float add_pair(uint32_t packed, float acc);
+template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t packed, float acc)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), ones, acc, false);
+}
+template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t packed, float acc)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    const bf2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, packed), ones, acc, false);
 }
 template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b)
 {
@@ -532,18 +552,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
         }
     };
-    // p = exp2(s * c - m) of two scores, packed; returns their sum
-    auto exp_pair = [&](float s0, float s1, float m_use, uint32_t& packed) -> float {
+    // p = exp2(s * c - m) of two scores, rounded and packed; the row sum accumulates the rounded values (the
+    // same numbers the P V product uses) with one dot instruction per pair
+    auto exp_pair = [&](float s0, float s1, float m_use, uint32_t& packed, float& sum) {
         float p0 = __builtin_amdgcn_exp2f(fmaf(s0, sl2, -m_use));
         float p1 = __builtin_amdgcn_exp2f(fmaf(s1, sl2, -m_use));
         packed = pack2_p<T>(p0, p1);
-        return p0 + p1;
+        sum = add_pair<T>(packed, sum);
     };
 
     // Per tile (64 keys = two 32-key sub-tiles) the work of a wave is pipelined so that the exponentials sit in
     // the shadow of the matrix pipe:   S0 = QK(sub 0) | S1 = QK(sub 1) with exp(S0) | PV(sub 0) with exp(S1) | PV(sub 1)
-    for (int j = 0; j < ntiles; j++) {
-        const int stage = j & 1;
+    // invariant per-lane read addresses; ring stage, sub-tile and key block enter as immediate offsets
+    uint32_t k_ad[DSTEPS], v_ad[DT];
+#pragma unroll
+    for (int s = 0; s < DSTEPS; s++) k_ad[s] = (lds0 + k_lane) ^ (uint32_t)(s << 5);
+#pragma unroll
+    for (int i = 0; i < DT; i++) v_ad[i] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(i << 6);
+
+    auto tile_body = [&](const int j, auto stage_c) {
+        constexpr int stage = decltype(stage_c)::value;
         if (j + 1 < ntiles) { issue_k(j + 1); issue_v(j + 1); }
         if (j < nact) {
             const int kv0 = j * BC;
@@ -563,13 +591,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
             // Fragment addresses: the swizzle is an XOR on address bits that only the lane's chunk index occupies,
             // so one base per tile and lane serves every step (XOR with a constant, then an immediate offset).
-            const uint32_t kA = lds0 + stage * KBYTES + k_lane;
-            const uint32_t vA = lds0 + 2 * KBYTES + stage * VBYTES + v_lane;
             auto k_frag = [&](int kt, int s) -> u32x4 {
-                return *(const __attribute__((address_space(3))) u32x4*)((kA ^ (uint32_t)(s << 5)) + kt * 32 * 256);
+                return *(const __attribute__((address_space(3))) u32x4*)(k_ad[s] + stage * KBYTES + kt * 32 * 256);
             };
             auto v_frag8 = [&](int kt, int s) -> u32x4 {          // s = 4 * (16-key half) + head-dim block
-                const uint32_t ad = (vA ^ (uint32_t)((s & 3) << 6)) + (32 * kt + 16 * (s >> 2)) * 256;
+                const uint32_t ad = v_ad[s & 3] + stage * VBYTES + (32 * kt + 16 * (s >> 2)) * 256;
                 u32x2 w0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)ad));
                 u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 8 * 256)));
                 return u32x4{w0[0], w0[1], w1[0], w1[1]};
@@ -602,7 +628,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 Mma32<T>::run(s1, fr[s & 3], qf[s]);
                 fr[s & 3] = s + 4 < DSTEPS ? k_frag(1, s + 4) : v_frag8(0, s + 4 - DSTEPS);
                 uint32_t pk;
-                psum += exp_pair(s0[2 * s], s0[2 * s + 1], m_use, pk);
+                exp_pair(s0[2 * s], s0[2 * s + 1], m_use, pk, psum);
                 asm volatile("" : "+v"(pk), "+v"(psum));       // keeps the exponentials here, between the MFMAs
                 p0f[s >> 2][s & 3] = pk;
                 __builtin_amdgcn_sched_barrier(0);
@@ -616,7 +642,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 Mma32<T>::run(oacc[s & 3], fr[s & 3], p0f[s >> 2]);
                 fr[s & 3] = s + 4 < 8 ? v_frag8(0, s + 4) : v_frag8(1, s + 4 - 8);
                 uint32_t pk;
-                psum1 += exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk);
+                exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk, psum1);
                 asm volatile("" : "+v"(pk), "+v"(psum1));
                 p1f[s >> 2][s & 3] = pk;
                 __builtin_amdgcn_sched_barrier(0);
@@ -632,7 +658,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 #pragma unroll
                 for (int s = 0; s < 8; s++) {
                     uint32_t pk;
-                    psum1 += exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk);
+                    exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk, psum1);
                     p1f[s >> 2][s & 3] = pk;
                 }
             }
@@ -647,6 +673,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         }
         __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA of tile j+1 has landed ...
         __syncthreads();                    // ... everyone's has, and everyone is done with tile j
+    };
+    for (int j = 0; j < ntiles; j += 2) {
+        tile_body(j, std::integral_constant<int, 0>{});
+        if (j + 1 < ntiles) tile_body(j + 1, std::integral_constant<int, 1>{});
     }
 
     const float l_tot = sum_with_partner32(l_run);
