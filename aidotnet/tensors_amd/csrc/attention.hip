@@ -572,7 +572,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
     auto tile_body = [&](const int j, auto stage_c) {
         constexpr int stage = decltype(stage_c)::value;
-        if (j + 1 < ntiles) { issue_k(j + 1); issue_v(j + 1); }
+        // Loads of the next tile: when this wave computes and the next tile lies fully inside the sequence they are
+        // issued one per MFMA inside the first phase below (a vector-memory instruction holds the wave's issue slot for
+        // some tens of cycles; there it is covered by the running MFMA).  Otherwise all at once here.
+        const bool spread = j < nact && j + 1 < ntiles && (j + 1) * BC + BC <= a.Sk;
+        if (j + 1 < ntiles && !spread) { issue_k(j + 1); issue_v(j + 1); }
         if (j < nact) {
             const int kv0 = j * BC;
             const bool need_mask = kv0 + BC - 1 > wave_klim;
@@ -610,11 +614,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             u32x4 fr[4];
 #pragma unroll
             for (int s = 0; s < 4; s++) fr[s] = k_frag(0, s);
+            if (spread) {
+                const unsigned char* ksrc = (const unsigned char*)K + (long long)((j + 1) * BC + 16 * wave_s) * k_row_bytes;
+                const unsigned char* vsrc = (const unsigned char*)V + (long long)((j + 1) * BC + 16 * wave_s) * v_row_bytes;
+                const uint32_t kdst = lds0 + (stage ^ 1) * KBYTES + wave_s * 4096;
+                const uint32_t vdst = lds0 + 2 * KBYTES + (stage ^ 1) * VBYTES + wave_s * 4096;
 #pragma unroll
-            for (int s = 0; s < DSTEPS; s++) {
-                Mma32<T>::run(s0, fr[s & 3], qf[s]);
-                fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int s = 0; s < DSTEPS; s++) {
+                    Mma32<T>::run(s0, fr[s & 3], qf[s]);
+                    fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
+                    if (s < 4) attn_dma16_base(ksrc + 4 * s * k_row_bytes, k_lane_off[s], kdst + s * 1024);
+                    else attn_dma16_base(vsrc + 4 * (s - 4) * v_row_bytes, v_lane_off, vdst + (s - 4) * 1024);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+#pragma unroll
+                for (int s = 0; s < DSTEPS; s++) {
+                    Mma32<T>::run(s0, fr[s & 3], qf[s]);
+                    fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
             if (need_mask) mask_sub(0, s0);
             lazy_rescale(sub_max(s0));
