@@ -53,6 +53,9 @@ SIGNATURES = {
     "aidn_mi355_sync": (_i, [_vp, _vp]),
     "aidn_mi355_sgemm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _f, _i]),
     "aidn_mi355_sgemm_batched": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _f]),
+    "aidn_mi355_sgemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f]),
+    "aidn_mi355_hgemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f]),
+    "aidn_mi355_bf16gemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f]),
     "aidn_mi355_hgemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_hgemm_f16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),

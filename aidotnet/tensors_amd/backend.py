@@ -223,6 +223,78 @@ class Mi355Backend:
                                                        M, N, K, batchCount, alpha, beta))
         self._done()
 
+    # ------------------------------------------------------------------ fused projection epilogues
+    # FusedActivationType numbering (src/AiDotNet.Tensors/Engines/FusedActivationType.cs:23-70)
+    ACT_NONE, ACT_RELU, ACT_GELU, ACT_SIGMOID, ACT_TANH, ACT_LEAKY_RELU, ACT_SWISH = range(7)
+
+    def GemmBiasActivationInto(self, A: GpuBuffer, B: GpuBuffer, bias: Optional[GpuBuffer], C: GpuBuffer,
+                               M: int, N: int, K: int, activation: int = 0, alpha: float = 0.0) -> None:
+        """C = act(A * B + bias) in one kernel, fp32 (the work of GemmBias + an activation kernel,
+        HipBackend.cs:1637-1785, without the intermediate buffers)."""
+        op = "GemmBiasActivation"
+        self._need(A, "A"); self._need(B, "B"); self._need(C, "C")
+        self._positive(M=M, N=N, K=K)
+        self._capacity(A, M * K * 4, "A", op); self._capacity(B, K * N * 4, "B", op); self._capacity(C, M * N * 4, "C", op)
+        if bias is not None:
+            self._capacity(bias, N * 4, "bias", op)
+        self._check(self._lib.aidn_mi355_sgemm_bias_act(self._ctx, self._stream(), A.Handle, B.Handle,
+                                                        bias.Handle if bias is not None else None, C.Handle,
+                                                        M, N, K, int(activation), float(alpha)))
+        self._done()
+
+    def _gemm_bias(self, A, B, bias, M, N, K, activation, alpha=0.0) -> GpuBuffer:
+        self._need(bias, "bias")
+        self._positive(M=M, N=N, K=K)
+        C = self.AllocateBuffer(M * N)
+        self.GemmBiasActivationInto(A, B, bias, C, M, N, K, activation, alpha)
+        return C
+
+    def GemmBias(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        """output = A * B + bias, bias broadcast across the M rows (IDirectGpuBackend.cs:254-265)."""
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_NONE)
+
+    def GemmBiasRelu(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        """ReLU(A * B + bias) (IDirectGpuBackend.cs:227-237)."""
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_RELU)
+
+    def GemmBiasGelu(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        """GELU(A * B + bias), tanh form (IDirectGpuBackend.cs:239-242; HipActivationKernels.cs:44-54)."""
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_GELU)
+
+    def GemmBiasSigmoid(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_SIGMOID)
+
+    def GemmBiasTanh(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_TANH)
+
+    def GemmBiasSwish(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int) -> GpuBuffer:
+        """x * sigmoid(x) of A * B + bias (IDirectGpuBackend.cs:267-270)."""
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_SWISH)
+
+    def GemmBiasLeakyRelu(self, A: GpuBuffer, B: GpuBuffer, bias: GpuBuffer, M: int, N: int, K: int,
+                          alpha: float = 0.01) -> GpuBuffer:
+        """LeakyReLU(A * B + bias, alpha) (IDirectGpuBackend.cs:272-275)."""
+        return self._gemm_bias(A, B, bias, M, N, K, self.ACT_LEAKY_RELU, alpha)
+
+    def GemmBiasActivationHalf(self, kind: str, a: GpuBuffer, b: GpuBuffer, bias: Optional[GpuBuffer], c: GpuBuffer,
+                               m: int, n: int, k: int, activation: int = 0, alpha: float = 0.0,
+                               outputIsFp32: bool = False) -> None:
+        """16-bit A and B ("f16" / "bf16"), fp32 bias, fp32 accumulation and epilogue, output fp32 or the input
+        type.  No member of this name exists in the reference interface (its fused epilogues are fp32 only)."""
+        fn = {"f16": self._lib.aidn_mi355_hgemm_bias_act, "bf16": self._lib.aidn_mi355_bf16gemm_bias_act}.get(kind)
+        if fn is None:
+            raise NotSupportedException("GemmBiasActivationHalf: kind must be 'f16' or 'bf16'")
+        op = "GemmBiasActivationHalf"
+        self._need(a, "a"); self._need(b, "b"); self._need(c, "c")
+        self._positive(m=m, n=n, k=k)
+        self._capacity(a, m * k * 2, "a", op); self._capacity(b, k * n * 2, "b", op)
+        self._capacity(c, m * n * (4 if outputIsFp32 else 2), "c", op)
+        if bias is not None:
+            self._capacity(bias, n * 4, "bias", op)
+        self._check(fn(self._ctx, self._stream(), a.Handle, b.Handle, bias.Handle if bias is not None else None, c.Handle,
+                       1 if outputIsFp32 else 0, m, n, k, int(activation), float(alpha)))
+        self._done()
+
     # ------------------------------------------------------------------ GEMM (16-bit)
     SupportsHgemm = True
     SupportsBf16Gemm = True   # no member of this name exists in the reference interface

@@ -127,7 +127,10 @@ int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, co
     return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, c->ws), "attn_decode");
 }
 
-int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32, int M, int N, int K)
+bool valid_activation(int act) { return act >= 0 && act <= 6; }
+
+int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32, int M, int N, int K,
+                  const float* bias = nullptr, int act = 0, float act_param = 0.0f)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
@@ -140,7 +143,8 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
         if (st) return st;
         ws = c->ws;
     }
-    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws), "gemm_16");
+    if (!valid_activation(act)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: unknown activation");
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, bias, act, act_param), "gemm_16");
 }
 
 int convert_common(void* ctx, void* stream, int kind, const void* in, void* out, int64_t n)
@@ -240,6 +244,25 @@ AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, c
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, 0, batch,
                                         (long long)M * K, (long long)K * N, (long long)M * N, tile), "gemm_f32 (batched)");
 }
+
+AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, const float* B, const float* bias, float* C,
+                              int M, int N, int K, int activation, float act_param)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: A, B and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: dimensions must be positive");
+    if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: unknown activation");
+    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param),
+                      "gemm_f32 (bias + activation)");
+}
+AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
+                              int out_is_f32, int M, int N, int K, int activation, float act_param)
+{ return gemm16_common(ctx, stream, 0, A, B, C, out_is_f32 != 0, M, N, K, bias, activation, act_param); }
+AIDN_API int aidn_mi355_bf16gemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
+                                 int out_is_f32, int M, int N, int K, int activation, float act_param)
+{ return gemm16_common(ctx, stream, 1, A, B, C, out_is_f32 != 0, M, N, K, bias, activation, act_param); }
 
 AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K)
 { return gemm16_common(ctx, stream, 0, A, B, C, 1, M, N, K); }

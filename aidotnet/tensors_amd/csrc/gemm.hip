@@ -26,7 +26,27 @@ struct GemmArgs {
     long long sA, sB, sC;   // batch strides in elements
     float alpha, beta;
     int tiles_m, tiles_n;
+    // fused epilogue: C = act(alpha * A B + beta * C + bias[col]); bias may be null, act 0 = none
+    const float* bias;
+    int act;
+    float act_param;
 };
+
+// Pointwise activations of the fused projection epilogues, numbered like the reference's FusedActivationType
+// (src/AiDotNet.Tensors/Engines/FusedActivationType.cs:23-70) and computed like its HIP activation kernels
+// (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/Kernels/HipActivationKernels.cs:19-70).
+__device__ __forceinline__ float apply_activation(float x, int act, float p)
+{
+    switch (act) {
+    case 1: return x < 0.0f ? 0.0f : x;                                                      // ReLU, NaN-preserving form (CpuFusedOperations.cs:1271-1274)
+    case 2: return 0.5f * x * (1.0f + tanhf(0.7978845608f * (x + 0.044715f * x * x * x)));   // GELU, tanh form
+    case 3: return 1.0f / (1.0f + expf(-x));                                                 // sigmoid
+    case 4: return tanhf(x);
+    case 5: return x > 0.0f ? x : p * x;                                                     // leaky ReLU, slope p
+    case 6: return x / (1.0f + expf(-x));                                                    // swish
+    default: return x;
+    }
+}
 
 constexpr int ROWB = 144;    // LDS row pitch in bytes
 constexpr int GROUP_M = 8;   // tile rows walked together so one XCD's L2 sees a compact footprint
@@ -253,6 +273,7 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
+            const float bias = (g.bias && (!CHECK || col < g.N)) ? g.bias[col] : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
@@ -261,9 +282,11 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
                     float v = g.alpha * acc[i][j][r];
                     if constexpr (Elem<OutT>::BYTES == 4) {
                         if (use_beta) v += g.beta * as_f32(*p);
+                        v = apply_activation(v + bias, g.act, g.act_param);
                         *p = as_u32(v);
                     } else {
                         if (use_beta) v += g.beta * Elem<OutT>::widen(*p);
+                        v = apply_activation(v + bias, g.act, g.act_param);
                         *p = (out_t)Elem<OutT>::narrow(v);
                     }
                 }
@@ -416,12 +439,14 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
+            const float bias = g.bias ? g.bias[col] : 0.0f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
                 out_t* p = C + (long long)row * g.ldc + col;
-                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(acc[i][j][r]);
-                else *p = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
+                const float v = apply_activation(acc[i][j][r] + bias, g.act, g.act_param);
+                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(v);
+                else *p = (out_t)Elem<OutT>::narrow(v);
             }
         }
 }
@@ -537,7 +562,8 @@ __global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, f
 }
 
 template <typename OutT>
-__global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv, int M, int N, int ksplit)
+__global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv, int M, int N, int ksplit,
+                                                             const float* __restrict__ bias, int act, float act_param)
 {
     typedef typename Raw<OutT>::type out_t;
     out_t* C = (out_t*)Cv;
@@ -545,6 +571,8 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
         float s = 0.0f;
         for (int k = 0; k < ksplit; k++) s += ws[(long long)k * total + i];
+        if (bias) s += bias[i % N];
+        s = apply_activation(s, act, act_param);
         if constexpr (Elem<OutT>::BYTES == 4) C[i] = as_u32(s);
         else C[i] = (out_t)Elem<OutT>::narrow(s);
     }
@@ -578,7 +606,7 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
     if (e != hipSuccess) return e;
     long long total = (long long)g.M * g.N;
     unsigned grid = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks);
+    hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks, g.bias, g.act, g.act_param);
     return hipGetLastError();
 }
 
@@ -640,18 +668,18 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
 
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile)
+                    int force_tile, const float* bias, int act, float act_param)
 {
-    GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0};
+    GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
     if (transB) return dispatch_gemm<float, float, true>(g, batch, stream, force_tile);
     return dispatch_gemm<float, float, false>(g, batch, stream, force_tile);
 }
 
 // kind: 0 = fp16, 1 = bf16; out32: C is fp32 (else the same 16-bit type as the inputs)
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace)
+                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
 {
-    GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0};
+    GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
     if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         float* ws = (float*)workspace;
         if (kind == 0) return out32 ? launch_skinny<f16_t, float>(g, stream, ws) : launch_skinny<f16_t, f16_t>(g, stream, ws);

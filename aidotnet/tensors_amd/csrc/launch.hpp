@@ -5,13 +5,16 @@
 
 namespace aidn {
 
+// bias (nullable, N floats added to every row) and act (0 none, 1 ReLU, 2 GELU-tanh, 3 sigmoid, 4 tanh, 5 leaky ReLU with slope
+// act_param, 6 swish) form the fused epilogue C = act(alpha A B + beta C + bias)
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile);
+                    int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f);
 // workspace: gemm_16_workspace_bytes(M, N, K) bytes (0 = none needed); without it the skinny-M path is not taken
 size_t gemm_16_workspace_bytes(int M, int N, int K);
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace);
+                   int M, int N, int K, int force_tile, void* workspace, const float* bias = nullptr, int act = 0,
+                   float act_param = 0.0f);
 
 // kind: 0 f32->f16, 1 f16->f32, 2 f32->bf16, 3 bf16->f32
 hipError_t convert(hipStream_t stream, int kind, const void* in, void* out, long long n);

@@ -56,6 +56,42 @@ class Mi355Engine:
             raise ArgumentException("batched TensorMatMul needs equal leading dimensions")
         return self.BatchMatMul(a, b)
 
+    _ACTIVATIONS = {"None": 0, "ReLU": 1, "GELU": 2, "Sigmoid": 3, "Tanh": 4, "LeakyReLU": 5, "Swish": 6}
+
+    def FusedLinear(self, input: torch.Tensor, weights: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                    activation="None", alpha: float = 0.01, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        """activation(input @ weights + bias): input [..., K] (leading dims collapse), weights [K, N], bias [N] or
+        None (IEngine.cs:5166; CpuEngine FusedLinear: GEMM, then the bias + activation epilogue of
+        Helpers/CpuFusedOperations.cs:590-700).  activation is a FusedActivationType name or number 0..6; alpha is
+        the LeakyReLU slope.  fp16 / bf16 inputs take an fp32 bias and accumulate in fp32."""
+        if input is None or weights is None:
+            raise ArgumentNullException("input" if input is None else "weights")
+        if weights.dim() != 2 or input.dim() < 2:
+            raise ArgumentException("FusedLinear needs input of rank >= 2 and weights of rank 2")
+        if input.dtype != weights.dtype or input.dtype not in _KIND:
+            raise NotSupportedException("FusedLinear: unsupported dtype combination %s x %s" % (input.dtype, weights.dtype))
+        K, N = weights.shape
+        if input.shape[-1] != K:
+            raise ArgumentException("Weight matrix shape mismatch: expected [%d, N], got %s" % (input.shape[-1], tuple(weights.shape)))
+        act = self._ACTIVATIONS.get(activation, activation) if isinstance(activation, str) else int(activation)
+        if not isinstance(act, int) or not 0 <= act <= 6:
+            raise NotSupportedException("FusedLinear: activation %r has no fused epilogue" % (activation,))
+        if bias is not None and (bias.dim() != 1 or bias.shape[0] != N):
+            raise ArgumentException("bias must have N = %d elements" % N)
+        be = self.backend
+        a = input.contiguous(); w = weights.contiguous()
+        M = a.numel() // K
+        bb = be.WrapTensor(bias.to(torch.float32).contiguous()) if bias is not None else None
+        if a.dtype == torch.float32:
+            out = torch.empty(*a.shape[:-1], N, dtype=torch.float32, device=a.device)
+            be.GemmBiasActivationInto(be.WrapTensor(a), be.WrapTensor(w), bb, be.WrapTensor(out), M, N, K, act, alpha)
+            return out
+        out_dtype = out_dtype or a.dtype
+        out = torch.empty(*a.shape[:-1], N, dtype=out_dtype, device=a.device)
+        be.GemmBiasActivationHalf(_KIND[a.dtype], be.WrapTensor(a), be.WrapTensor(w), bb, be.WrapTensor(out), M, N, K, act, alpha,
+                                  outputIsFp32=out_dtype == torch.float32)
+        return out
+
     def BatchMatMul(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """[..., M, K] x [..., K, N], fp32 (DirectGpuTensorEngine.cs:19987-20019 -> BatchedGemm)."""
         if a.dtype != torch.float32 or b.dtype != torch.float32:

@@ -68,6 +68,23 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
 AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, const float* B, float* C,
                              int M, int N, int K, int batch, float alpha, float beta);
 
+/* ---- fused projection epilogues ---------------------------------------------------------------
+ * C[M,N] = act(A[M,K] * B[K,N] + bias[N]), bias broadcast over rows (may be null), in one kernel.
+ * activation: 0 none, 1 ReLU, 2 GELU (tanh form), 3 sigmoid, 4 tanh, 5 leaky ReLU with slope act_param,
+ * 6 swish -- the numbering of FusedActivationType (Engines/FusedActivationType.cs:23-70).  Replaces
+ * IDirectGpuBackend.GemmBias / GemmBiasRelu / GemmBiasGelu / GemmBiasSigmoid / GemmBiasTanh /
+ * GemmBiasSwish / GemmBiasLeakyRelu (IDirectGpuBackend.cs:227-275; host HipBackend.cs:1637-1785, which
+ * runs the GEMM, a bias kernel and an activation kernel one after the other) and is what
+ * IEngine.FusedLinear needs (Engines/IEngine.cs:5166; CPU epilogue Helpers/CpuFusedOperations.cs:590-700).
+ * The 16-bit forms take fp16 / bf16 A and B, an fp32 bias, accumulate and apply the epilogue in fp32 and
+ * store fp32 (out_is_f32 != 0) or one rounding to the input type. */
+AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, const float* B, const float* bias, float* C,
+                              int M, int N, int K, int activation, float act_param);
+AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
+                              int out_is_f32, int M, int N, int K, int activation, float act_param);
+AIDN_API int aidn_mi355_bf16gemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
+                                 int out_is_f32, int M, int N, int K, int activation, float act_param);
+
 /* ---- 16-bit GEMM, fp32 accumulation ------------------------------------------------------------
  * C[M,N] = A[M,K] * B[K,N].  *_f32out replaces IGpuHalfPrecisionBackend.GemmFp16In32fOut
  * (Engines/Gpu/IGpuHalfPrecisionBackend.cs:39-48; host HipBackend.HalfPrecision.cs:125-150,

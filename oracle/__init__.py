@@ -129,6 +129,16 @@ def gemm_alpha_beta(a, b, c, m, n, k, alpha=1.0, beta=0.0, trans_b=False, thread
     return c
 
 
+def bias_activation(c, bias, act: int = 0, param: float = 0.0) -> np.ndarray:
+    """The FusedLinear epilogue act(c + bias) on a [M, N] fp32 matrix (bias [N] or None); returns a new array."""
+    out = np.array(c, np.float32, copy=True, order="C")
+    m, n = out.shape
+    b = _c(bias, np.float32) if bias is not None else None
+    lib().orc_bias_act_f32(_p(out, _f32p), _p(b, _f32p) if b is not None else None, ctypes.c_long(m), ctypes.c_long(n),
+                           int(act), ctypes.c_float(param))
+    return out
+
+
 def gemm_f64(a, b, m, k, n, trans_b=False, threads: int = 0) -> np.ndarray:
     a = _c(a, np.float32); b = _c(b, np.float32)
     c = np.empty((m, n), np.float64)

@@ -319,6 +319,35 @@ void orc_bf16gemm(const uint16_t* a, int lda, const uint16_t* b, int ldb,
         }
 }
 
+/* Bias + activation epilogue of FusedLinear: the scalar loop of CpuFusedOperations.ApplyBiasActivationInPlace
+ * (src/AiDotNet.Tensors/Helpers/CpuFusedOperations.cs:676-690) with the pointwise functions of its table
+ * (:1268-1280; ApplyGelu :1452-1460).  act uses the FusedActivationType numbers (Engines/FusedActivationType.cs:23-70):
+ * 0 none, 1 ReLU (NaN-preserving form x < 0 ? 0 : x), 2 GELU tanh form, 3 sigmoid, 4 tanh, 5 leaky ReLU with
+ * slope p, 6 swish.  The reference's SIMD variants of None/ReLU/GELU compute the same functions; last-ulp
+ * agreement with MathF.Exp / MathF.Tanh is unpinned (libm here). */
+static float orc_activation(float x, int act, float p)
+{
+    switch (act) {
+    case 1: return x < 0.0f ? 0.0f : x;
+    case 2: { float x3 = x * x * x; float inner = 0.7978845608028654f * (x + 0.044715f * x3); return 0.5f * x * (1.0f + tanhf(inner)); }
+    case 3: return 1.0f / (1.0f + expf(-x));
+    case 4: return tanhf(x);
+    case 5: return x > 0.0f ? x : p * x;
+    case 6: return x / (1.0f + expf(-x));
+    default: return x;
+    }
+}
+
+void orc_bias_act_f32(float* c, const float* bias, long m, long n, int act, float p)
+{
+    for (long i = 0; i < m; i++)
+        for (long j = 0; j < n; j++) {
+            float v = c[i * n + j];
+            if (bias) v += bias[j];
+            c[i * n + j] = orc_activation(v, act, p);
+        }
+}
+
 int orc_max_threads(void)
 {
 #ifdef _OPENMP
