@@ -56,6 +56,9 @@ SIGNATURES = {
     "aidn_mi355_sgemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f]),
     "aidn_mi355_hgemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f]),
     "aidn_mi355_bf16gemm_bias_act": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f]),
+    "aidn_mi355_mha_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_mha_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_mha_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aidn_mi355_hgemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_hgemm_f16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),

@@ -295,6 +295,44 @@ class Mi355Backend:
                        1 if outputIsFp32 else 0, m, n, k, int(activation), float(alpha)))
         self._done()
 
+    # ------------------------------------------------------------------ multi-head attention forward
+    def MultiHeadAttentionForward(self, kind: str, input: GpuBuffer, qWeight: GpuBuffer, kWeight: GpuBuffer, vWeight: GpuBuffer,
+                                  outWeight: GpuBuffer, mask: Optional[GpuBuffer], output: GpuBuffer,
+                                  batch: int, seqLen: int, dModel: int, numHeads: int) -> None:
+        """output[B,S,dModel] = MHA(input) with [dModel,dModel] weights and no biases, as three launches over a packed
+        QKV activation (CpuEngine.MultiHeadAttention.cs:155-285 restated for the device; the reference has no GPU route).
+        kind "f32" / "f16" / "bf16"; mask: fp32 keep-mask of seqLen*seqLen (shared) or batch*numHeads*seqLen*seqLen elements."""
+        fn = {"f32": self._lib.aidn_mi355_mha_fwd_f32, "f16": self._lib.aidn_mi355_mha_fwd_f16,
+              "bf16": self._lib.aidn_mi355_mha_fwd_bf16}.get(kind)
+        if fn is None:
+            raise NotSupportedException("MultiHeadAttentionForward: kind must be 'f32', 'f16' or 'bf16'")
+        op = "MultiHeadAttentionForward"
+        for b, n in ((input, "input"), (qWeight, "qWeight"), (kWeight, "kWeight"), (vWeight, "vWeight"), (outWeight, "outWeight"),
+                     (output, "output")):
+            self._need(b, n)
+        self._positive(batch=batch, seqLen=seqLen, dModel=dModel, numHeads=numHeads)
+        if dModel % numHeads != 0:
+            raise ArgumentException("dModel (%d) must be divisible by numHeads (%d)." % (dModel, numHeads))
+        if dModel // numHeads > 256:
+            raise ArgumentException("head dimension %d exceeds 256" % (dModel // numHeads))          # GpuKernelGuards.cs:12
+        es = 4 if kind == "f32" else 2
+        self._capacity(input, batch * seqLen * dModel * es, "input", op)
+        self._capacity(output, batch * seqLen * dModel * es, "output", op)
+        for b, n in ((qWeight, "qWeight"), (kWeight, "kWeight"), (vWeight, "vWeight"), (outWeight, "outWeight")):
+            self._capacity(b, dModel * dModel * es, n, op)
+        mode = 0
+        if mask is not None:
+            plane = seqLen * seqLen
+            if mask.SizeInBytes == plane * 4:
+                mode = 1
+            elif mask.SizeInBytes == batch * numHeads * plane * 4:
+                mode = 2
+            else:
+                raise ArgumentException("mask must hold seqLen*seqLen or batch*numHeads*seqLen*seqLen floats")
+        self._check(fn(self._ctx, self._stream(), input.Handle, qWeight.Handle, kWeight.Handle, vWeight.Handle, outWeight.Handle,
+                       mask.Handle if mask is not None else None, mode, output.Handle, batch, seqLen, dModel, numHeads))
+        self._done()
+
     # ------------------------------------------------------------------ GEMM (16-bit)
     SupportsHgemm = True
     SupportsBf16Gemm = True   # no member of this name exists in the reference interface

@@ -7,6 +7,7 @@
 #include "launch.hpp"
 
 #include <mutex>
+#include <math.h>
 #include <string>
 #include <cstdio>
 #include <cstring>
@@ -145,6 +146,63 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
     }
     if (!valid_activation(act)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: unknown activation");
     return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, bias, act, act_param), "gemm_16");
+}
+
+// Multi-head attention forward as three launches and no permutes: fused [Wq|Wk|Wv] projection into a packed
+// [B*S, 3*dModel] activation, attention reading it through strides and writing [B, S, H, d], output projection.
+// kind: 0 fp32, 1 fp16, 2 bf16 (16-bit: every intermediate stays in the input type, accumulation in fp32).
+int mha_common(void* ctx, void* stream, int kind, const void* input, const void* wq, const void* wk, const void* wv, const void* wo,
+               const float* mask, int mask_mode, void* output, int B, int S, int dModel, int heads)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!input || !wq || !wk || !wv || !wo || !output)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: input, weights and output must not be null");
+    if (B <= 0 || S <= 0 || dModel <= 0 || heads <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: dimensions must be positive");
+    if (dModel % heads != 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: dModel must be divisible by the number of heads");
+    const int dHead = dModel / heads;
+    if (dHead > 256) return fail(c, AIDN_ERR_UNSUPPORTED, "mha: head dimension above 256");
+    if (mask_mode < 0 || mask_mode > 2) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: mask_mode must be 0, 1 or 2");
+    if (mask_mode != 0 && !mask) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: mask_mode set but mask is null");
+    const long long rows = (long long)B * S;
+    if (rows > 0x7FFFFFFFLL || 3LL * dModel > 0x7FFFFFFFLL) return fail(c, AIDN_ERR_UNSUPPORTED, "mha: B*S or 3*dModel exceeds 2^31");
+    const size_t es = kind == 0 ? 4 : 2;
+    auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    const size_t wf_bytes = up((size_t)dModel * 3 * dModel * es), qkv_bytes = up((size_t)rows * 3 * dModel * es);
+    const size_t cc_bytes = up((size_t)rows * dModel * es);
+    int st = ensure_ws(c, wf_bytes + qkv_bytes + cc_bytes);
+    if (st) return st;
+    unsigned char* wf = (unsigned char*)c->ws;
+    unsigned char* qkv = wf + wf_bytes;
+    unsigned char* cc = qkv + qkv_bytes;
+    hipStream_t sm = (hipStream_t)stream;
+    const void* w3[3] = {wq, wk, wv};
+    for (int j = 0; j < 3; j++) {
+        hipError_t e = hipMemcpy2DAsync(wf + (size_t)j * dModel * es, (size_t)3 * dModel * es, w3[j], (size_t)dModel * es,
+                                        (size_t)dModel * es, (size_t)dModel, hipMemcpyDeviceToDevice, sm);
+        if (e != hipSuccess) return hip_status(c, e, "mha: weight gather");
+    }
+    const int M = (int)rows, N3 = 3 * dModel;
+    const int tile32 = c->force_tile == 256 ? 0 : c->force_tile;
+    hipError_t e;
+    if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)wf, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
+    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)wf, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
+    if (e != hipSuccess) return hip_status(c, e, "mha: QKV projection");
+
+    aidn::AttnParams p{};
+    p.q = qkv; p.k = qkv + (size_t)dModel * es; p.v = qkv + (size_t)2 * dModel * es; p.o = cc;
+    p.lse = nullptr; p.bias = nullptr; p.mask = mask_mode ? mask : nullptr; p.weights = nullptr;
+    p.B = B; p.H = heads; p.Hkv = heads; p.Sq = S; p.Sk = S; p.D = dHead;
+    p.scale = 1.0f / sqrtf((float)dHead); p.causal = 0; p.qoff = 0; p.softcap = 0.0f; p.mask_mode = mask_mode; p.out16 = kind != 0;
+    p.bias_bs = 0;
+    for (int i = 0; i < 3; i++) { long long v = i == 0 ? (long long)S * N3 : (i == 1 ? dHead : N3); p.qs[i] = v; p.ks[i] = v; p.vs[i] = v; }
+    p.os[0] = (long long)S * dModel; p.os[1] = dHead; p.os[2] = dModel;
+    e = aidn::attn_fwd(sm, kind, p);
+    if (e != hipSuccess) return hip_status(c, e, "mha: attention");
+
+    if (kind == 0) e = aidn::gemm_f32(sm, (const float*)cc, (const float*)wo, (float*)output, M, dModel, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
+    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)cc, (const uint16_t*)wo, output, 0, M, dModel, dModel, c->force_tile, nullptr);
+    return hip_status(c, e, "mha: output projection");
 }
 
 int convert_common(void* ctx, void* stream, int kind, const void* in, void* out, int64_t n)
@@ -291,6 +349,16 @@ AIDN_API int aidn_mi355_attn_fwd_f16(void* ctx, void* stream, const aidn_attn_de
 AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
                              void* o, float* lse, const float* bias, const float* mask, float* weights)
 { return attn_common(ctx, stream, 2, desc, q, k, v, o, lse, bias, mask, weights); }
+
+AIDN_API int aidn_mi355_mha_fwd_f32(void* ctx, void* stream, const float* input, const float* wq, const float* wk, const float* wv,
+                           const float* wo, const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads)
+{ return mha_common(ctx, stream, 0, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
+AIDN_API int aidn_mi355_mha_fwd_f16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
+                           const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
+{ return mha_common(ctx, stream, 1, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
+AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
+                            const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
+{ return mha_common(ctx, stream, 2, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
 
 AIDN_API int aidn_mi355_attn_decode_f32(void* ctx, void* stream, const aidn_attn_desc* desc, const float* q, const float* k, const float* v,
                                float* o, float* lse, int splits)

@@ -15,7 +15,8 @@ from typing import Optional, Tuple
 
 import torch
 
-from .backend import ArgumentException, ArgumentNullException, Mi355Backend, NotSupportedException
+from .backend import (ArgumentException, ArgumentNullException, ArgumentOutOfRangeException, Mi355Backend,
+                      NotSupportedException)
 
 _KIND = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}
 
@@ -154,6 +155,42 @@ class Mi355Engine:
                 be.FlashAttentionHalf(kind, be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out),
                                       be.WrapTensor(lse), B, H, Sq, Sk, D, scale, isCausal, queryOffset, key.shape[1])
         return out, lse
+
+    def MultiHeadAttentionForward(self, input: torch.Tensor, qWeight: torch.Tensor, kWeight: torch.Tensor, vWeight: torch.Tensor,
+                                  outWeight: torch.Tensor, numHeads: int, mask: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """input [B, seq, dModel], four [dModel, dModel] projections, optional boolean keep-mask broadcastable to
+        [B, H, seq, seq] -> [B, seq, dModel]; inference only (CpuEngine.MultiHeadAttention.cs:68-143 for the argument rules).
+        fp32, fp16 and bf16 tensors are accepted; the output has the input's dtype."""
+        for t, n in ((input, "input"), (qWeight, "qWeight"), (kWeight, "kWeight"), (vWeight, "vWeight"), (outWeight, "outWeight")):
+            if t is None:
+                raise ArgumentNullException(n)
+        if input.dim() != 3:
+            raise ArgumentException("MultiHeadAttentionForward expects rank-3 input [B, seq, dModel]; got rank %d." % input.dim())
+        if numHeads <= 0:
+            raise ArgumentOutOfRangeException("numHeads must be positive.")
+        B, S, dM = input.shape
+        if dM % numHeads != 0:
+            raise ArgumentException("dModel (%d) must be divisible by numHeads (%d)." % (dM, numHeads))
+        for w, n in ((qWeight, "qWeight"), (kWeight, "kWeight"), (vWeight, "vWeight"), (outWeight, "outWeight")):
+            if w.dim() != 2 or w.shape[0] != dM or w.shape[1] != dM:
+                raise ArgumentException("%s must be [%d, %d]." % (n, dM, dM))
+            if w.dtype != input.dtype:
+                raise NotSupportedException("MultiHeadAttentionForward: %s dtype differs from the input's" % n)
+        if input.dtype not in _KIND:
+            raise NotSupportedException("MultiHeadAttentionForward: unsupported dtype %s" % input.dtype)
+        be = self.backend
+        m = None
+        if mask is not None:
+            if mask.dim() != 4:
+                raise ArgumentException("mask must be rank 4, broadcastable to [B,H,seq,seq]")
+            shared = mask.shape[0] == 1 and mask.shape[1] == 1
+            full = mask.expand(1 if shared else B, 1 if shared else numHeads, S, S)
+            m = be.WrapTensor(full.to(torch.float32).contiguous().reshape(-1))
+        out = torch.empty(B, S, dM, dtype=input.dtype, device=input.device)
+        W = be.WrapTensor
+        be.MultiHeadAttentionForward(_KIND[input.dtype], W(input.contiguous()), W(qWeight.contiguous()), W(kWeight.contiguous()),
+                                     W(vWeight.contiguous()), W(outWeight.contiguous()), m, W(out), B, S, dM, numHeads)
+        return out
 
     def ScaledDotProductAttention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                                   mask: Optional[torch.Tensor] = None, scale: Optional[float] = None,

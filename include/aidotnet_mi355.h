@@ -184,6 +184,21 @@ AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn
 AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc,
                                 const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
 
+/* ---- multi-head attention forward --------------------------------------------------------------------
+ * output[B,S,dModel] = (softmax(Q K^T / sqrt(d)) V) Wo with [Q|K|V] = input[B,S,dModel] [Wq|Wk|Wv], heads = dModel / d, all
+ * weights [dModel,dModel] row-major, no biases: IEngine.MultiHeadAttentionForward (Engines/CpuEngine.MultiHeadAttention.cs:68-143;
+ * fp32 path :155-285, fused SDPA over the packed activation :358-522), which has no GPU route in the reference.
+ * Three launches and no permutes: one GEMM writes the packed [B*S, 3 dModel] activation, the attention kernel reads it through
+ * strides and writes [B,S,H,d], one GEMM projects.  mask (may be null): fp32, non-zero = keep; mask_mode 1 = one [S,S] plane
+ * shared by all (b,h), 2 = full [B,H,S,S] (what a broadcast of the reference's Tensor<bool> mask materialises to).
+ * The 16-bit forms keep every intermediate in the input type and accumulate in fp32.  Intermediates live in the context's workspace. */
+AIDN_API int aidn_mi355_mha_fwd_f32(void* ctx, void* stream, const float* input, const float* wq, const float* wk, const float* wv,
+                           const float* wo, const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads);
+AIDN_API int aidn_mi355_mha_fwd_f16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
+                           const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
+AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
+                            const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
+
 /* ---- test / tuning hook --------------------------------------------------------------------------------
  * Forces the GEMM tile edge (64, 128 or 256; 0 = automatic choice) for subsequent calls on this
  * context, so the parity suite can exercise every kernel instance.  No counterpart in the reference. */

@@ -224,6 +224,25 @@ def attention_f64(q, k, v, scale, causal=False, query_offset=0, bias=None, keep=
     return out, lse
 
 
+def mha_forward(x, wq, wk, wv, wo, heads: int, keep=None) -> np.ndarray:
+    """``MultiHeadAttentionForwardFloat`` (src/AiDotNet.Tensors/Engines/CpuEngine.MultiHeadAttention.cs:155-285): fused
+    ``[Wq|Wk|Wv]`` SimdGemm on ``[B*S, dModel]``, per-(b, h) attention with scale 1/sqrt(dHead) and an optional boolean
+    keep-mask broadcastable to ``[B,H,S,S]``, heads concatenated back to ``[B*S, dModel]``, output SimdGemm.
+    Composed from the restated GEMM and attention above, as the reference composes ``SimdGemm.Sgemm`` and its SDPA."""
+    x = _c(x, np.float32)
+    B, S, dM = x.shape
+    d = dM // heads
+    wf = np.concatenate([_c(wq, np.float32), _c(wk, np.float32), _c(wv, np.float32)], axis=1)
+    qkv = sgemm(x.reshape(B * S, dM), wf, B * S, dM, 3 * dM, threads=max_threads()).reshape(B, S, 3, heads, d)
+    q = np.ascontiguousarray(qkv[:, :, 0].transpose(0, 2, 1, 3)); k = np.ascontiguousarray(qkv[:, :, 1].transpose(0, 2, 1, 3))
+    v = np.ascontiguousarray(qkv[:, :, 2].transpose(0, 2, 1, 3))
+    if keep is not None:
+        keep = np.broadcast_to(np.asarray(keep, bool), (B, heads, S, S))
+    o, _, _ = attention_f32(q, k, v, 1.0 / float(np.sqrt(d)), keep=keep)
+    cc = np.ascontiguousarray(o.transpose(0, 2, 1, 3)).reshape(B * S, dM)
+    return sgemm(cc, _c(wo, np.float32), B * S, dM, dM, threads=max_threads()).reshape(B, S, dM)
+
+
 def decode_f32(q, k, v, heads, kv_heads, head_dim, seq_len, scale) -> np.ndarray:
     """The reference decode test's oracle: q [heads, d], k/v [seqLen, kvHeads, d] -> [heads, d]."""
     q = _c(q, np.float32); k = _c(k, np.float32); v = _c(v, np.float32)
