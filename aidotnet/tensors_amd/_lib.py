@@ -59,6 +59,15 @@ SIGNATURES = {
     "aidn_mi355_mha_fwd_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aidn_mi355_mha_fwd_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aidn_mi355_mha_fwd_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_paged_attn_decode_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
+    "aidn_mi355_paged_attn_prefill_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
+    "aidn_mi355_paged_attn_decode_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
+    "aidn_mi355_paged_attn_prefill_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
+    "aidn_mi355_paged_attn_decode_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
+    "aidn_mi355_paged_attn_prefill_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
+    "aidn_mi355_rope_interleaved_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
+    "aidn_mi355_rope_interleaved_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
+    "aidn_mi355_rope_interleaved_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
     "aidn_mi355_hgemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_hgemm_f16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),

@@ -295,6 +295,115 @@ class Mi355Backend:
                        1 if outputIsFp32 else 0, m, n, k, int(activation), float(alpha)))
         self._done()
 
+    # ------------------------------------------------------------------ rotary position embedding
+    def RopeInterleaved(self, input: GpuBuffer, cos: GpuBuffer, sin: GpuBuffer, output: GpuBuffer,
+                        rows: int, headDim: int, seqLen: int, startPosition: int, kind: str = "f32") -> None:
+        """Rotates every adjacent pair (2i, 2i+1) of a [rows, headDim] view by the angle of position
+        startPosition + row % seqLen; caches [maxSeq, headDim/2] fp32; output may alias input
+        (IDirectGpuBackend.cs:1427-1446; HipBackend.cs:6177-6210).  kind "f16" / "bf16" is an addition."""
+        fn = {"f32": self._lib.aidn_mi355_rope_interleaved_f32, "f16": self._lib.aidn_mi355_rope_interleaved_f16,
+              "bf16": self._lib.aidn_mi355_rope_interleaved_bf16}.get(kind)
+        if fn is None:
+            raise NotSupportedException("RopeInterleaved: kind must be 'f32', 'f16' or 'bf16'")
+        if rows <= 0 or headDim <= 0 or seqLen <= 0:
+            raise ArgumentOutOfRangeException("RoPE dimensions must be positive.")
+        if headDim & 1:
+            raise ArgumentException("RoPE requires an even head dimension.")
+        if startPosition < 0:
+            raise ArgumentOutOfRangeException("startPosition")
+        for b, n in ((input, "input"), (cos, "cos"), (sin, "sin"), (output, "output")):
+            self._need(b, n)
+        es = 4 if kind == "f32" else 2
+        if input.SizeInBytes < rows * headDim * es or output.SizeInBytes < rows * headDim * es:
+            raise ArgumentException("RoPE input/output buffers are smaller than rows * headDim.")
+        need = (startPosition + min(seqLen, rows)) * (headDim // 2) * 4
+        if cos.SizeInBytes < need or sin.SizeInBytes < need:
+            raise ArgumentException("RoPE cos/sin caches are shorter than startPosition + seqLen positions.")
+        self._check(fn(self._ctx, self._stream(), input.Handle, cos.Handle, sin.Handle, output.Handle, rows, headDim, seqLen,
+                       startPosition))
+        self._done()
+
+    # ------------------------------------------------------------------ paged K/V cache attention
+    def _paged(self, op, kind, q, kcache, vcache, blockTable, heads, kvHeads, headDim, blockSize, numQueries, keyLen, startPos,
+               scale, splits, decode) -> GpuBuffer:
+        # GpuKernelGuards.Attention / Gqa / PagedAttentionBuffers (GpuKernelGuards.cs:14-30, 87-108)
+        if heads <= 0:
+            raise ArgumentOutOfRangeException("%s: heads must be > 0 (got %d)." % (op, heads))
+        if headDim <= 0 or headDim > 256:
+            raise ArgumentOutOfRangeException("%s: headDim must be in [1, 256] (got %d)." % (op, headDim))
+        if blockSize <= 0:
+            raise ArgumentOutOfRangeException("%s: blockSize must be > 0 (got %d)." % (op, blockSize))
+        if numQueries <= 0 or keyLen <= 0:
+            raise ArgumentOutOfRangeException("%s: sequence/query count must be > 0." % op)
+        if kvHeads <= 0 or kvHeads > heads or heads % kvHeads != 0:
+            raise ArgumentOutOfRangeException("%s: kvHeads must satisfy 1 <= kvHeads <= heads and heads %% kvHeads == 0." % op)
+        if startPos < 0:
+            raise ArgumentOutOfRangeException("startPos")
+        for b, n in ((q, "q"), (kcache, "kcache"), (vcache, "vcache"), (blockTable, "blockTable")):
+            self._need(b, n)
+        es = 4 if kind == "f32" else 2
+        self._capacity(q, numQueries * heads * headDim * es, "q", op)
+        blocks = (keyLen + blockSize - 1) // blockSize
+        self._capacity(blockTable, blocks * 4, "blockTable", op)
+        per_block = blockSize * kvHeads * headDim * es
+        if kcache.SizeInBytes <= 0 or kcache.SizeInBytes != vcache.SizeInBytes:
+            raise ArgumentException("%s: kcache/vcache must be equal-sized, non-empty K/V pools." % op)
+        if kcache.SizeInBytes % per_block != 0:
+            raise ArgumentException("%s: K/V pool size is not a whole number of blocks." % op)
+        bt = blockTable.tensor.reshape(-1)[:blocks]
+        if bt.dtype != torch.int32:
+            raise ArgumentException("%s: blockTable must hold 32-bit block ids." % op)
+        if int(bt.min()) < 0 or int(bt.max()) >= kcache.SizeInBytes // per_block:
+            raise ArgumentException("%s: blockTable names a block outside the pool." % op)
+        out = self.AllocateBuffer(numQueries * heads * headDim)
+        if decode:
+            fn = getattr(self._lib, "aidn_mi355_paged_attn_decode_" + kind)
+            self._check(fn(self._ctx, self._stream(), q.Handle, kcache.Handle, vcache.Handle, blockTable.Handle, out.Handle,
+                           heads, kvHeads, headDim, blockSize, keyLen, float(scale), int(splits)))
+        else:
+            fn = getattr(self._lib, "aidn_mi355_paged_attn_prefill_" + kind)
+            self._check(fn(self._ctx, self._stream(), q.Handle, kcache.Handle, vcache.Handle, blockTable.Handle, out.Handle,
+                           heads, kvHeads, headDim, blockSize, numQueries, startPos, float(scale)))
+        self._done()
+        return out
+
+    def PagedAttentionDecode(self, q: GpuBuffer, kcache: GpuBuffer, vcache: GpuBuffer, blockTable: GpuBuffer,
+                             heads: int, headDim: int, blockSize: int, seqLen: int, scale: float) -> GpuBuffer:
+        """out[heads*headDim] = softmax(scale q K) V over a paged cache [numBlocks, blockSize, heads, headDim] gathered through
+        blockTable (IDirectGpuBackend.cs:3614-3618; HipBackend.cs:831-852)."""
+        return self._paged("PagedAttentionDecode", "f32", q, kcache, vcache, blockTable, heads, heads, headDim, blockSize, 1, seqLen, 0,
+                           scale, 0, True)
+
+    def PagedAttentionDecodeGqa(self, q: GpuBuffer, kcache: GpuBuffer, vcache: GpuBuffer, blockTable: GpuBuffer,
+                                heads: int, kvHeads: int, headDim: int, blockSize: int, seqLen: int, scale: float) -> GpuBuffer:
+        """Query head h reads KV head h / (heads / kvHeads) (IDirectGpuBackend.cs:3625-3627)."""
+        return self._paged("PagedAttentionDecodeGqa", "f32", q, kcache, vcache, blockTable, heads, kvHeads, headDim, blockSize, 1, seqLen,
+                           0, scale, 0, True)
+
+    def PagedAttentionPrefill(self, q: GpuBuffer, kcache: GpuBuffer, vcache: GpuBuffer, blockTable: GpuBuffer,
+                              heads: int, headDim: int, blockSize: int, numQueries: int, startPos: int, scale: float) -> GpuBuffer:
+        """Causal multi-query form: query i attends to keys 0 .. startPos + i; out [numQueries, heads, headDim]
+        (IDirectGpuBackend.cs:3620-3623; HipBackend.cs:854-876)."""
+        return self._paged("PagedAttentionPrefill", "f32", q, kcache, vcache, blockTable, heads, heads, headDim, blockSize, numQueries,
+                           startPos + numQueries, startPos, scale, 0, False)
+
+    def PagedAttentionPrefillGqa(self, q: GpuBuffer, kcache: GpuBuffer, vcache: GpuBuffer, blockTable: GpuBuffer,
+                                 heads: int, kvHeads: int, headDim: int, blockSize: int, numQueries: int, startPos: int,
+                                 scale: float) -> GpuBuffer:
+        return self._paged("PagedAttentionPrefillGqa", "f32", q, kcache, vcache, blockTable, heads, kvHeads, headDim, blockSize,
+                           numQueries, startPos + numQueries, startPos, scale, 0, False)
+
+    def PagedAttentionHalf(self, kind: str, q: GpuBuffer, kcache: GpuBuffer, vcache: GpuBuffer, blockTable: GpuBuffer,
+                           heads: int, kvHeads: int, headDim: int, blockSize: int, numQueries: int, startPos: int, scale: float,
+                           splits: int = 0) -> GpuBuffer:
+        """fp16 / bf16 pools and queries, fp32 output; numQueries == 1 and startPos = seqLen - 1 is decode.  No member of this
+        name exists in the reference interface (its paged attention is fp32 only)."""
+        if kind not in ("f16", "bf16"):
+            raise NotSupportedException("PagedAttentionHalf: kind must be 'f16' or 'bf16'")
+        decode = numQueries == 1
+        return self._paged("PagedAttentionHalf", kind, q, kcache, vcache, blockTable, heads, kvHeads, headDim, blockSize, numQueries,
+                           startPos + numQueries, 0 if decode else startPos, scale, splits, decode)
+
     # ------------------------------------------------------------------ multi-head attention forward
     def MultiHeadAttentionForward(self, kind: str, input: GpuBuffer, qWeight: GpuBuffer, kWeight: GpuBuffer, vWeight: GpuBuffer,
                                   outWeight: GpuBuffer, mask: Optional[GpuBuffer], output: GpuBuffer,

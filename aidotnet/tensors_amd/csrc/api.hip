@@ -205,6 +205,55 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
     return hip_status(c, e, "mha: output projection");
 }
 
+// Attention over a paged K/V cache: pools [numBlocks, blockSize, kvHeads, headDim], logical key j in pool row
+// blockTable[j / blockSize] * blockSize + j % blockSize.  numQueries == 1: decode kernel; otherwise causal prefill
+// (query i at logical position startPos + i sees keys 0 .. startPos + i).
+int paged_common(void* ctx, void* stream, int kind, const void* q, const void* kcache, const void* vcache, const int32_t* block_table,
+                 void* o, int heads, int kv_heads, int head_dim, int block_size, int num_queries, int key_len, int start_pos,
+                 float scale, int splits, bool decode)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!q || !kcache || !vcache || !block_table || !o)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "paged attention: q, pools, block table and o must not be null");
+    if (heads <= 0 || head_dim <= 0 || block_size <= 0 || num_queries <= 0 || key_len <= 0)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "paged attention: heads, headDim, blockSize and lengths must be positive");
+    if (head_dim > 256) return fail(c, AIDN_ERR_UNSUPPORTED, "paged attention: head dimension above 256");
+    if (kv_heads <= 0) kv_heads = heads;
+    if (kv_heads > heads || heads % kv_heads != 0)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "paged attention: heads must be an integer multiple of kvHeads");
+    if (start_pos < 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "paged attention: startPos must not be negative");
+    aidn::AttnParams p{};
+    p.q = q; p.k = kcache; p.v = vcache; p.o = o;
+    p.B = 1; p.H = heads; p.Hkv = kv_heads; p.Sq = num_queries; p.Sk = key_len; p.D = head_dim;
+    p.scale = scale; p.causal = decode ? 0 : 1; p.qoff = start_pos; p.softcap = 0.0f; p.mask_mode = 0; p.out16 = 0; p.bias_bs = 0;
+    // q and o are [numQueries, heads, headDim]; pool rows are [kvHeads, headDim] wide
+    p.qs[0] = 0; p.qs[1] = head_dim; p.qs[2] = (long long)heads * head_dim;
+    p.os[0] = 0; p.os[1] = head_dim; p.os[2] = (long long)heads * head_dim;
+    p.ks[0] = 0; p.ks[1] = head_dim; p.ks[2] = (long long)kv_heads * head_dim;
+    p.vs[0] = 0; p.vs[1] = head_dim; p.vs[2] = (long long)kv_heads * head_dim;
+    p.block_table = block_table; p.block_size = block_size; p.block_table_stride = 0;
+    if (decode) {
+        int eff = aidn::attn_decode_splits(p, splits);
+        size_t need = aidn::attn_decode_workspace_bytes(p, eff);
+        if (need) { int st = ensure_ws(c, need); if (st) return st; }
+        return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, c->ws), "paged attn_decode");
+    }
+    return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "paged attn_fwd");
+}
+
+int rope_common(void* ctx, void* stream, int kind, const void* in, const float* cosc, const float* sinc, void* out,
+                int64_t rows, int head_dim, int seq_len, int start_position)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!in || !cosc || !sinc || !out) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "rope: buffers must not be null");
+    if (rows <= 0 || head_dim <= 0 || seq_len <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "rope: dimensions must be positive");
+    if (head_dim & 1) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "rope: head dimension must be even");
+    if (start_position < 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "rope: start position must not be negative");
+    return hip_status(c, aidn::rope_interleaved((hipStream_t)stream, kind, in, cosc, sinc, out, rows, head_dim, seq_len, start_position), "rope");
+}
+
 int convert_common(void* ctx, void* stream, int kind, const void* in, void* out, int64_t n)
 {
     Ctx* c = (Ctx*)ctx;
@@ -349,6 +398,56 @@ AIDN_API int aidn_mi355_attn_fwd_f16(void* ctx, void* stream, const aidn_attn_de
 AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
                              void* o, float* lse, const float* bias, const float* mask, float* weights)
 { return attn_common(ctx, stream, 2, desc, q, k, v, o, lse, bias, mask, weights); }
+
+AIDN_API int aidn_mi355_paged_attn_decode_f32(void* ctx, void* stream, const float* q, const float* kcache, const float* vcache,
+                                     const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                     int seq_len, float scale, int splits)
+{ return paged_common(ctx, stream, 0, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, 1, seq_len, 0, scale, splits, true); }
+AIDN_API int aidn_mi355_paged_attn_decode_f16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                     const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                     int seq_len, float scale, int splits)
+{ return paged_common(ctx, stream, 1, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, 1, seq_len, 0, scale, splits, true); }
+AIDN_API int aidn_mi355_paged_attn_decode_bf16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int seq_len, float scale, int splits)
+{ return paged_common(ctx, stream, 2, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, 1, seq_len, 0, scale, splits, true); }
+AIDN_API int aidn_mi355_paged_attn_prefill_f32(void* ctx, void* stream, const float* q, const float* kcache, const float* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int num_queries, int start_pos, float scale)
+{
+    long long key_len = (long long)start_pos + num_queries;
+    if (key_len > 0x7FFFFFFFLL) return AIDN_ERR_INVALID_ARGUMENT;
+    return paged_common(ctx, stream, 0, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, num_queries, (int)key_len,
+                        start_pos, scale, 0, false);
+}
+AIDN_API int aidn_mi355_paged_attn_prefill_f16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int num_queries, int start_pos, float scale)
+{
+    long long key_len = (long long)start_pos + num_queries;
+    if (key_len > 0x7FFFFFFFLL) return AIDN_ERR_INVALID_ARGUMENT;
+    return paged_common(ctx, stream, 1, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, num_queries, (int)key_len,
+                        start_pos, scale, 0, false);
+}
+AIDN_API int aidn_mi355_paged_attn_prefill_bf16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                       const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                       int num_queries, int start_pos, float scale)
+{
+    long long key_len = (long long)start_pos + num_queries;
+    if (key_len > 0x7FFFFFFFLL) return AIDN_ERR_INVALID_ARGUMENT;
+    return paged_common(ctx, stream, 2, q, kcache, vcache, block_table, o, heads, kv_heads, head_dim, block_size, num_queries, (int)key_len,
+                        start_pos, scale, 0, false);
+}
+
+AIDN_API int aidn_mi355_rope_interleaved_f32(void* ctx, void* stream, const float* input, const float* cos_cache, const float* sin_cache,
+                                    float* output, int64_t rows, int head_dim, int seq_len, int start_position)
+{ return rope_common(ctx, stream, 0, input, cos_cache, sin_cache, output, rows, head_dim, seq_len, start_position); }
+AIDN_API int aidn_mi355_rope_interleaved_f16(void* ctx, void* stream, const uint16_t* input, const float* cos_cache, const float* sin_cache,
+                                    uint16_t* output, int64_t rows, int head_dim, int seq_len, int start_position)
+{ return rope_common(ctx, stream, 1, input, cos_cache, sin_cache, output, rows, head_dim, seq_len, start_position); }
+AIDN_API int aidn_mi355_rope_interleaved_bf16(void* ctx, void* stream, const uint16_t* input, const float* cos_cache, const float* sin_cache,
+                                     uint16_t* output, int64_t rows, int head_dim, int seq_len, int start_position)
+{ return rope_common(ctx, stream, 2, input, cos_cache, sin_cache, output, rows, head_dim, seq_len, start_position); }
 
 AIDN_API int aidn_mi355_mha_fwd_f32(void* ctx, void* stream, const float* input, const float* wq, const float* wk, const float* wv,
                            const float* wo, const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads)

@@ -34,6 +34,7 @@ struct AttnArgs {
     int qtiles;
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
+    const int* bt; int bsz; long long bt_bs;   // block table of a paged K/V cache (null = contiguous), block size, batch stride
 };
 
 template <typename T> struct Raw2;
@@ -108,6 +109,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
     const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+    const int* __restrict__ bt = a.bt ? a.bt + b * a.bt_bs : nullptr;
 
     // ---- Q fragments (B operand of S^T): row qi, 16-byte chunk (2 s + h)
     u32x4 qf[DSTEPS];
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             int row = u / CPR, ch = u - row * CPR;
             int key = kv0 + row, d0 = ch * E;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if ((NKC % NT == 0 || u < NKC) && key < a.Sk) v = ld16<T>(K + (long long)key * a.ks[2] + d0, a.D - d0, vec);
+            if ((NKC % NT == 0 || u < NKC) && key < a.Sk) v = ld16<T>(K + paged_row(bt, a.bsz, key) * a.ks[2] + d0, a.D - d0, vec);
             rk[i] = v;
         }
 #pragma unroll
@@ -147,7 +149,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             for (int r = 0; r < 4; r++) {
                 int key = kv0 + kb * 4 + r;
                 u32x4 v = {0u, 0u, 0u, 0u};
-                if ((NVU % NT == 0 || u < NVU) && key < a.Sk) v = ld16<T>(V + (long long)key * a.vs[2] + d0, a.D - d0, vec);
+                if ((NVU % NT == 0 || u < NVU) && key < a.Sk) v = ld16<T>(V + paged_row(bt, a.bsz, key) * a.vs[2] + d0, a.D - d0, vec);
                 rv[i * 4 + r] = v;
             }
         }
@@ -828,6 +830,8 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     a.bias_bs = p.bias_bs;
     for (int i = 0; i < 3; i++) { a.qs[i] = p.qs[i]; a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; a.os[i] = p.os[i]; }
     a.qtiles = 0;
+    a.bt = p.block_table; a.bsz = p.block_size; a.bt_bs = p.block_table_stride;
+    if (p.block_table && p.weights) return hipErrorInvalidValue;      // the weights output does not follow a block table
     const int eb = kind == 0 ? 4 : 2, e = 16 / eb;
     const int oeb = (kind == 0 || !p.out16) ? 4 : 2;
     auto al = [](const void* ptr, const long long* s, int bytes) {
@@ -840,7 +844,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     // fast path: 16-bit, head dim 128, aligned rows, plain (optionally causal) attention
     // the fast kernel addresses K/V rows of a 4-key load group with unsigned 32-bit byte offsets
     const bool rows32 = p.ks[2] > 0 && p.ks[2] < (1LL << 28) && p.vs[2] > 0 && p.vs[2] < (1LL << 28);
-    const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && rows32 && g_attn_allow_dl;
+    const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && rows32 && !p.block_table && g_attn_allow_dl;
     if (dl) {
         if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
         else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);

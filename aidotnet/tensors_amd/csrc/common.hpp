@@ -132,6 +132,14 @@ __device__ __forceinline__ void transpose4x4_b32(const u32x4 (&in)[4], u32x4 (&o
         for (int w = 0; w < 4; w++) out[c][w] = in[w][c];
 }
 
+// Pool row of logical key `key` under a block table (vLLM-style paged K/V cache; null table = identity).
+__device__ __forceinline__ long long paged_row(const int* __restrict__ bt, int bsz, int key)
+{
+    if (!bt) return key;
+    const int blk = key / bsz;
+    return (long long)bt[blk] * bsz + (key - blk * bsz);
+}
+
 // ---------------------------------------------------------------- wave helpers
 __device__ __forceinline__ float shfl_xor_f(float v, int mask) { return __shfl_xor(v, mask, WAVE); }
 

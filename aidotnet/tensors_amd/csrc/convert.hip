@@ -68,4 +68,49 @@ hipError_t convert(hipStream_t stream, int kind, const void* in, void* out, long
     return hipGetLastError();
 }
 
+// Interleaved rotary position embedding (GPT-NeoX / LLaMA / GGML form): the pair (2i, 2i+1) of row r is rotated by the
+// angle of absolute position startPosition + r % seqLen; cos / sin caches are fp32 [maxSeq, headDim / 2].
+// Replaces rope_interleaved (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/Kernels/HipAttentionKernels.cs:958-989, one thread
+// per pair).  HBM-bound; one thread per pair with 8-byte (fp32) or 4-byte (16-bit) accesses, output may alias input.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_interleaved_kernel(const void* __restrict__ in, const float* __restrict__ cosc,
+                                                               const float* __restrict__ sinc, void* out,
+                                                               long long rows, int headDim, int seqLen, int startPosition)
+{
+    const int half = headDim >> 1;
+    const long long total = rows * half;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+        const long long row = g / half;
+        const int i = (int)(g - row * half);
+        const long long pos = startPosition + row % seqLen;
+        const float c = cosc[pos * half + i], sn = sinc[pos * half + i];
+        float xe, xo;
+        if constexpr (Elem<T>::BYTES == 4) {
+            u32x2 v = ((const u32x2*)in)[g];
+            xe = as_f32(v[0]); xo = as_f32(v[1]);
+        } else {
+            uint32_t v = ((const uint32_t*)in)[g];
+            xe = Elem<T>::widen(v & 0xFFFFu); xo = Elem<T>::widen(v >> 16);
+        }
+        const float re = xe * c - xo * sn, ro = xe * sn + xo * c;
+        if constexpr (Elem<T>::BYTES == 4) ((u32x2*)out)[g] = u32x2{as_u32(re), as_u32(ro)};
+        else ((uint32_t*)out)[g] = Elem<T>::narrow(re) | (Elem<T>::narrow(ro) << 16);
+    }
+}
+
+// kind: 0 fp32, 1 fp16, 2 bf16
+hipError_t rope_interleaved(hipStream_t stream, int kind, const void* in, const float* cosc, const float* sinc, void* out,
+                            long long rows, int headDim, int seqLen, int startPosition)
+{
+    long long pairs = rows * (headDim / 2);
+    if (pairs <= 0) return hipSuccess;
+    unsigned grid = (unsigned)((pairs + 255) / 256 > 256 * 32 ? 256 * 32 : (pairs + 255) / 256);
+    if (kind == 0) hipLaunchKernelGGL(rope_interleaved_kernel<float>, dim3(grid), dim3(256), 0, stream, in, cosc, sinc, out, rows, headDim, seqLen, startPosition);
+    else if (kind == 1) hipLaunchKernelGGL(rope_interleaved_kernel<f16_t>, dim3(grid), dim3(256), 0, stream, in, cosc, sinc, out, rows, headDim, seqLen, startPosition);
+    else if (kind == 2) hipLaunchKernelGGL(rope_interleaved_kernel<bf16_t>, dim3(grid), dim3(256), 0, stream, in, cosc, sinc, out, rows, headDim, seqLen, startPosition);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 }  // namespace aidn

@@ -25,6 +25,7 @@ struct DecodeArgs {
     int splits, chunk;       // keys per split
     long long qs[2], ks[3], vs[3], os[2];   // q/o: batch, head; k/v: batch, head, row
     int vec_in;
+    const int* bt; int bsz; long long bt_bs;   // block table of a paged cache (null = contiguous), block size, batch stride
 };
 
 template <typename T> struct Raw3;
@@ -91,6 +92,7 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
     const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
     const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
+    const int* __restrict__ bt = a.bt ? a.bt + b * a.bt_bs : nullptr;
 
     float qf[E];
     {
@@ -115,8 +117,9 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
         for (int u = 0; u < U; u++) {
             int key = base + u * KPW + sk;
             bool ok = key < kend;
-            kx[u] = ok ? ld16d<T>(K + (long long)key * a.ks[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
-            vx[u] = ok ? ld16d<T>(V + (long long)key * a.vs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+            const long long row = ok ? paged_row(bt, a.bsz, key) : 0;
+            kx[u] = ok ? ld16d<T>(K + row * a.ks[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+            vx[u] = ok ? ld16d<T>(V + row * a.vs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
         }
         float s[U];
         float mloc = -INFINITY;
@@ -295,6 +298,7 @@ hipError_t attn_decode(hipStream_t stream, int kind, const AttnParams& p, int ef
     a.splits = eff_splits;
     a.qs[0] = p.qs[0]; a.qs[1] = p.qs[1]; a.os[0] = p.os[0]; a.os[1] = p.os[1];
     for (int i = 0; i < 3; i++) { a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; }
+    a.bt = p.block_table; a.bsz = p.block_size; a.bt_bs = p.block_table_stride;
     const int eb = kind == 0 ? 4 : 2, e = 16 / eb;
     const int lpk = lanes_per_key(p.D, eb) < 4 ? 4 : lanes_per_key(p.D, eb);
     // keys per split: a multiple of the keys one workgroup iteration covers

@@ -19,6 +19,10 @@ hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16
 // kind: 0 f32->f16, 1 f16->f32, 2 f32->bf16, 3 bf16->f32
 hipError_t convert(hipStream_t stream, int kind, const void* in, void* out, long long n);
 
+// interleaved RoPE; kind: 0 fp32, 1 fp16, 2 bf16 (cos / sin caches fp32)
+hipError_t rope_interleaved(hipStream_t stream, int kind, const void* in, const float* cosc, const float* sinc, void* out,
+                            long long rows, int headDim, int seqLen, int startPosition);
+
 // Attention problem description shared by the prefill and decode launchers (host side).
 struct AttnParams {
     const void* q; const void* k; const void* v; void* o;
@@ -27,6 +31,11 @@ struct AttnParams {
     float scale; int causal; int qoff; float softcap; int mask_mode; int out16;
     long long bias_bs;
     long long qs[3], ks[3], vs[3], os[3];   // batch, head, row strides in elements
+    // paged K/V (null = contiguous rows): logical key j lives in pool row block_table[j / block_size] * block_size + j % block_size;
+    // batch b uses the table at block_table + b * block_table_stride.  The row stride ks[2] / vs[2] is that of the pool.
+    const int* block_table = nullptr;
+    int block_size = 0;
+    long long block_table_stride = 0;
 };
 
 // kind: 0 fp32, 1 fp16, 2 bf16

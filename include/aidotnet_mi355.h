@@ -184,6 +184,45 @@ AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn
 AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc,
                                 const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
 
+/* ---- attention over a paged K/V cache --------------------------------------------------------------------
+ * K and V pools [numBlocks, blockSize, kvHeads, headDim]; block_table[i] = pool block of logical block i (int32, at least
+ * ceil(keyLen / blockSize) entries); q and o [numQueries, heads, headDim]; o is fp32 for every input type.  kv_heads <= 0
+ * means heads.  *_decode: one query over seq_len keys, splits as for aidn_mi355_attn_decode_*.  *_prefill: causal, query i
+ * (logical position start_pos + i) sees keys 0 .. start_pos + i.  Replace IDirectGpuBackend.PagedAttentionDecode[Gqa] /
+ * PagedAttentionPrefill[Gqa] (IDirectGpuBackend.cs:3614-3633; host HipBackend.cs:831-913, one thread per head in
+ * Kernels/HipPagedAttentionKernels.cs:26-58); the reference interface is fp32 only, the 16-bit forms are additions. */
+AIDN_API int aidn_mi355_paged_attn_decode_f32(void* ctx, void* stream, const float* q, const float* kcache, const float* vcache,
+                                     const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                     int seq_len, float scale, int splits);
+AIDN_API int aidn_mi355_paged_attn_decode_f16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                     const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                     int seq_len, float scale, int splits);
+AIDN_API int aidn_mi355_paged_attn_decode_bf16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int seq_len, float scale, int splits);
+AIDN_API int aidn_mi355_paged_attn_prefill_f32(void* ctx, void* stream, const float* q, const float* kcache, const float* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int num_queries, int start_pos, float scale);
+AIDN_API int aidn_mi355_paged_attn_prefill_f16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                      const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                      int num_queries, int start_pos, float scale);
+AIDN_API int aidn_mi355_paged_attn_prefill_bf16(void* ctx, void* stream, const uint16_t* q, const uint16_t* kcache, const uint16_t* vcache,
+                                       const int32_t* block_table, float* o, int heads, int kv_heads, int head_dim, int block_size,
+                                       int num_queries, int start_pos, float scale);
+
+/* ---- rotary position embedding, interleaved pairs -----------------------------------------------------------
+ * output[r, 2i] = x[r, 2i] cos - x[r, 2i+1] sin, output[r, 2i+1] = x[r, 2i] sin + x[r, 2i+1] cos with the angle of absolute
+ * position start_position + r % seq_len; input / output [rows, head_dim] (rows = leading x seq_len), caches fp32
+ * [maxSeq, head_dim / 2] with at least start_position + seq_len rows; output may alias input.  Replaces
+ * IDirectGpuBackend.RopeInterleaved (IDirectGpuBackend.cs:1427-1446; host HipBackend.cs:6177-6210, kernel
+ * Kernels/HipAttentionKernels.cs:958-989).  The 16-bit forms rotate in fp32 and round once. */
+AIDN_API int aidn_mi355_rope_interleaved_f32(void* ctx, void* stream, const float* input, const float* cos_cache, const float* sin_cache,
+                                    float* output, int64_t rows, int head_dim, int seq_len, int start_position);
+AIDN_API int aidn_mi355_rope_interleaved_f16(void* ctx, void* stream, const uint16_t* input, const float* cos_cache, const float* sin_cache,
+                                    uint16_t* output, int64_t rows, int head_dim, int seq_len, int start_position);
+AIDN_API int aidn_mi355_rope_interleaved_bf16(void* ctx, void* stream, const uint16_t* input, const float* cos_cache, const float* sin_cache,
+                                     uint16_t* output, int64_t rows, int head_dim, int seq_len, int start_position);
+
 /* ---- multi-head attention forward --------------------------------------------------------------------
  * output[B,S,dModel] = (softmax(Q K^T / sqrt(d)) V) Wo with [Q|K|V] = input[B,S,dModel] [Wq|Wk|Wv], heads = dModel / d, all
  * weights [dModel,dModel] row-major, no biases: IEngine.MultiHeadAttentionForward (Engines/CpuEngine.MultiHeadAttention.cs:68-143;

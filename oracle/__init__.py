@@ -224,6 +224,40 @@ def attention_f64(q, k, v, scale, causal=False, query_offset=0, bias=None, keep=
     return out, lse
 
 
+def paged_attention(q, kcache, vcache, block_table, heads: int, kv_heads: int, head_dim: int, block_size: int,
+                    num_queries: int, start_pos: int, scale: float) -> np.ndarray:
+    """The reference's paged-attention kernels (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/Kernels/HipPagedAttentionKernels.cs:
+    decode :26-58, causal prefill :61-105, GQA head map h / (heads / kvHeads)): pools ``[numBlocks, blockSize, kvHeads, d]``,
+    logical key t in pool row ``blockTable[t / blockSize] * blockSize + t % blockSize``, query i sees keys 0 .. startPos + i
+    (decode = one query with startPos = seqLen - 1).  q ``[numQueries, heads, d]`` -> ``[numQueries, heads, d]`` fp32.
+    Restated as gather + the attention above (the kernels' per-key online softmax is the same function)."""
+    q = _c(q, np.float32).reshape(num_queries, heads, head_dim)
+    kc = _c(kcache, np.float32).reshape(-1, block_size, kv_heads, head_dim)
+    vc = _c(vcache, np.float32).reshape(-1, block_size, kv_heads, head_dim)
+    key_len = start_pos + num_queries
+    t = np.arange(key_len)
+    rows = np.asarray(block_table, np.int64)[t // block_size]
+    k = kc[rows, t % block_size]                  # [keyLen, kvHeads, d]
+    v = vc[rows, t % block_size]
+    o, _, _ = attention_f32(q.transpose(1, 0, 2)[None], k.transpose(1, 0, 2)[None], v.transpose(1, 0, 2)[None], scale,
+                            causal=True, query_offset=start_pos)
+    return np.ascontiguousarray(o[0].transpose(1, 0, 2))
+
+
+def rope_interleaved(x, cos, sin, seq_len: int, start_position: int) -> np.ndarray:
+    """``rope_interleaved`` (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/Kernels/HipAttentionKernels.cs:958-989) in fp32:
+    x ``[rows, headDim]``, caches ``[maxSeq, headDim/2]``; pair (2i, 2i+1) of row r rotated by position start + r % seqLen."""
+    x = _c(x, np.float32); cos = _c(cos, np.float32); sin = _c(sin, np.float32)
+    rows, hd = x.shape
+    pos = start_position + np.arange(rows) % seq_len
+    c = cos.reshape(-1, hd // 2)[pos]; s = sin.reshape(-1, hd // 2)[pos]
+    xe = x[:, 0::2]; xo = x[:, 1::2]
+    out = np.empty_like(x)
+    out[:, 0::2] = (xe * c).astype(np.float32) - (xo * s).astype(np.float32)
+    out[:, 1::2] = (xe * s).astype(np.float32) + (xo * c).astype(np.float32)
+    return out
+
+
 def mha_forward(x, wq, wk, wv, wo, heads: int, keep=None) -> np.ndarray:
     """``MultiHeadAttentionForwardFloat`` (src/AiDotNet.Tensors/Engines/CpuEngine.MultiHeadAttention.cs:155-285): fused
     ``[Wq|Wk|Wv]`` SimdGemm on ``[B*S, dModel]``, per-(b, h) attention with scale 1/sqrt(dHead) and an optional boolean
