@@ -16,6 +16,7 @@
 //   tile's MFMAs and stored to the other stage after them; one barrier per K-tile.
 #include "common.hpp"
 #include "launch.hpp"
+#include <type_traits>
 
 namespace aidn {
 
@@ -268,31 +269,38 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
     typedef typename Raw<OutT>::type out_t;
     out_t* __restrict__ C = (out_t*)g.C + bz * g.sC;
     const bool use_beta = g.beta != 0.0f;
+    const bool fused = g.bias != nullptr || g.act != 0;
+    auto store_all = [&](auto fused_c) {
+        constexpr bool FUSED = decltype(fused_c)::value;
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+        for (int i = 0; i < TM; i++) {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int col = n0 + wn * WTN + j * 32 + l32;
-            const float bias = (g.bias && (!CHECK || col < g.N)) ? g.bias[col] : 0.0f;
+            for (int j = 0; j < TN; j++) {
+                const int col = n0 + wn * WTN + j * 32 + l32;
+                float bias = 0.0f;
+                if constexpr (FUSED) bias = (g.bias && (!CHECK || col < g.N)) ? g.bias[col] : 0.0f;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
-                if (!CHECK || (row < g.M && col < g.N)) {
-                    out_t* p = C + (long long)row * g.ldc + col;
-                    float v = g.alpha * acc[i][j][r];
-                    if constexpr (Elem<OutT>::BYTES == 4) {
-                        if (use_beta) v += g.beta * as_f32(*p);
-                        v = apply_activation(v + bias, g.act, g.act_param);
-                        *p = as_u32(v);
-                    } else {
-                        if (use_beta) v += g.beta * Elem<OutT>::widen(*p);
-                        v = apply_activation(v + bias, g.act, g.act_param);
-                        *p = (out_t)Elem<OutT>::narrow(v);
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                    if (!CHECK || (row < g.M && col < g.N)) {
+                        out_t* p = C + (long long)row * g.ldc + col;
+                        float v = g.alpha * acc[i][j][r];
+                        if constexpr (Elem<OutT>::BYTES == 4) {
+                            if (use_beta) v += g.beta * as_f32(*p);
+                            if constexpr (FUSED) v = apply_activation(v + bias, g.act, g.act_param);
+                            *p = as_u32(v);
+                        } else {
+                            if (use_beta) v += g.beta * Elem<OutT>::widen(*p);
+                            if constexpr (FUSED) v = apply_activation(v + bias, g.act, g.act_param);
+                            *p = (out_t)Elem<OutT>::narrow(v);
+                        }
                     }
                 }
             }
         }
-    }
+    };
+    if (fused) store_all(std::true_type{});
+    else store_all(std::false_type{});
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -434,19 +442,23 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 
     typedef typename Raw<OutT>::type out_t;
     out_t* __restrict__ C = (out_t*)g.C;
+    const bool fused = g.bias != nullptr || g.act != 0;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
-            const float bias = g.bias ? g.bias[col] : 0.0f;
+            if (fused) {                                  // bias and / or activation folded into the store
+                const float bias = g.bias ? g.bias[col] : 0.0f;
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = apply_activation(acc[i][j][r] + bias, g.act, g.act_param);
+            }
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
                 out_t* p = C + (long long)row * g.ldc + col;
-                const float v = apply_activation(acc[i][j][r] + bias, g.act, g.act_param);
-                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(v);
-                else *p = (out_t)Elem<OutT>::narrow(v);
+                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(acc[i][j][r]);
+                else *p = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
             }
         }
 }
