@@ -420,24 +420,37 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
+    // Software pipeline: the fragments of k-step s+1 are read from LDS before the MFMAs of step s are issued, so the
+    // LDS latency runs under 8 MFMAs; the barrier that publishes tile kt+1 sits before the MFMAs of the last step, and the
+    // first fragments of tile kt+1 are read there too.  sched_barrier pins this order (the scheduler otherwise sinks
+    // the reads next to their use to save registers, which exposes the LDS latency every few MFMAs).
+    u32x4 fa[2][TM], fb[2][TN];
+    read_frags(smem, smem + ABYTES, 0, fa[0], fb[0]);
     for (int kt = 0; kt < KT; kt++) {
         const int stage = kt & 1;
         const unsigned char* as = smem + stage * STAGE;
         const unsigned char* bs = as + ABYTES;
-        // the other stage was last read before the barrier that ended the previous iteration
+        // the other stage was last read before the barrier inside the previous iteration
         if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
-        u32x4 fa[2][TM], fb[2][TN];
-        read_frags(as, bs, 0, fa[0], fb[0]);
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            if (s < 3) read_frags(as, bs, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+            if (s < 3) {
+                read_frags(as, bs, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1]);
+            } else {
+                __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed and its LDS reads of this tile are done ...
+                __syncthreads();                    // ... and so have everyone else's
+                if (kt + 1 < KT) {
+                    const unsigned char* an = smem + (stage ^ 1) * STAGE;
+                    read_frags(an, an + ABYTES, 0, fa[0], fb[0]);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed ...
-        __syncthreads();                    // ... and so has everyone else's
     }
 
     typedef typename Raw<OutT>::type out_t;
