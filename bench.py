@@ -82,7 +82,7 @@ def main() -> int:
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards without "
-              "communication over (batch, head) and over row slabs of C, see DESIGN.md)" % args.gpus, file=sys.stderr)
+              "communication over (batch, head) and over row slabs of C)" % args.gpus, file=sys.stderr)
         return 2
 
     import torch
