@@ -1,0 +1,53 @@
+"""The entry points are launch-only once the context workspace is sized: a decode step (three skinny projections, RoPE,
+decode attention, output projection) is captured into a HIP graph and replayed; every replay must equal the eager result.
+Between replays the program does its own eager work and synchronises, and the inputs change, so stale-node effects show."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def test_decode_step_under_hip_graph_matches_eager():
+    from aidotnet.tensors_amd import Mi355Backend
+    be = Mi355Backend(synchronous=False)
+    W = be.WrapTensor
+    torch.manual_seed(0)
+    B, H, Hkv, D, S, dM = 4, 16, 4, 128, 1024, 2048
+    x = torch.randn(B, dM, device="cuda").to(torch.bfloat16)
+    wq = (0.02 * torch.randn(dM, H * D, device="cuda")).to(torch.bfloat16)
+    wo = (0.02 * torch.randn(H * D, dM, device="cuda")).to(torch.bfloat16)
+    kc = torch.randn(B, Hkv, S, D, device="cuda").to(torch.bfloat16); vc = torch.randn(B, Hkv, S, D, device="cuda").to(torch.bfloat16)
+    half = D // 2
+    ang = torch.arange(S, device="cuda", dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(half, device="cuda") * 2.0 / D))[None, :]
+    cos, sin = torch.cos(ang).contiguous(), torch.sin(ang).contiguous()
+    q = torch.empty(B, H * D, device="cuda", dtype=torch.bfloat16)
+    att = torch.empty(B, H * D, device="cuda", dtype=torch.bfloat16)
+    y = torch.empty(B, dM, device="cuda", dtype=torch.bfloat16)
+
+    def step():
+        be.Bf16Gemm(W(x), W(wq), W(q), B, H * D, dM)                                        # query projection (skinny, split-K)
+        be.RopeInterleaved(W(q), W(cos), W(sin), W(q), B * H, D, 1, S - 1, "bf16")          # rotate at position S-1, in place
+        be.DecodeAttention("bf16", W(q), W(kc), W(vc), W(att), B, H, S, D, 1 / math.sqrt(D), Hkv, 0, True)
+        be.Bf16Gemm(W(att), W(wo), W(y), B, dM, H * D)                                      # output projection
+
+    step(); torch.cuda.synchronize()                      # sizes the context workspace; nothing allocates after this
+    eager = y.clone()
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    for it in range(4):
+        y.fill_(0); att.fill_(0); q.fill_(0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager), "replay %d differs from the eager result" % it
+        # eager work of the program between replays, and new inputs for the next comparison
+        x.copy_(torch.randn(B, dM, device="cuda").to(torch.bfloat16))
+        step(); torch.cuda.synchronize()
+        eager = y.clone()
