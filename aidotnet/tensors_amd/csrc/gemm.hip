@@ -89,13 +89,17 @@ __device__ __forceinline__ u32x4 load16_guarded(const typename Raw<T>::type* p, 
     return v;
 }
 
-template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK>
-__global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
+// KS = 2: two groups of WM x WN waves work on the same output tile, each on half of the k-steps of every K-tile, and the
+// second group's accumulators are added through LDS at the end (for grids too small to give every SIMD two waves).
+template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1>
+__global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs g)
 {
     typedef typename Raw<T>::type raw_t;
     constexpr int E = Elem<T>::PER16;
     constexpr int BK = 8 * E;                  // elements of K per tile (128 bytes)
-    constexpr int NT = WM * WN * 64;
+    constexpr int NT = WM * WN * KS * 64;
+    constexpr int SPG = 4 / KS;                // fragment steps of a K-tile per wave group
+    static_assert(KS == 1 || KS == 2, "KS must be 1 or 2");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int UA = (BM * 8 + NT - 1) / NT;                   // 16-byte chunks of A per thread
@@ -111,7 +115,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
     const int t = threadIdx.x;
     const int lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    const int wm = wave / WN, wn = wave % WN;
+    const int kgrp = wave / (WM * WN), wq = wave - kgrp * (WM * WN);
+    const int wm = wq / WN, wn = wq % WN;
 
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -239,8 +244,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
     for (int kt = 0; kt < KT; kt++) {
         const int stage = kt & 1;
         if (kt + 1 < KT) load_tile((kt + 1) * BK);
-        const unsigned char* as = As + stage * BM * ROWB + (wm * WTM + l32) * ROWB + h * 16;
-        const unsigned char* bs = Bs + stage * BN * ROWB + (wn * WTN + l32) * ROWB + h * 16;
+        const unsigned char* as = As + stage * BM * ROWB + (wm * WTM + l32) * ROWB + h * 16 + kgrp * SPG * 32;
+        const unsigned char* bs = Bs + stage * BN * ROWB + (wn * WTN + l32) * ROWB + h * 16 + kgrp * SPG * 32;
         // fragments are double-buffered in registers: the LDS reads of step s+1 are in flight during the
         // MFMAs of step s
         u32x4 fa[2][TM], fb[2][TN];
@@ -249,8 +254,8 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TN; j++) fb[0][j] = *(const u32x4*)(bs + j * 32 * ROWB);
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            if (s < 3) {
+        for (int s = 0; s < SPG; s++) {
+            if (s < SPG - 1) {
 #pragma unroll
                 for (int i = 0; i < TM; i++) fa[(s + 1) & 1][i] = *(const u32x4*)(as + i * 32 * ROWB + (s + 1) * 32);
 #pragma unroll
@@ -263,6 +268,27 @@ __global__ __launch_bounds__(WM * WN * 64) void gemm_kernel(const GemmArgs g)
         }
         if (kt + 1 < KT) store_tile(stage ^ 1);
         __syncthreads();
+    }
+
+    if constexpr (KS == 2) {
+        // second wave group hands its partial sums over through LDS (the tile stages are free after the last barrier)
+        float* xs = (float*)smem;
+        if (kgrp == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) xs[((wq * TM + i) * TN + j) * 1024 + r * 64 + lane] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kgrp == 1) return;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += xs[((wq * TM + i) * TN + j) * 1024 + r * 64 + lane];
     }
 
     // ---- epilogue: lane holds column l32 of each 32x32 tile, 16 rows
@@ -636,11 +662,12 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
 }
 
 // ------------------------------------------------------------------ host side
-template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK>
+template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1>
 static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK>;
-    constexpr int smem = 2 * (BM + BN) * ROWB;
+    auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK, KS>;
+    constexpr int tiles_smem = 2 * (BM + BN) * ROWB, merge_smem = KS == 2 ? BM * BN * 4 : 0;
+    constexpr int smem = tiles_smem > merge_smem ? tiles_smem : merge_smem;
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -650,7 +677,7 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch);
-    hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), smem, stream, g);
+    hipLaunchKernelGGL(kern, grid, dim3(WM * WN * KS * 64), smem, stream, g);
     return hipGetLastError();
 }
 
@@ -685,6 +712,8 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, false, true>(g, batch, stream);
     }
     if (tile == 64) {
+        // at most about one 64 x 64 tile per CU: split every K-tile between two wave groups so each SIMD still holds two waves
+        if (vec && tiles(64, 64) <= 320 && g.K >= 4 * 8 * E) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true, 2>(g, batch, stream);
         if (vec) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true>(g, batch, stream);
         return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, false, true>(g, batch, stream);
     }
