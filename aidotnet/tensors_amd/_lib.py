@@ -68,6 +68,7 @@ SIGNATURES = {
     "aidn_mi355_rope_interleaved_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
     "aidn_mi355_rope_interleaved_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
     "aidn_mi355_rope_interleaved_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i, _i, _i]),
+    "aidn_mi355_sgemm_f16weight": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f]),
     "aidn_mi355_hgemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_hgemm_f16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),

@@ -276,6 +276,22 @@ class Mi355Backend:
         """LeakyReLU(A * B + bias, alpha) (IDirectGpuBackend.cs:272-275)."""
         return self._gemm_bias(A, B, bias, M, N, K, self.ACT_LEAKY_RELU, alpha)
 
+    def GemmFp16WeightB(self, A: GpuBuffer, bFp16: GpuBuffer, bias: Optional[GpuBuffer], C: GpuBuffer,
+                        M: int, N: int, K: int, activation: int = 0, alpha: float = 0.0) -> None:
+        """C = act(A * widen(B) + bias) with fp32 A, fp16 weights B [K,N] and fp32 C: the weight-only fp16 GEMM of
+        SimdGemm.SgemmFp16WeightB (Engines/Simd/SimdGemm.Fp16Weight.cs:22-91).  No member of this name exists in the
+        reference's GPU interface."""
+        op = "GemmFp16WeightB"
+        self._need(A, "A"); self._need(bFp16, "bFp16"); self._need(C, "C")
+        self._positive(M=M, N=N, K=K)
+        self._capacity(A, M * K * 4, "A", op); self._capacity(bFp16, K * N * 2, "bFp16", op); self._capacity(C, M * N * 4, "C", op)
+        if bias is not None:
+            self._capacity(bias, N * 4, "bias", op)
+        self._check(self._lib.aidn_mi355_sgemm_f16weight(self._ctx, self._stream(), A.Handle, bFp16.Handle,
+                                                         bias.Handle if bias is not None else None, C.Handle,
+                                                         M, N, K, int(activation), float(alpha)))
+        self._done()
+
     def GemmBiasActivationHalf(self, kind: str, a: GpuBuffer, b: GpuBuffer, bias: Optional[GpuBuffer], c: GpuBuffer,
                                m: int, n: int, k: int, activation: int = 0, alpha: float = 0.0,
                                outputIsFp32: bool = False) -> None:

@@ -364,6 +364,17 @@ AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, 
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param),
                       "gemm_f32 (bias + activation)");
 }
+AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A, const uint16_t* B_f16, const float* bias, float* C,
+                               int M, int N, int K, int activation, float act_param)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B_f16 || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: A, B and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: dimensions must be positive");
+    if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: unknown activation");
+    return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param),
+                      "gemm_f32_f16weight");
+}
 AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
                               int out_is_f32, int M, int N, int K, int activation, float act_param)
 { return gemm16_common(ctx, stream, 0, A, B, C, out_is_f32 != 0, M, N, K, bias, activation, act_param); }

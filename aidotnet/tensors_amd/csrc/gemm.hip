@@ -91,9 +91,12 @@ __device__ __forceinline__ u32x4 load16_guarded(const typename Raw<T>::type* p, 
 
 // KS = 2: two groups of WM x WN waves work on the same output tile, each on half of the k-steps of every K-tile, and the
 // second group's accumulators are added through LDS at the end (for grids too small to give every SIMD two waves).
-template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1>
+// B16 (fp32 kernels only): B holds fp16 weights [K,N]; they are widened to fp32 on the way into LDS, so the product is that
+// of the fp32 A with the exactly widened weights, accumulated in fp32 (weight-only fp16 GEMM).
+template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1, bool B16 = false>
 __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs g)
 {
+    static_assert(!B16 || (Elem<T>::BYTES == 4 && !TRANSB), "fp16 weights: fp32 kernel, B stored [K,N]");
     typedef typename Raw<T>::type raw_t;
     constexpr int E = Elem<T>::PER16;
     constexpr int BK = 8 * E;                  // elements of K per tile (128 bytes)
@@ -175,11 +178,25 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
                     int gk = k0 + kb * E + r;
                     u32x4 v = {0u, 0u, 0u, 0u};
                     if (NBLK % NT == 0 || u < NBLK) {
+                        if constexpr (B16) {
+                            const uint16_t* p = (const uint16_t*)g.B + bz * g.sB + (long long)gk * g.ldb + gn;
+                            if (gk < g.K && gn < g.N) {
+                                if (VEC && gn + 4 <= g.N) {
+                                    u32x2 w = *(const u32x2*)p;
+                                    v = u32x4{as_u32(f16_bits_to_float(w[0] & 0xFFFFu)), as_u32(f16_bits_to_float(w[0] >> 16)),
+                                              as_u32(f16_bits_to_float(w[1] & 0xFFFFu)), as_u32(f16_bits_to_float(w[1] >> 16))};
+                                } else {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) if (gn + e < g.N) v[e] = as_u32(f16_bits_to_float(p[e]));
+                                }
+                            }
+                        } else {
                         const raw_t* p = B + (long long)gk * g.ldb + gn;
                         if constexpr (!CHECK) v = *(const u32x4*)p;
                         else if (gk < g.K && gn < g.N) {
                             if constexpr (VEC) v = *(const u32x4*)p;
                             else v = load16_guarded<T>(p, g.N - gn);
+                        }
                         }
                     }
                     rb[i * E + r] = v;
@@ -662,10 +679,10 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
 }
 
 // ------------------------------------------------------------------ host side
-template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1>
+template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1, bool B16 = false>
 static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK, KS>;
+    auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK, KS, B16>;
     constexpr int tiles_smem = 2 * (BM + BN) * ROWB, merge_smem = KS == 2 ? BM * BN * 4 : 0;
     constexpr int smem = tiles_smem > merge_smem ? tiles_smem : merge_smem;
     static bool attr_set = false;
@@ -727,6 +744,23 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
     if (transB) return dispatch_gemm<float, float, true>(g, batch, stream, force_tile);
     return dispatch_gemm<float, float, false>(g, batch, stream, force_tile);
+}
+
+// fp32 A [M,K] x fp16 weights B [K,N] -> fp32 C, optional fused epilogue
+hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K,
+                              int force_tile, const float* bias, int act, float act_param)
+{
+    GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
+    // rows of A in 16-byte steps, rows of the fp16 B in 8-byte steps
+    const bool vec = aligned16(A) && K % 4 == 0 && (((uintptr_t)B) & 7u) == 0 && N % 4 == 0;
+    auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+    int tile = force_tile == 64 || force_tile == 128 ? force_tile : (tiles(128, 128) >= 192 ? 128 : 64);
+    if (tile == 128) {
+        if (vec) return launch_gemm<float, float, 128, 128, 2, 2, false, true, true, 1, true>(g, 1, stream);
+        return launch_gemm<float, float, 128, 128, 2, 2, false, false, true, 1, true>(g, 1, stream);
+    }
+    if (vec) return launch_gemm<float, float, 64, 64, 2, 2, false, true, true, 1, true>(g, 1, stream);
+    return launch_gemm<float, float, 64, 64, 2, 2, false, false, true, 1, true>(g, 1, stream);
 }
 
 // kind: 0 = fp16, 1 = bf16; out32: C is fp32 (else the same 16-bit type as the inputs)

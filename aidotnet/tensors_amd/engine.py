@@ -93,6 +93,34 @@ class Mi355Engine:
                                   outputIsFp32=out_dtype == torch.float32)
         return out
 
+    def TensorMatMulFp16WeightB(self, a: torch.Tensor, bFp16: torch.Tensor) -> torch.Tensor:
+        """fp32 activations [..., K] x fp16 weights [K, N] -> fp32 [..., N] (CpuEngine.TensorMatMulFp16WeightB ->
+        SimdGemm.SgemmFp16WeightB, Engines/Simd/SimdGemm.Fp16Weight.cs:22-91)."""
+        return self.FusedLinearFp16WeightB(a, bFp16, None, "None")
+
+    def FusedLinearFp16WeightB(self, input: torch.Tensor, weightsFp16: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                               activation="None", alpha: float = 0.01) -> torch.Tensor:
+        """activation(input @ widen(weightsFp16) + bias) in fp32 with fp16-stored weights (CpuEngine.FusedLinearFp16WeightB)."""
+        if input is None or weightsFp16 is None:
+            raise ArgumentNullException("input" if input is None else "weightsFp16")
+        if input.dtype != torch.float32 or weightsFp16.dtype != torch.float16:
+            raise NotSupportedException("Fp16WeightB: fp32 activations and fp16 weights are required")
+        if weightsFp16.dim() != 2 or input.dim() < 1 or input.shape[-1] != weightsFp16.shape[0]:
+            raise ArgumentException("Fp16WeightB: input [..., K] (or [K]) and weights [K, N] are required")
+        act = self._ACTIVATIONS.get(activation, activation) if isinstance(activation, str) else int(activation)
+        if not isinstance(act, int) or not 0 <= act <= 6:
+            raise NotSupportedException("Fp16WeightB: activation %r has no fused epilogue" % (activation,))
+        K, N = weightsFp16.shape
+        if bias is not None and (bias.dim() != 1 or bias.shape[0] != N):
+            raise ArgumentException("bias must have N = %d elements" % N)
+        be = self.backend
+        a = input.contiguous(); w = weightsFp16.contiguous()
+        M = a.numel() // K
+        out = torch.empty(*a.shape[:-1], N, dtype=torch.float32, device=a.device)
+        bb = be.WrapTensor(bias.to(torch.float32).contiguous()) if bias is not None else None
+        be.GemmFp16WeightB(be.WrapTensor(a), be.WrapTensor(w), bb, be.WrapTensor(out), M, N, K, act, alpha)
+        return out
+
     def BatchMatMul(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """[..., M, K] x [..., K, N], fp32 (DirectGpuTensorEngine.cs:19987-20019 -> BatchedGemm)."""
         if a.dtype != torch.float32 or b.dtype != torch.float32:

@@ -85,6 +85,15 @@ AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* 
 AIDN_API int aidn_mi355_bf16gemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
                                  int out_is_f32, int M, int N, int K, int activation, float act_param);
 
+/* ---- weight-only fp16 GEMM ----------------------------------------------------------------------
+ * C[M,N] = act(A[M,K] * widen(B_f16[K,N]) + bias): fp32 activations, fp16 weights widened exactly on the way into LDS (never
+ * materialised in fp32), fp32 products and accumulation, the same optional epilogue as above (bias may be null,
+ * activation 0 = none).  The GPU form of SimdGemm.SgemmFp16WeightB / PackBFromHalf
+ * (Engines/Simd/SimdGemm.Fp16Weight.cs:22-91, 208-261), reached through CpuEngine.TensorMatMulFp16WeightB and
+ * FusedLinearFp16WeightB; the reference has no GPU member for it. */
+AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A, const uint16_t* B_f16, const float* bias, float* C,
+                               int M, int N, int K, int activation, float act_param);
+
 /* ---- 16-bit GEMM, fp32 accumulation ------------------------------------------------------------
  * C[M,N] = A[M,K] * B[K,N].  *_f32out replaces IGpuHalfPrecisionBackend.GemmFp16In32fOut
  * (Engines/Gpu/IGpuHalfPrecisionBackend.cs:39-48; host HipBackend.HalfPrecision.cs:125-150,

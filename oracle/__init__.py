@@ -129,6 +129,13 @@ def gemm_alpha_beta(a, b, c, m, n, k, alpha=1.0, beta=0.0, trans_b=False, thread
     return c
 
 
+def sgemm_fp16_weight_b(a, b_bits, m: int, k: int, n: int, threads: int = 1) -> np.ndarray:
+    """``SimdGemm.SgemmFp16WeightB`` (src/AiDotNet.Tensors/Engines/Simd/SimdGemm.Fp16Weight.cs:22-91): fp32 A times fp16
+    weights (bit patterns) -> fp32.  The reference widens the weights exactly while packing B (``PackBFromHalf``, :208-261) and
+    then runs the ordinary fp32 macro-kernel, so the value is the restated SimdGemm on the widened weights."""
+    return sgemm(a, f16_to_f32(np.asarray(b_bits, np.uint16)).reshape(k, n), m, k, n, threads)
+
+
 def bias_activation(c, bias, act: int = 0, param: float = 0.0) -> np.ndarray:
     """The FusedLinear epilogue act(c + bias) on a [M, N] fp32 matrix (bias [N] or None); returns a new array."""
     out = np.array(c, np.float32, copy=True, order="C")

@@ -181,3 +181,83 @@ def test_gpu_unknown_activation_is_an_argument_error(be):
     t = be.WrapTensor(torch.zeros(16, device="cuda"))
     with pytest.raises(ArgumentException):
         be.GemmBiasActivationInto(t, t, None, t, 4, 4, 4, 9)
+
+
+# ------------------------------------------------------------------------------------------------ weight-only fp16 GEMM
+def test_oracle_fp16_weight_gemm_matches_float64_of_widened_weights():
+    rng = np.random.default_rng(12)
+    m, k, n = 37, 71, 53
+    a = rng.standard_normal((m, k)).astype(np.float32); b = rng.standard_normal((k, n)).astype(np.float32)
+    bb, br = round_to(b, "f16")
+    got = oracle.sgemm_fp16_weight_b(a, bb, m, k, n)
+    assert mixed_err(got, a.astype(np.float64) @ br.astype(np.float64)) <= 1e-5
+    assert not np.array_equal(got, oracle.sgemm(a, b, m, k, n))          # the weights really are the rounded ones
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [(7, 13, 11), (96, 130, 80), (37, 53, 71), (256, 512, 192), (8, 4096, 1024), (4096, 768, 768)])
+def test_gpu_fp16_weight_gemm(be, m, n, k):
+    rng = np.random.default_rng(m + n + k)
+    a = rng.standard_normal((m, k)).astype(np.float32); b = (rng.standard_normal((k, n)) / math.sqrt(k)).astype(np.float32)
+    bias = rng.standard_normal(n).astype(np.float32)
+    bb, br = round_to(b, "f16")
+    W = be.WrapTensor
+    c = torch.full((m * n,), 3.0e30, device="cuda")
+    be.GemmFp16WeightB(W(dev(a)), W(from_bits16(bb, torch.float16)), None, W(c), m, n, k)
+    got = c.cpu().numpy().reshape(m, n)
+    truth = a.astype(np.float64) @ br.astype(np.float64)
+    assert mixed_err(got, truth) <= 1e-4
+    if m * n * k <= 1 << 24:
+        assert mixed_err(got, oracle.sgemm_fp16_weight_b(a, bb, m, k, n)) <= 1e-4
+    be.GemmFp16WeightB(W(dev(a)), W(from_bits16(bb, torch.float16)), W(dev(bias)), W(c), m, n, k, 2)
+    assert mixed_err(c.cpu().numpy().reshape(m, n), act64(truth + bias[None, :], 2)) <= 1e-4
+
+
+@pytest.mark.gpu
+def test_gpu_fp16_weight_gemm_exact_on_dyadic_inputs_and_engine_route(be):
+    from aidotnet.tensors_amd import Mi355Engine
+    rng = np.random.default_rng(2)
+    m, n, k = 128, 192, 96
+    a = rng.integers(-4, 5, (m, k)).astype(np.float32) / 4; b = rng.integers(-4, 5, (k, n)).astype(np.float32) / 4
+    eng = Mi355Engine(be)
+    out = eng.TensorMatMulFp16WeightB(dev(a), dev(b).half())
+    assert np.array_equal(out.cpu().numpy().astype(np.float64), a.astype(np.float64) @ b.astype(np.float64))
+    out = eng.FusedLinearFp16WeightB(dev(a).reshape(2, 64, k), dev(b).half(), None, "ReLU")
+    assert tuple(out.shape) == (2, 64, n)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,k,n", [(64, 128, 100), (48, 96, 96), (3, 5, 7), (1, 320, 1280)])
+def test_gpu_fp16_weight_matmul_matches_upcast_then_matmul(be, m, k, n):
+    """The shapes and the bound (1e-3 + 1e-4 |e|) of tests/AiDotNet.Tensors.Tests/Engines/Fp16WeightGemmTests.cs:43-73: the fused
+    path and 'widen the whole weight, then MatMul' decode the same fp16 bit patterns."""
+    from aidotnet.tensors_amd import Mi355Engine
+    rng = np.random.default_rng(1234 + m * 31 + k * 7 + n)
+    a = (rng.random((m, k)) * 2 - 1).astype(np.float32)
+    w = dev((rng.random((k, n)) * 2 - 1).astype(np.float32)).half()
+    eng = Mi355Engine(be)
+    fused = eng.TensorMatMulFp16WeightB(dev(a), w).cpu().numpy()
+    assert fused.shape == (m, n)
+    upcast = eng.TensorMatMul(dev(a), w.float()).cpu().numpy()
+    assert np.all(np.abs(fused - upcast) < 1e-3 + 1e-4 * np.abs(upcast))
+    assert mixed_err(fused, oracle.sgemm_fp16_weight_b(a, w.cpu().view(torch.int16).numpy().view(np.uint16), m, k, n)) <= 1e-4
+
+
+@pytest.mark.gpu
+def test_gpu_fused_linear_fp16_weight_bias_and_rank_one_input(be):
+    """Fp16WeightGemmTests.cs:75-120: bias without activation, and a rank-1 input giving a rank-1 result."""
+    from aidotnet.tensors_amd import Mi355Engine
+    rng = np.random.default_rng(99)
+    eng = Mi355Engine(be)
+    m, k, n = 32, 64, 48
+    a = dev((rng.random((m, k)) * 2 - 1).astype(np.float32)); w = dev((rng.random((k, n)) * 2 - 1).astype(np.float32)).half()
+    bias = dev((rng.random(n) - 0.5).astype(np.float32))
+    ref = (a.cpu().double() @ w.cpu().double() + bias.cpu().double()).numpy()
+    got = eng.FusedLinearFp16WeightB(a, w, bias, "None").cpu().numpy()
+    assert got.shape == (m, n) and np.all(np.abs(got - ref) < 1e-3 + 1e-4 * np.abs(ref))
+    k, n = 40, 24
+    a1 = dev((rng.random(k) * 2 - 1).astype(np.float32)); w = dev((rng.random((k, n)) * 2 - 1).astype(np.float32)).half()
+    got = eng.FusedLinearFp16WeightB(a1, w, None, "None")
+    assert tuple(got.shape) == (n,)
+    ref = (a1.cpu().double() @ w.cpu().double()).numpy()
+    assert np.all(np.abs(got.cpu().numpy() - ref) < 1e-3 + 1e-4 * np.abs(ref))
