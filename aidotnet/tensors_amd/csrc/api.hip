@@ -327,6 +327,19 @@ AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
     return AIDN_OK;
 }
 
+// workspace of the small-M fp32 path (M <= 8, B [K,N]); *ws stays null when the path does not apply or a tile size is forced
+static int smallm_ws(Ctx* c, int M, int N, int K, int transB, void** ws)
+{
+    *ws = nullptr;
+    if (c->force_tile != 0 || transB) return 0;
+    size_t need = aidn::gemm_f32_workspace_bytes(M, N, K);
+    if (!need) return 0;
+    int st = ensure_ws(c, need);
+    if (st) return st;
+    *ws = c->ws;
+    return 0;
+}
+
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
                      int M, int N, int K, float alpha, float beta, int transB)
 {
@@ -335,7 +348,10 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
     int tile = c->force_tile == 256 ? 0 : c->force_tile;
-    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile), "gemm_f32");
+    void* ws = nullptr;
+    if (int st = smallm_ws(c, M, N, K, transB, &ws)) return st;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),
+                      "gemm_f32");
 }
 
 AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, const float* B, float* C,
@@ -361,7 +377,9 @@ AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, 
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: unknown activation");
     int tile = c->force_tile == 256 ? 0 : c->force_tile;
-    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param),
+    void* ws = nullptr;
+    if (int st = smallm_ws(c, M, N, K, 0, &ws)) return st;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param, ws),
                       "gemm_f32 (bias + activation)");
 }
 AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A, const uint16_t* B_f16, const float* bias, float* C,
@@ -372,7 +390,9 @@ AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A,
     if (!A || !B_f16 || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: unknown activation");
-    return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param),
+    void* ws = nullptr;
+    if (int st = smallm_ws(c, M, N, K, 0, &ws)) return st;
+    return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param, ws),
                       "gemm_f32_f16weight");
 }
 AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,

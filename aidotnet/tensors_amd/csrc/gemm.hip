@@ -631,14 +631,27 @@ __global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, f
 
 template <typename OutT>
 __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restrict__ ws, void* __restrict__ Cv, int M, int N, int ksplit,
-                                                             const float* __restrict__ bias, int act, float act_param)
+                                                             const float* __restrict__ bias, int act, float act_param,
+                                                             float alpha = 1.0f, float beta = 0.0f)
 {
     typedef typename Raw<OutT>::type out_t;
     out_t* C = (out_t*)Cv;
     const long long total = (long long)M * N;
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
         float s = 0.0f;
-        for (int k = 0; k < ksplit; k++) s += ws[(long long)k * total + i];
+        int k = 0;
+        for (; k + 8 <= ksplit; k += 8) {              // eight loads in flight, summed in split order
+            float t[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) t[u] = ws[(long long)(k + u) * total + i];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += t[u];
+        }
+        for (; k < ksplit; k++) s += ws[(long long)k * total + i];
+        if constexpr (Elem<OutT>::BYTES == 4) {
+            s *= alpha;
+            if (beta != 0.0f) s += beta * as_f32(C[i]);
+        }
         if (bias) s += bias[i % N];
         s = apply_activation(s, act, act_param);
         if constexpr (Elem<OutT>::BYTES == 4) C[i] = as_u32(s);
@@ -674,7 +687,158 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
     if (e != hipSuccess) return e;
     long long total = (long long)g.M * g.N;
     unsigned grid = (unsigned)((total + 255) / 256);
-    hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks, g.bias, g.act, g.act_param);
+    hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks, g.bias, g.act, g.act_param,
+                       1.0f, 0.0f);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
+// Small-M fp32 path (M <= 8, B stored [K,N] as fp32 or as fp16 weights): the GPU form of the N-parallel small-M GEMM.
+// HBM-bound: B is read exactly once and nothing is staged, every lane owns four adjacent columns (one 16-byte load of a
+// B row, 8 bytes for fp16 weights) and MR rows of accumulators; the A values of a k-row are the same for the whole wave
+// and come through scalar loads.  grid = (ceil(N / 256), ksplit): the four waves of a workgroup take a quarter of the
+// workgroup's K range each and are summed through LDS, the K ranges of different workgroups through an fp32 workspace that
+// skinny_reduce_kernel sums in split order (deterministic) and finishes with alpha, beta, bias and activation.
+template <int MR, bool B16, bool VEC>
+__global__ __launch_bounds__(256) void gemm_smallm_kernel(const GemmArgs g, float* __restrict__ ws, int kper)
+{
+    __shared__ f32x4 red[3][MR][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int n = blockIdx.x * 256 + lane * 4;
+    const int ks = blockIdx.y;
+    const int kb = ks * kper, ke = min(g.K, kb + kper);
+    const int kq = ((ke - kb + 3) >> 2);
+    const int k0 = min(ke, kb + wave * kq), k1 = min(ke, k0 + kq);
+    const float* __restrict__ A = (const float*)g.A;
+    const int nvalid = g.N - n;                       // columns this lane owns: min(4, nvalid), none if <= 0
+
+    auto load_b = [&](int k) -> f32x4 {
+        f32x4 r = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (nvalid <= 0) return r;
+        if constexpr (B16) {
+            const uint16_t* p = (const uint16_t*)g.B + (long long)k * g.ldb + n;
+            if (VEC) {
+                u32x2 w = *(const u32x2*)p;
+                r[0] = f16_bits_to_float(w[0] & 0xFFFFu); r[1] = f16_bits_to_float(w[0] >> 16);
+                r[2] = f16_bits_to_float(w[1] & 0xFFFFu); r[3] = f16_bits_to_float(w[1] >> 16);
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (e < nvalid) r[e] = f16_bits_to_float(p[e]);
+            }
+        } else {
+            const float* p = (const float*)g.B + (long long)k * g.ldb + n;
+            if (VEC) r = *(const f32x4*)p;
+            else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) if (e < nvalid) r[e] = p[e];
+            }
+        }
+        return r;
+    };
+
+    f32x4 acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) acc[m] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const float* arow[MR];
+#pragma unroll
+    for (int m = 0; m < MR; m++) arow[m] = A + (long long)min(m, g.M - 1) * g.lda;
+
+    int k = k0;
+    for (; k + 8 <= k1; k += 8) {
+        f32x4 b[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) b[u] = load_b(k + u);
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float av = arow[m][k + u];
+#pragma unroll
+                for (int e = 0; e < 4; e++) acc[m][e] = fmaf(av, b[u][e], acc[m][e]);
+            }
+        }
+    }
+    for (; k < k1; k++) {
+        const f32x4 b = load_b(k);
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            const float av = arow[m][k];
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc[m][e] = fmaf(av, b[e], acc[m][e]);
+        }
+    }
+
+    if (wave > 0) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) red[wave - 1][m][lane] = acc[m];
+    }
+    __syncthreads();
+    if (wave == 0 && nvalid > 0) {
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            if (m < g.M) {
+                f32x4 v = acc[m];
+#pragma unroll
+                for (int w = 0; w < 3; w++) {
+                    const f32x4 o = red[w][m][lane];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[e] += o[e];
+                }
+                float* dst = ws + ((long long)ks * g.M + m) * g.N + n;
+                if (VEC) *(f32x4*)dst = v;
+                else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) if (e < nvalid) dst[e] = v[e];
+                }
+            }
+        }
+    }
+}
+
+static bool smallm_applies(int M, int N, int K) { return M >= 1 && M <= 8 && (long long)N * K >= 4096; }
+
+// K range of one workgroup: about 1024 workgroups, at least 128 k-rows each (32 per wave), a multiple of 32
+static int smallm_kper(int N, int K)
+{
+    const int colblocks = (N + 255) / 256;
+    int ks = (1024 + colblocks - 1) / colblocks;
+    int kper = (K + ks - 1) / ks;
+    if (kper < 128) kper = 128;
+    kper = (kper + 31) / 32 * 32;
+    return kper;
+}
+
+size_t gemm_f32_workspace_bytes(int M, int N, int K)
+{
+    if (!smallm_applies(M, N, K)) return 0;
+    const int kper = smallm_kper(N, K);
+    return (size_t)((K + kper - 1) / kper) * M * N * sizeof(float);
+}
+
+template <bool B16>
+static hipError_t launch_smallm(const GemmArgs& g, hipStream_t stream, float* ws)
+{
+    const int kper = smallm_kper(g.N, g.K);
+    const int ks = (g.K + kper - 1) / kper;
+    const bool vec = g.N % 4 == 0 && g.ldb % 4 == 0 && (((uintptr_t)g.B) & (B16 ? 7u : 15u)) == 0;
+    const dim3 grid((unsigned)((g.N + 255) / 256), (unsigned)ks);
+    const int mr = g.M <= 1 ? 1 : g.M <= 2 ? 2 : g.M <= 4 ? 4 : 8;
+#define AIDN_SMALLM(MR_)                                                                                               \
+    do {                                                                                                               \
+        if (vec) hipLaunchKernelGGL((gemm_smallm_kernel<MR_, B16, true>), grid, dim3(256), 0, stream, g, ws, kper);     \
+        else hipLaunchKernelGGL((gemm_smallm_kernel<MR_, B16, false>), grid, dim3(256), 0, stream, g, ws, kper);        \
+    } while (0)
+    if (mr == 1) AIDN_SMALLM(1);
+    else if (mr == 2) AIDN_SMALLM(2);
+    else if (mr == 4) AIDN_SMALLM(4);
+    else AIDN_SMALLM(8);
+#undef AIDN_SMALLM
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const long long total = (long long)g.M * g.N;
+    hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks,
+                       g.bias, g.act, g.act_param, g.alpha, g.beta);
     return hipGetLastError();
 }
 
@@ -739,18 +903,21 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
 
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile, const float* bias, int act, float act_param)
+                    int force_tile, const float* bias, int act, float act_param, void* workspace)
 {
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
+    if (force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
+        return launch_smallm<false>(g, stream, (float*)workspace);
     if (transB) return dispatch_gemm<float, float, true>(g, batch, stream, force_tile);
     return dispatch_gemm<float, float, false>(g, batch, stream, force_tile);
 }
 
 // fp32 A [M,K] x fp16 weights B [K,N] -> fp32 C, optional fused epilogue
 hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K,
-                              int force_tile, const float* bias, int act, float act_param)
+                              int force_tile, const float* bias, int act, float act_param, void* workspace)
 {
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
+    if (force_tile == 0 && workspace && smallm_applies(M, N, K)) return launch_smallm<true>(g, stream, (float*)workspace);
     // rows of A in 16-byte steps, rows of the fp16 B in 8-byte steps
     const bool vec = aligned16(A) && K % 4 == 0 && (((uintptr_t)B) & 7u) == 0 && N % 4 == 0;
     auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };

@@ -58,7 +58,10 @@ AIDN_API int aidn_mi355_sync(void* ctx, void* stream);
  * [N,K] (C = A * B^T).  Replaces IDirectGpuBackend.Gemm (IDirectGpuBackend.cs:160-172; host
  * HipBackend.cs:1370-1447, hipblasSgemm :1502-1545) and MatMulTransposed (:184-203; host
  * HipBackend.cs:1450-1490).  Argument order (M, N, K) as at that layer.  True fp32 MFMA, fp32
- * accumulation (no TF32-style truncation). */
+ * accumulation (no TF32-style truncation).  M <= 8 with B [K,N] takes the bandwidth-bound small-M path (B streamed once,
+ * split-K partials in the context workspace, summed in a fixed order): the GPU form of SimdGemm.SgemmNParallelSmallM /
+ * SgemmConcatenatedProjections (Engines/Simd/SimdGemm.NParallelSmallM.cs:31-109); the same holds for the bias/activation
+ * and fp16-weight entry points below. */
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
                      int M, int N, int K, float alpha, float beta, int transB);
 

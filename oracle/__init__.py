@@ -136,6 +136,17 @@ def sgemm_fp16_weight_b(a, b_bits, m: int, k: int, n: int, threads: int = 1) -> 
     return sgemm(a, f16_to_f32(np.asarray(b_bits, np.uint16)).reshape(k, n), m, k, n, threads)
 
 
+def sgemm_small_m(a, b, m: int, k: int, n: int, c0=None) -> np.ndarray:
+    """``SimdGemm.SgemmNParallelSmallM`` (src/AiDotNet.Tensors/Engines/Simd/SimdGemm.NParallelSmallM.cs:31-85): the m <= 8 GEMM that
+    splits the output columns among workers; ``c0`` None = overwrite (``clearedOutput``), else accumulate into a copy of it.
+    ``SgemmConcatenatedProjections`` (:95-109) is this call on the concatenated weight."""
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    assert a.size == m * k and b.size == k * n
+    c = np.zeros((m, n), np.float32) if c0 is None else np.array(c0, np.float32).reshape(m, n).copy()
+    lib().orc_sgemm_small_m(_p(a, _f32p), k, _p(b, _f32p), n, _p(c, _f32p), m, k, n, 1 if c0 is None else 0)
+    return c
+
+
 def bias_activation(c, bias, act: int = 0, param: float = 0.0) -> np.ndarray:
     """The FusedLinear epilogue act(c + bias) on a [M, N] fp32 matrix (bias [N] or None); returns a new array."""
     out = np.array(c, np.float32, copy=True, order="C")

@@ -348,6 +348,28 @@ void orc_bias_act_f32(float* c, const float* bias, long m, long n, int act, floa
         }
 }
 
+/* SimdGemm.SgemmNParallelSmallM (src/AiDotNet.Tensors/Engines/Simd/SimdGemm.NParallelSmallM.cs:31-85): C[m,n] (+)= A[m,k] B[k,n]
+ * for small m.  Every output column is owned by one worker and is updated once per k in ascending k (one multiply and one
+ * add per step, :66-81), so the value of an element does not depend on how the columns are chunked: c = ((c0 + a0 b0) + a1 b1) + ...
+ * cleared != 0 starts from 0 (overwrite), otherwise from the existing C (accumulate). */
+void orc_sgemm_small_m(const float* a, int lda, const float* b, int ldb, float* c, int m, int k, int n, int cleared)
+{
+    if (m <= 0 || k <= 0 || n <= 0) return;
+#pragma omp parallel for schedule(static)
+    for (int j0 = 0; j0 < n; j0 += 64) {
+        int j1 = imin(n, j0 + 64);
+        for (int i = 0; i < m; i++) {
+            float* crow = c + (long)i * n;
+            if (cleared) for (int j = j0; j < j1; j++) crow[j] = 0.0f;
+            for (int p = 0; p < k; p++) {
+                float av = a[(long)i * lda + p];
+                const float* brow = b + (long)p * ldb;
+                for (int j = j0; j < j1; j++) crow[j] = crow[j] + av * brow[j];
+            }
+        }
+    }
+}
+
 int orc_max_threads(void)
 {
 #ifdef _OPENMP
