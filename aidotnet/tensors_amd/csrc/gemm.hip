@@ -235,7 +235,11 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
                     } else {
                         u32x4 in[4], out[4];
 #pragma unroll
-                        for (int r = 0; r < 4; r++) in[r] = rb[i * 4 + r];
+                        for (int r = 0; r < 4; r++) {
+                            in[r] = rb[i * 4 + r];
+                            // the renaming moves belong here, not behind the global loads (where they would wait for them)
+                            asm volatile("" : "+v"(in[r]));
+                        }
                         transpose4x4_b32(in, out);
 #pragma unroll
                         for (int c = 0; c < 4; c++) *(u32x4*)(bs + (nb * 4 + c) * ROWB + kb * 16) = out[c];
@@ -258,33 +262,43 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
     store_tile(0);
     __syncthreads();
 
+    // Fragments are double-buffered in registers: the LDS reads of step s+1 are in flight during the MFMAs of step s.
+    // The next tile is published (register -> LDS stores, barrier) BEFORE the last step of the current one, and its first
+    // fragments are read right after the barrier, so the barrier wait and the LDS latency are covered by that step's MFMAs.
+    const int frag_off = (wm * WTM + l32) * ROWB + h * 16 + kgrp * SPG * 32;
+    const int frag_off_b = (wn * WTN + l32) * ROWB + h * 16 + kgrp * SPG * 32;
+    u32x4 fa[2][TM], fb[2][TN];
+    auto read_frags = [&](int stage, int step, int buf) {
+        const unsigned char* as = As + stage * BM * ROWB + frag_off + step * 32;
+        const unsigned char* bs = Bs + stage * BN * ROWB + frag_off_b + step * 32;
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[buf][i] = *(const u32x4*)(as + i * 32 * ROWB);
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[buf][j] = *(const u32x4*)(bs + j * 32 * ROWB);
+    };
+    read_frags(0, 0, 0);
     for (int kt = 0; kt < KT; kt++) {
         const int stage = kt & 1;
-        if (kt + 1 < KT) load_tile((kt + 1) * BK);
-        const unsigned char* as = As + stage * BM * ROWB + (wm * WTM + l32) * ROWB + h * 16 + kgrp * SPG * 32;
-        const unsigned char* bs = Bs + stage * BN * ROWB + (wn * WTN + l32) * ROWB + h * 16 + kgrp * SPG * 32;
-        // fragments are double-buffered in registers: the LDS reads of step s+1 are in flight during the
-        // MFMAs of step s
-        u32x4 fa[2][TM], fb[2][TN];
-#pragma unroll
-        for (int i = 0; i < TM; i++) fa[0][i] = *(const u32x4*)(as + i * 32 * ROWB);
-#pragma unroll
-        for (int j = 0; j < TN; j++) fb[0][j] = *(const u32x4*)(bs + j * 32 * ROWB);
+        // The unchecked instance has no branch in the loop body (its last iteration fetches the last tile once more and
+        // publishes it to the unused stage), so loads, LDS traffic and MFMAs of one iteration can be interleaved freely.
+        const bool more = !CHECK || kt + 1 < KT;
+        if constexpr (!CHECK) load_tile(min(kt + 1, KT - 1) * BK);
+        else if (more) load_tile((kt + 1) * BK);
 #pragma unroll
         for (int s = 0; s < SPG; s++) {
-            if (s < SPG - 1) {
-#pragma unroll
-                for (int i = 0; i < TM; i++) fa[(s + 1) & 1][i] = *(const u32x4*)(as + i * 32 * ROWB + (s + 1) * 32);
-#pragma unroll
-                for (int j = 0; j < TN; j++) fb[(s + 1) & 1][j] = *(const u32x4*)(bs + j * 32 * ROWB + (s + 1) * 32);
+            if (s < SPG - 1) read_frags(stage, s + 1, (s + 1) & 1);
+            else {
+                __builtin_amdgcn_sched_barrier(0);      // keep the MFMAs of the last step below the barrier
+                if (more) store_tile(stage ^ 1);
+                __syncthreads();
+                if (more) read_frags(stage ^ 1, 0, SPG & 1);
             }
+            __builtin_amdgcn_sched_barrier(0);          // fragment reads of the next step are issued before this step's MFMAs
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
         }
-        if (kt + 1 < KT) store_tile(stage ^ 1);
-        __syncthreads();
     }
 
     if constexpr (KS == 2) {
@@ -864,6 +878,14 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
+// 128 x 128 or 64 x 64 tile, by how well the workgroups fill their rounds (512 resident 128 x 128 workgroups, 1024 of
+// 64 x 64); the larger tile is about 10 % more efficient per flop when both fill their rounds equally well.
+static int choose_tile(long long tiles128, long long tiles64)
+{
+    auto fill = [](long long t, long long slots) { return (double)t / (double)(((t + slots - 1) / slots) * slots); };
+    return fill(tiles128, 512) >= 0.9 * fill(tiles64, 1024) ? 128 : 64;
+}
+
 // Tile choice: the largest tile that still gives the 256 CUs roughly a full wave of
 // workgroups; the unchecked 256x256 instance only for shapes it divides exactly.
 template <typename T, typename OutT, bool TRANSB>
@@ -879,7 +901,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 &&
                 tiles(256, 256) >= 128) tile = 256;
         }
-        if (tile == 0) tile = tiles(128, 128) >= 192 ? 128 : 64;
+        if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64));
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 256) {
@@ -888,13 +910,20 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             return launch_gemm_dl<T, OutT>(g, stream);
         }
     }
+    // shapes the tile divides exactly take the instance without bounds checks
+    auto exact = [&](int bt) { return vec && g.M % bt == 0 && g.N % bt == 0 && g.K % (8 * E) == 0; };
     if (tile == 128) {
+        if (exact(128)) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, false>(g, batch, stream);
         if (vec) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, true>(g, batch, stream);
         return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, false, true>(g, batch, stream);
     }
     if (tile == 64) {
         // at most about one 64 x 64 tile per CU: split every K-tile between two wave groups so each SIMD still holds two waves
-        if (vec && tiles(64, 64) <= 320 && g.K >= 4 * 8 * E) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true, 2>(g, batch, stream);
+        if (vec && tiles(64, 64) <= 320 && g.K >= 4 * 8 * E) {
+            if (exact(64)) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, false, 2>(g, batch, stream);
+            return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true, 2>(g, batch, stream);
+        }
+        if (exact(64)) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, false>(g, batch, stream);
         if (vec) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true>(g, batch, stream);
         return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, false, true>(g, batch, stream);
     }
@@ -921,7 +950,7 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
     // rows of A in 16-byte steps, rows of the fp16 B in 8-byte steps
     const bool vec = aligned16(A) && K % 4 == 0 && (((uintptr_t)B) & 7u) == 0 && N % 4 == 0;
     auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    int tile = force_tile == 64 || force_tile == 128 ? force_tile : (tiles(128, 128) >= 192 ? 128 : 64);
+    int tile = force_tile == 64 || force_tile == 128 ? force_tile : choose_tile(tiles(128, 128), tiles(64, 64));
     if (tile == 128) {
         if (vec) return launch_gemm<float, float, 128, 128, 2, 2, false, true, true, 1, true>(g, 1, stream);
         return launch_gemm<float, float, 128, 128, 2, 2, false, false, true, 1, true>(g, 1, stream);
