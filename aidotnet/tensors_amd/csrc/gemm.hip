@@ -91,6 +91,24 @@ __device__ __forceinline__ u32x4 load16_guarded(const typename Raw<T>::type* p, 
 
 // KS = 2: two groups of WM x WN waves work on the same output tile, each on half of the k-steps of every K-tile, and the
 // second group's accumulators are added through LDS at the end (for grids too small to give every SIMD two waves).
+// Scheduling pattern for one step of straight-line code: NM MFMAs, each followed by its share of ND LDS reads, NV global
+// loads and NW LDS writes (in that order of urgency).
+template <int NM, int ND, int NV, int NW>
+__device__ __forceinline__ void spread_schedule()
+{
+    constexpr int TOT = ND + NV + NW;
+#pragma unroll
+    for (int i = 0; i < NM; i++) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+#pragma unroll
+        for (int o = i * TOT / NM; o < (i + 1) * TOT / NM; o++) {
+            if (o < ND) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            else if (o < ND + NV) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            else __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+        }
+    }
+}
+
 // B16 (fp32 kernels only): B holds fp16 weights [K,N]; they are widened to fp32 on the way into LDS, so the product is that
 // of the fp32 A with the exactly widened weights, accumulated in fp32 (weight-only fp16 GEMM).
 template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB, bool VEC, bool CHECK, int KS = 1, bool B16 = false>
@@ -128,10 +146,16 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
     const raw_t* __restrict__ A = (const raw_t*)g.A + bz * g.sA;
     const raw_t* __restrict__ B = (const raw_t*)g.B + bz * g.sB;
 
-    u32x4 ra[UA];
-    u32x4 rb[TRANSB ? UBT : UBN * E];
+    // Global loads run two tiles ahead where the registers allow it (tile t travels in register set t & 1 and has two
+    // iterations to arrive from memory: what a small problem with one workgroup per CU needs), otherwise one tile ahead.
+    constexpr bool AHEAD2 = BM * BN <= 64 * 64;
+    constexpr int NSETS = AHEAD2 ? 2 : 1;
+    u32x4 ra2[NSETS][UA];
+    u32x4 rb2[NSETS][TRANSB ? UBT : UBN * E];
 
-    auto load_tile = [&](int k0) {
+    auto load_tile = [&](int k0, auto setc) {
+        auto& ra = ra2[decltype(setc)::value];
+        auto& rb = rb2[decltype(setc)::value];
         // ---- A (and B when stored [N,K]): 16-byte chunks along K
 #pragma unroll
         for (int i = 0; i < UA; i++) {
@@ -205,7 +229,9 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
         }
     };
 
-    auto store_tile = [&](int stage) {
+    auto store_tile = [&](int stage, auto setc) {
+        auto& ra = ra2[decltype(setc)::value];
+        auto& rb = rb2[decltype(setc)::value];
         unsigned char* as = As + stage * BM * ROWB;
         unsigned char* bs = Bs + stage * BN * ROWB;
 #pragma unroll
@@ -258,13 +284,18 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
     const int KT = (g.K + BK - 1) / BK;
-    load_tile(0);
-    store_tile(0);
+    typedef std::integral_constant<int, 0> Set0;
+    typedef std::integral_constant<int, 1> Set1;
+    load_tile(0, Set0{});
+    store_tile(0, Set0{});
+    if constexpr (AHEAD2) {
+        if (!CHECK || KT > 1) load_tile(min(1, KT - 1) * BK, Set1{});
+    }
     __syncthreads();
 
     // Fragments are double-buffered in registers: the LDS reads of step s+1 are in flight during the MFMAs of step s.
-    // The next tile is published (register -> LDS stores, barrier) BEFORE the last step of the current one, and its first
-    // fragments are read right after the barrier, so the barrier wait and the LDS latency are covered by that step's MFMAs.
+    // Tile kt+1 is published (register -> LDS stores, barrier) BEFORE the last step of tile kt, and its first fragments are
+    // read right after the barrier, so the barrier wait and the LDS latency are covered by that step's MFMAs.
     const int frag_off = (wm * WTM + l32) * ROWB + h * 16 + kgrp * SPG * 32;
     const int frag_off_b = (wn * WTN + l32) * ROWB + h * 16 + kgrp * SPG * 32;
     u32x4 fa[2][TM], fb[2][TN];
@@ -276,22 +307,24 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int j = 0; j < TN; j++) fb[buf][j] = *(const u32x4*)(bs + j * 32 * ROWB);
     };
-    read_frags(0, 0, 0);
-    for (int kt = 0; kt < KT; kt++) {
-        const int stage = kt & 1;
-        // The unchecked instance has no branch in the loop body (its last iteration fetches the last tile once more and
+    // iteration kt works on LDS stage kt & 1 = SET, requests tile kt+2 into register set SET (free: tile kt was stored one
+    // iteration ago) and publishes tile kt+1 from the other set; with one set it requests tile kt+1 and publishes it
+    auto iteration = [&](int kt, int SET, auto intoc, auto otherc) {
+        typedef decltype(intoc) Into;
+        typedef decltype(otherc) Other;
+        // The unchecked instance has no branch in the loop body (past the end it fetches the last tile once more and
         // publishes it to the unused stage), so loads, LDS traffic and MFMAs of one iteration can be interleaved freely.
         const bool more = !CHECK || kt + 1 < KT;
-        if constexpr (!CHECK) load_tile(min(kt + 1, KT - 1) * BK);
-        else if (more) load_tile((kt + 1) * BK);
+        if constexpr (!CHECK) load_tile(min(kt + NSETS, KT - 1) * BK, Into{});
+        else if (kt + NSETS < KT) load_tile((kt + NSETS) * BK, Into{});
 #pragma unroll
         for (int s = 0; s < SPG; s++) {
-            if (s < SPG - 1) read_frags(stage, s + 1, (s + 1) & 1);
+            if (s < SPG - 1) read_frags(SET, s + 1, (s + 1) & 1);
             else {
                 __builtin_amdgcn_sched_barrier(0);      // keep the MFMAs of the last step below the barrier
-                if (more) store_tile(stage ^ 1);
+                if (more) store_tile(SET ^ 1, Other{});
                 __syncthreads();
-                if (more) read_frags(stage ^ 1, 0, SPG & 1);
+                if (more) read_frags(SET ^ 1, 0, SPG & 1);
             }
             __builtin_amdgcn_sched_barrier(0);          // fragment reads of the next step are issued before this step's MFMAs
 #pragma unroll
@@ -299,6 +332,56 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
                 for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
         }
+    };
+    // Unchecked instance: one iteration is straight-line code, and the order of its instructions is given explicitly: every
+    // MFMA is followed by its share of the step's other memory instructions (next fragments, the global loads in the first
+    // step, the LDS stores of the next tile in the last step before the barrier), so the matrix pipe never waits behind a
+    // burst of them.
+    auto mfma_step = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
+    };
+    auto iteration_il = [&](int kt, int SET, auto intoc, auto otherc) {
+        typedef decltype(intoc) Into;
+        typedef decltype(otherc) Other;
+        constexpr int NM = TM * TN * (E == 4 ? 4 : 1);          // MFMAs per step
+        constexpr int NL = UA + (TRANSB ? UBT : UBN * E);       // global loads = LDS stores per tile and thread
+        constexpr int NR = TM + TN;                             // fragment reads per step
+        load_tile(min(kt + NSETS, KT - 1) * BK, Into{});
+#pragma unroll
+        for (int s = 0; s < SPG - 1; s++) {
+            read_frags(SET, s + 1, (s + 1) & 1);
+            if (s == SPG - 2) store_tile(SET ^ 1, Other{});
+            mfma_step(s);
+            if (s == 0 && s == SPG - 2) spread_schedule<NM, NR, NL, NL>();
+            else if (s == 0) spread_schedule<NM, NR, NL, 0>();
+            else if (s == SPG - 2) spread_schedule<NM, NR, 0, NL>();
+            else spread_schedule<NM, NR, 0, 0>();
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        __syncthreads();
+        read_frags(SET ^ 1, 0, SPG & 1);
+        mfma_step(SPG - 1);
+        spread_schedule<NM, NR, 0, 0>();
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    read_frags(0, 0, 0);
+    if constexpr (!CHECK && AHEAD2) {
+        for (int kt = 0; kt < KT; kt += 2) {
+            iteration_il(kt, 0, Set0{}, Set1{});
+            if (kt + 1 < KT) iteration_il(kt + 1, 1, Set1{}, Set0{});
+        }
+    } else if constexpr (!CHECK) {
+        for (int kt = 0; kt < KT; kt++) iteration_il(kt, kt & 1, Set0{}, Set0{});
+    } else if constexpr (AHEAD2) {
+        for (int kt = 0; kt < KT; kt += 2) {
+            iteration(kt, 0, Set0{}, Set1{});
+            if (kt + 1 < KT) iteration(kt + 1, 1, Set1{}, Set0{});
+        }
+    } else {
+        for (int kt = 0; kt < KT; kt++) iteration(kt, kt & 1, Set0{}, Set0{});
     }
 
     if constexpr (KS == 2) {
@@ -878,12 +961,14 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
-// 128 x 128 or 64 x 64 tile, by how well the workgroups fill their rounds (512 resident 128 x 128 workgroups, 1024 of
-// 64 x 64); the larger tile is about 10 % more efficient per flop when both fill their rounds equally well.
-static int choose_tile(long long tiles128, long long tiles64)
+// 128 x 128 or 64 x 64 tile, by how evenly the workgroups load the 256 CUs (a CU works through 128 x 128 tiles at about
+// the same rate whether it holds one or two, so rounds of 256; two 64 x 64 tiles at a time, so rounds of 512); rel64 =
+// efficiency per flop of the smaller tile relative to the larger one when both fill their rounds equally well (measured:
+// about 0.85 for fp32, 0.55 for the 16-bit types).
+static int choose_tile(long long tiles128, long long tiles64, double rel64)
 {
     auto fill = [](long long t, long long slots) { return (double)t / (double)(((t + slots - 1) / slots) * slots); };
-    return fill(tiles128, 512) >= 0.9 * fill(tiles64, 1024) ? 128 : 64;
+    return fill(tiles128, 256) >= rel64 * fill(tiles64, 512) ? 128 : 64;
 }
 
 // Tile choice: the largest tile that still gives the 256 CUs roughly a full wave of
@@ -901,7 +986,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 &&
                 tiles(256, 256) >= 128) tile = 256;
         }
-        if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64));
+        if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 256) {
@@ -950,7 +1035,7 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
     // rows of A in 16-byte steps, rows of the fp16 B in 8-byte steps
     const bool vec = aligned16(A) && K % 4 == 0 && (((uintptr_t)B) & 7u) == 0 && N % 4 == 0;
     auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
-    int tile = force_tile == 64 || force_tile == 128 ? force_tile : choose_tile(tiles(128, 128), tiles(64, 64));
+    int tile = force_tile == 64 || force_tile == 128 ? force_tile : choose_tile(tiles(128, 128), tiles(64, 64), 0.85);
     if (tile == 128) {
         if (vec) return launch_gemm<float, float, 128, 128, 2, 2, false, true, true, 1, true>(g, 1, stream);
         return launch_gemm<float, float, 128, 128, 2, 2, false, false, true, 1, true>(g, 1, stream);
