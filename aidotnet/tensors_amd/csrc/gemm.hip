@@ -49,7 +49,11 @@ __device__ __forceinline__ float apply_activation(float x, int act, float p)
     }
 }
 
-constexpr int ROWB = 144;    // LDS row pitch in bytes
+// K extent of one tile of the general kernel in 16-byte chunks per row, and the LDS row pitch (one chunk of padding keeps the
+// b128 fragment reads conflict-free).  The 64 x 64 tile takes twice the K per barrier: its waves have too little MFMA work
+// per tile to hide one barrier every 128 bytes of K.
+constexpr int gemm_k_chunks(int bm, int bn) { return bm * bn <= 64 * 64 ? 16 : 8; }
+constexpr int gemm_row_pitch(int bm, int bn) { return gemm_k_chunks(bm, bn) * 16 + 16; }
 constexpr int GROUP_M = 8;   // tile rows walked together so one XCD's L2 sees a compact footprint
 
 // Workgroup id -> (tile row, tile col).  Hardware hands consecutive workgroup ids to the 8
@@ -117,15 +121,17 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
     static_assert(!B16 || (Elem<T>::BYTES == 4 && !TRANSB), "fp16 weights: fp32 kernel, B stored [K,N]");
     typedef typename Raw<T>::type raw_t;
     constexpr int E = Elem<T>::PER16;
-    constexpr int BK = 8 * E;                  // elements of K per tile (128 bytes)
+    constexpr int KC = gemm_k_chunks(BM, BN);  // 16-byte chunks of K per tile row
+    constexpr int BK = KC * E;                 // elements of K per tile
+    constexpr int ROWB = gemm_row_pitch(BM, BN);
     constexpr int NT = WM * WN * KS * 64;
-    constexpr int SPG = 4 / KS;                // fragment steps of a K-tile per wave group
+    constexpr int SPG = KC / 2 / KS;                // fragment steps of a K-tile per wave group
     static_assert(KS == 1 || KS == 2, "KS must be 1 or 2");
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int UA = (BM * 8 + NT - 1) / NT;                   // 16-byte chunks of A per thread
-    constexpr int UBT = (BN * 8 + NT - 1) / NT;                  // same for B stored [N,K]
-    constexpr int NBLK = 8 * (BN / E);                           // E x E blocks of B stored [K,N]
+    constexpr int UA = (BM * KC + NT - 1) / NT;                   // 16-byte chunks of A per thread
+    constexpr int UBT = (BN * KC + NT - 1) / NT;                  // same for B stored [N,K]
+    constexpr int NBLK = KC * (BN / E);                           // E x E blocks of B stored [K,N]
     constexpr int UBN = (NBLK + NT - 1) / NT;
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of 32x32");
 
@@ -160,10 +166,10 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int i = 0; i < UA; i++) {
             int u = t + i * NT;
-            int row = u >> 3, ch = u & 7;
+            int row = u / KC, ch = u % KC;
             int gm = m0 + row, gk = k0 + ch * E;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if ((BM * 8) % NT == 0 || u < BM * 8) {
+            if ((BM * KC) % NT == 0 || u < BM * KC) {
                 const raw_t* p = A + (long long)gm * g.lda + gk;
                 if constexpr (!CHECK) v = *(const u32x4*)p;
                 else if (gm < g.M && gk < g.K) {
@@ -177,10 +183,10 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
             for (int i = 0; i < UBT; i++) {
                 int u = t + i * NT;
-                int row = u >> 3, ch = u & 7;
+                int row = u / KC, ch = u % KC;
                 int gn = n0 + row, gk = k0 + ch * E;
                 u32x4 v = {0u, 0u, 0u, 0u};
-                if ((BN * 8) % NT == 0 || u < BN * 8) {
+                if ((BN * KC) % NT == 0 || u < BN * KC) {
                     const raw_t* p = B + (long long)gn * g.ldb + gk;
                     if constexpr (!CHECK) v = *(const u32x4*)p;
                     else if (gn < g.N && gk < g.K) {
@@ -195,7 +201,7 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
             for (int i = 0; i < UBN; i++) {
                 int u = t + i * NT;
-                int kb = u & 7, nb = u >> 3;
+                int kb = u % KC, nb = u / KC;
                 int gn = n0 + nb * E;
 #pragma unroll
                 for (int r = 0; r < E; r++) {
@@ -237,19 +243,19 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
 #pragma unroll
         for (int i = 0; i < UA; i++) {
             int u = t + i * NT;
-            if ((BM * 8) % NT == 0 || u < BM * 8) *(u32x4*)(as + (u >> 3) * ROWB + (u & 7) * 16) = ra[i];
+            if ((BM * KC) % NT == 0 || u < BM * KC) *(u32x4*)(as + (u / KC) * ROWB + (u % KC) * 16) = ra[i];
         }
         if constexpr (TRANSB) {
 #pragma unroll
             for (int i = 0; i < UBT; i++) {
                 int u = t + i * NT;
-                if ((BN * 8) % NT == 0 || u < BN * 8) *(u32x4*)(bs + (u >> 3) * ROWB + (u & 7) * 16) = rb[i];
+                if ((BN * KC) % NT == 0 || u < BN * KC) *(u32x4*)(bs + (u / KC) * ROWB + (u % KC) * 16) = rb[i];
             }
         } else {
 #pragma unroll
             for (int i = 0; i < UBN; i++) {
                 int u = t + i * NT;
-                int kb = u & 7, nb = u >> 3;
+                int kb = u % KC, nb = u / KC;
                 if (NBLK % NT == 0 || u < NBLK) {
                     if constexpr (E == 8) {
                         u32x4 in[8], out[8];
@@ -944,7 +950,7 @@ template <typename T, typename OutT, int BM, int BN, int WM, int WN, bool TRANSB
 static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 {
     auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK, KS, B16>;
-    constexpr int tiles_smem = 2 * (BM + BN) * ROWB, merge_smem = KS == 2 ? BM * BN * 4 : 0;
+    constexpr int tiles_smem = 2 * (BM + BN) * gemm_row_pitch(BM, BN), merge_smem = KS == 2 ? BM * BN * 4 : 0;
     constexpr int smem = tiles_smem > merge_smem ? tiles_smem : merge_smem;
     static bool attr_set = false;
     if (!attr_set) {
@@ -996,7 +1002,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         }
     }
     // shapes the tile divides exactly take the instance without bounds checks
-    auto exact = [&](int bt) { return vec && g.M % bt == 0 && g.N % bt == 0 && g.K % (8 * E) == 0; };
+    auto exact = [&](int bt) { return vec && g.M % bt == 0 && g.N % bt == 0 && g.K % (gemm_k_chunks(bt, bt) * E) == 0; };
     if (tile == 128) {
         if (exact(128)) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, false>(g, batch, stream);
         if (vec) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, true>(g, batch, stream);
@@ -1004,7 +1010,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     }
     if (tile == 64) {
         // at most about one 64 x 64 tile per CU: split every K-tile between two wave groups so each SIMD still holds two waves
-        if (vec && tiles(64, 64) <= 320 && g.K >= 4 * 8 * E) {
+        if (vec && tiles(64, 64) <= 320 && g.K >= 4 * 16 * E) {
             if (exact(64)) return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, false, 2>(g, batch, stream);
             return launch_gemm<T, OutT, 64, 64, 2, 2, TRANSB, true, true, 2>(g, batch, stream);
         }
