@@ -473,6 +473,13 @@ __device__ __forceinline__ void dma16_to_lds(const void* gptr, void* lds_dst_wav
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(l), "v"(gptr));
 }
 
+// same, source = wave-uniform base (scalar register pair) + per-lane unsigned 32-bit byte offset, destination given as the LDS
+// byte address
+__device__ __forceinline__ void dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
+}
+
 template <typename T, typename OutT>
 __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 {
@@ -496,28 +503,31 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     const raw_t* __restrict__ A = (const raw_t*)g.A;
     const raw_t* __restrict__ B = (const raw_t*)g.B;
 
-    // per-lane global sources of this wave's loads at k0 = 0
-    const raw_t* pa[LA];
-    const raw_t* pb[LB];
+    // Sources of this wave's loads: a wave-uniform base (scalar registers, advanced per tile by scalar adds) plus a per-lane
+    // 32-bit byte offset that never changes, so issuing a load costs no vector instruction.  Wave-load w = 4 wave + i covers
+    // A rows 8w .. 8w+7 resp. B k-rows 2w, 2w+1; the swizzle of a lane depends on w only through its parity, i.e. on i & 1.
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+    uint32_t a_lane_off[2], b_lane_off[2];
 #pragma unroll
-    for (int i = 0; i < LA; i++) {
-        int w = wave * LA + i;                                // A wave-load w: rows 8w .. 8w+7
-        int row = 8 * w + (lane >> 3), pos = lane & 7;
-        pa[i] = A + (long long)(m0 + row) * g.lda + (pos ^ ((row >> 1) & 7)) * 8;
+    for (int par = 0; par < 2; par++) {
+        const int ra = lane >> 3, pos_a = lane & 7;           // row inside the wave-load, 16-byte chunk
+        a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * 8) * 2u;
+        const int rb = lane >> 5, pos_b = lane & 31;
+        b_lane_off[par] = (uint32_t)(rb * g.ldb + (pos_b ^ (((2 * par + rb) & 3) << 2)) * 8) * 2u;
     }
-#pragma unroll
-    for (int i = 0; i < LB; i++) {
-        int w = wave * LB + i;                                // B wave-load w: k-rows 2w, 2w+1
-        int row = 2 * w + (lane >> 5), pos = lane & 31;
-        pb[i] = B + (long long)row * g.ldb + n0 + (pos ^ ((row & 3) << 2)) * 8;
-    }
+    const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + 8 * LA * wave_s) * g.lda);
+    const unsigned char* b_base = (const unsigned char*)(B + (long long)(2 * LB * wave_s) * g.ldb + n0);
+    const long long a_step = 8LL * g.lda * 2, b_step = 2LL * g.ldb * 2;        // bytes between consecutive wave-loads
     auto issue_loads = [&](int kt, int stage) {
-        unsigned char* as = smem + stage * STAGE;
-        unsigned char* bs = as + ABYTES;
+        const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
+        const uint32_t bs = lds0 + stage * STAGE + ABYTES + wave_s * (LB * 1024);
+        const unsigned char* a_src = a_base + (long long)kt * (BK * 2);
+        const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * 2;
 #pragma unroll
-        for (int i = 0; i < LA; i++) dma16_to_lds(pa[i] + kt * BK, as + (wave * LA + i) * 1024);
+        for (int i = 0; i < LA; i++) dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
 #pragma unroll
-        for (int i = 0; i < LB; i++) dma16_to_lds(pb[i] + (long long)kt * BK * g.ldb, bs + (wave * LB + i) * 1024);
+        for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i & 1], bs + i * 1024);
     };
 
     // per-lane LDS read offsets
@@ -590,11 +600,14 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
                     read_frags(an, an + ABYTES, 0, fa[0], fb[0]);
                 }
             }
-            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int i = 0; i < TM; i++)
 #pragma unroll
                 for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
+            // the next step's fragment reads go behind the first half of this step's MFMAs (two each), so the matrix pipe does
+            // not wait behind a burst of reads and the last read still has half a step to complete
+            spread_schedule<TM * TN / 2, TM + 2 * TN, 0, 0>();
+            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM * TN / 2, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
