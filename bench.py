@@ -39,12 +39,21 @@ TRAFFIC_BYTES = {
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
+# untimed warm-up of every secondary configuration lasts at least this long (their steps are tens of microseconds)
+OTHERS_MIN_WARM_MS = 60.0
 
 
-def _events_time(torch, fn, steps, warmup):
+def _events_time(torch, fn, steps, warmup, min_warm_ms=0.0):
+    """`warmup` untimed steps, continued until `min_warm_ms` of wall time has passed (short kernels need some tens of
+    milliseconds of their own load before the clock management of the device settles), then exactly `steps` timed steps."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    t_warm = time.perf_counter()
+    while (time.perf_counter() - t_warm) * 1e3 < min_warm_ms:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
     start = torch.cuda.Event(enable_timing=True)
     end = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
@@ -73,7 +82,7 @@ def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--only", default="", help="comma list of workloads to time besides the headline (default: all)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -150,7 +159,7 @@ def main() -> int:
 
         def fn():
             fn1(Bs[it[0] % rotate]); it[0] += 1
-        ms_, _ = _events_time(torch, fn, steps, warmup)
+        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
         fl = 2.0 * M * N * K
         if hbm:
             eb = a_.element_size()
@@ -172,7 +181,7 @@ def main() -> int:
             fn = lambda: be.FlashAttentionV2(W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, sc, True)
         else:
             fn = lambda: be.FlashAttentionHalf(kind, W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, sc, True)
-        ms_, _ = _events_time(torch, fn, steps, warmup)
+        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
         exact = 4.0 * Bn * H * D * (S * (S + 1) / 2)
         roof = _roof_flops(kind, exact, ms_, TRAFFIC_BYTES.get(name))
         roof["tflops_full_matrix_convention"] = round(4.0 * Bn * H * S * S * D / (ms_ * 1e-3) / 1e12, 3)
@@ -185,7 +194,7 @@ def main() -> int:
         o = torch.empty(Bn, H, 1, D, device="cuda")
         sc = 1.0 / math.sqrt(D)
         fn = lambda: be.DecodeAttention(kind, W(q), W(k), W(v), W(o), Bn, H, S, D, sc)
-        ms_, _ = _events_time(torch, fn, steps, warmup)
+        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
         nbytes = 2.0 * Bn * H * S * D * q.element_size()
         add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)))
 
