@@ -480,7 +480,10 @@ __device__ __forceinline__ void dma16_base(const void* base_uniform, uint32_t la
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
 }
 
-template <typename T, typename OutT>
+// EDGE: M and N need not be multiples of 256 (N still a multiple of 8, K of 64): loads of rows / column chunks past the end
+// are redirected to the last valid one (their products land in accumulator elements that are never stored) and the stores
+// are guarded.
+template <typename T, typename OutT, bool EDGE = false>
 __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 {
     typedef uint16_t raw_t;
@@ -508,15 +511,26 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     // A rows 8w .. 8w+7 resp. B k-rows 2w, 2w+1; the swizzle of a lane depends on w only through its parity, i.e. on i & 1.
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
-    uint32_t a_lane_off[2], b_lane_off[2];
+    uint32_t a_lane_off[EDGE ? LA : 2], b_lane_off[2];
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         const int ra = lane >> 3, pos_a = lane & 7;           // row inside the wave-load, 16-byte chunk
-        a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * 8) * 2u;
+        if constexpr (!EDGE) a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * 8) * 2u;
         const int rb = lane >> 5, pos_b = lane & 31;
-        b_lane_off[par] = (uint32_t)(rb * g.ldb + (pos_b ^ (((2 * par + rb) & 3) << 2)) * 8) * 2u;
+        int chunk = pos_b ^ (((2 * par + rb) & 3) << 2);
+        if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / 8 - 1);          // N % 8 == 0 and n0 < N: at least one chunk
+        b_lane_off[par] = (uint32_t)(rb * g.ldb + chunk * 8) * 2u;
     }
-    const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + 8 * LA * wave_s) * g.lda);
+    if constexpr (EDGE) {
+#pragma unroll
+        for (int i = 0; i < LA; i++) {
+            const int ra = lane >> 3, pos_a = lane & 7;
+            const int row = min(8 * (LA * wave + i) + ra, g.M - 1 - m0);      // source row inside the tile (m0 < M)
+            a_lane_off[i] = (uint32_t)(row * g.lda + (pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7)) * 8) * 2u;
+        }
+    }
+    // (EDGE: the A offsets are relative to the tile's first row, since a clamped row may lie before the wave's own rows)
+    const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda);
     const unsigned char* b_base = (const unsigned char*)(B + (long long)(2 * LB * wave_s) * g.ldb + n0);
     const long long a_step = 8LL * g.lda * 2, b_step = 2LL * g.ldb * 2;        // bytes between consecutive wave-loads
     auto issue_loads = [&](int kt, int stage) {
@@ -525,7 +539,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
         const unsigned char* a_src = a_base + (long long)kt * (BK * 2);
         const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * 2;
 #pragma unroll
-        for (int i = 0; i < LA; i++) dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
+        for (int i = 0; i < LA; i++) {
+            if constexpr (EDGE) dma16_base(a_src, a_lane_off[i], as + i * 1024);
+            else dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
+        }
 #pragma unroll
         for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i & 1], bs + i * 1024);
     };
@@ -620,6 +637,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
+            if (EDGE && col >= g.N) continue;
             if (fused) {                                  // bias and / or activation folded into the store
                 const float bias = g.bias ? g.bias[col] : 0.0f;
 #pragma unroll
@@ -628,6 +646,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                if (EDGE && row >= g.M) continue;
                 out_t* p = C + (long long)row * g.ldc + col;
                 if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(acc[i][j][r]);
                 else *p = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
@@ -635,10 +654,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
         }
 }
 
-template <typename T, typename OutT>
+template <typename T, typename OutT, bool EDGE = false>
 static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
 {
-    auto kern = gemm_dl_kernel<T, OutT>;
+    auto kern = gemm_dl_kernel<T, OutT, EDGE>;
     constexpr int smem = 2 * (256 * 128 + 64 * 512);
     static bool attr_set = false;
     if (!attr_set) {
@@ -646,8 +665,8 @@ static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    g.tiles_m = g.M / 256;
-    g.tiles_n = g.N / 256;
+    g.tiles_m = (g.M + 255) / 256;
+    g.tiles_n = (g.N + 255) / 256;
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), smem, stream, g);
     return hipGetLastError();
 }
@@ -1002,16 +1021,19 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     int tile = force_tile;
     if (tile == 0) {
         if constexpr (E == 8 && !TRANSB) {
-            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0 &&
+            // the 256 x 256 kernel: K a multiple of 64, rows of B in whole 16-byte chunks, leading dimensions within the 32-bit
+            // lane offsets of its loads; M and N may be ragged
+            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldb < (1 << 22) &&
                 tiles(256, 256) >= 128) tile = 256;
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 256) {
-            if (!(vec && g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0)) return hipErrorInvalidValue;
+            if (!(vec && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldb < (1 << 22))) return hipErrorInvalidValue;
             if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
-            return launch_gemm_dl<T, OutT>(g, stream);
+            if (g.M % 256 == 0 && g.N % 256 == 0) return launch_gemm_dl<T, OutT>(g, stream);
+            return launch_gemm_dl<T, OutT, true>(g, stream);
         }
     }
     // shapes the tile divides exactly take the instance without bounds checks

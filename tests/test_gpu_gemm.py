@@ -219,12 +219,51 @@ def test_half_gemm_large_tile_direct_to_lds_path(be, kind, M, N, K):
         truth = oracle.gemm_f64(aw, bw, M, K, N)
         got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
         assert mixed_err(got32, truth) <= 1e-4
-        # a shape the large tile does not divide is refused rather than mis-computed
+        # a K the kernel's 64-wide K-tile does not divide is refused rather than mis-computed
         from aidotnet.tensors_amd import HipException
         with pytest.raises(HipException):
-            _half_gemm(be, kind, ab[:M * K - K].copy(), bb, M - 1, N, K, True)
+            _half_gemm(be, kind, ab.reshape(M, K)[:, :K - 8].copy(), bb.reshape(K, N)[:K - 8].copy(), M, N, K - 8, True)
     finally:
         be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(257, 264, 64), (300, 520, 128), (1, 8, 64), (255, 248, 192), (511, 1000, 256), (700, 72, 64)])
+def test_half_gemm_large_tile_ragged_edges(be, kind, M, N, K):
+    # the 256 x 256 tile kernel on M and N it does not divide (clamped loads, guarded stores); C is pre-filled so a store
+    # outside the matrix or a missing one shows
+    be.SetGemmTile(256)
+    try:
+        rng = np.random.default_rng(M + 2 * N + 3 * K)
+        a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+        ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+        fn = oracle.hgemm if kind == "f16" else oracle.bf16gemm
+        want16, want32 = fn(ab, bb, M, K, N)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, True), want32)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, False), want16)
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+        assert mixed_err(_half_gemm(be, kind, ab, bb, M, N, K, True), oracle.gemm_f64(aw, bw, M, K, N)) <= 1e-4
+        # guard band: the output buffer has one extra row and the kernel must leave it alone
+        A = be.WrapTensor(from_bits16(ab, TORCH16[kind])); B = be.WrapTensor(from_bits16(bb, TORCH16[kind]))
+        c = torch.full(((M + 1) * N,), -7.0, device="cuda")
+        (be.GemmFp16In32fOut if kind == "f16" else be.GemmBf16In32fOut)(A, B, be.WrapTensor(c), M, N, K)
+        assert bool((c[M * N:] == -7.0).all())
+    finally:
+        be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_half_gemm_ragged_large_shape_takes_the_large_tile(be, kind):
+    # 3000 x 3080 x 512: 156 tiles of 256 x 256, chosen automatically; sampled rows against the float64 truth
+    M, N, K = 3000, 3080, 512
+    rng = np.random.default_rng(7)
+    a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+    ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+    got = _half_gemm(be, kind, ab, bb, M, N, K, True)
+    rows = np.r_[0:4, 255:258, 2815:2818, 2996:3000]
+    truth = aw[rows].astype(np.float64) @ bw.astype(np.float64)
+    assert mixed_err(got[rows], truth) <= 1e-4
 
 
 def test_bf16_literal_known_answer(be):
