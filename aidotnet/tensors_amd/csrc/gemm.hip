@@ -170,8 +170,8 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
             int gm = m0 + row, gk = k0 + ch * E;
             u32x4 v = {0u, 0u, 0u, 0u};
             if ((BM * KC) % NT == 0 || u < BM * KC) {
-                const raw_t* p = A + (long long)gm * g.lda + gk;
-                if constexpr (!CHECK) v = *(const u32x4*)p;
+                const raw_t* p = A + (long long)(CHECK ? gm : min(gm, g.M - 1)) * g.lda + gk;
+                if constexpr (!CHECK) v = *(const u32x4*)p;       // rows past the end repeat the last one (never stored)
                 else if (gm < g.M && gk < g.K) {
                     if constexpr (VEC) v = *(const u32x4*)p;
                     else v = load16_guarded<T>(p, g.K - gk);
@@ -187,7 +187,7 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
                 int gn = n0 + row, gk = k0 + ch * E;
                 u32x4 v = {0u, 0u, 0u, 0u};
                 if ((BN * KC) % NT == 0 || u < BN * KC) {
-                    const raw_t* p = B + (long long)gn * g.ldb + gk;
+                    const raw_t* p = B + (long long)(CHECK ? gn : min(gn, g.N - 1)) * g.ldb + gk;
                     if constexpr (!CHECK) v = *(const u32x4*)p;
                     else if (gn < g.N && gk < g.K) {
                         if constexpr (VEC) v = *(const u32x4*)p;
@@ -221,8 +221,8 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
                                 }
                             }
                         } else {
-                        const raw_t* p = B + (long long)gk * g.ldb + gn;
-                        if constexpr (!CHECK) v = *(const u32x4*)p;
+                        const raw_t* p = B + (long long)gk * g.ldb + (CHECK ? gn : min(gn, g.N - E));
+                        if constexpr (!CHECK) v = *(const u32x4*)p;   // column blocks past the end repeat the last one
                         else if (gk < g.K && gn < g.N) {
                             if constexpr (VEC) v = *(const u32x4*)p;
                             else v = load16_guarded<T>(p, g.N - gn);
@@ -424,11 +424,11 @@ __global__ __launch_bounds__(WM * WN * KS * 64) void gemm_kernel(const GemmArgs 
             for (int j = 0; j < TN; j++) {
                 const int col = n0 + wn * WTN + j * 32 + l32;
                 float bias = 0.0f;
-                if constexpr (FUSED) bias = (g.bias && (!CHECK || col < g.N)) ? g.bias[col] : 0.0f;
+                if constexpr (FUSED) bias = (g.bias && col < g.N) ? g.bias[col] : 0.0f;
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
-                    if (!CHECK || (row < g.M && col < g.N)) {
+                    if (row < g.M && col < g.N) {
                         out_t* p = C + (long long)row * g.ldc + col;
                         float v = g.alpha * acc[i][j][r];
                         if constexpr (Elem<OutT>::BYTES == 4) {
@@ -1036,8 +1036,9 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             return launch_gemm_dl<T, OutT, true>(g, stream);
         }
     }
-    // shapes the tile divides exactly take the instance without bounds checks
-    auto exact = [&](int bt) { return vec && g.M % bt == 0 && g.N % bt == 0 && g.K % (gemm_k_chunks(bt, bt) * E) == 0; };
+    // 16-byte aligned operands whose K the K-tile divides take the instance without bounds checks in its loop (no zero fill
+    // is needed; rows and column blocks past the end are clamped loads whose products are never stored)
+    auto exact = [&](int bt) { return vec && g.N >= E && g.K % (gemm_k_chunks(bt, bt) * E) == 0; };
     if (tile == 128) {
         if (exact(128)) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, false>(g, batch, stream);
         if (vec) return launch_gemm<T, OutT, 128, 128, 2, 2, TRANSB, true, true>(g, batch, stream);

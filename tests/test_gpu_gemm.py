@@ -20,7 +20,9 @@ HALF_TOL = 2e-2
 # Fp16Bf16GemmTests.cs:23-62, SgemmCachedBTests.cs:10-41) plus tile-boundary cases for the 64/128/256 tiles.
 SHAPES = [(1, 1, 1), (7, 13, 11), (96, 130, 80), (37, 53, 71), (13, 10, 17), (4, 32, 8), (16, 24, 20), (3, 5, 7),
           (1, 64, 1), (64, 64, 32), (65, 63, 33), (128, 128, 64), (129, 127, 65), (256, 256, 64), (200, 300, 100),
-          (32, 4096, 128), (8, 512, 1030), (512, 512, 512)]
+          (32, 4096, 128), (8, 512, 1030), (512, 512, 512),
+          # ragged M / N with a K the K-tile divides: the branch-free loop with clamped loads
+          (200, 300, 128), (129, 132, 256), (1000, 1000, 256), (65, 8, 512)]
 
 
 @pytest.fixture(scope="module")
@@ -146,7 +148,7 @@ def test_argument_errors_match_reference_behaviour(be):
 HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7, 13, 11), (96, 130, 80), (37, 53, 71),
                (128, 128, 64), (256, 256, 128), (512, 256, 192), (130, 260, 70), (32, 512, 4096),
                # skinny-M (decode projection) path: M <= 32, N % 128 == 0, K % 64 == 0
-               (1, 128, 64), (5, 256, 192), (17, 384, 1024), (32, 128, 64), (8, 4096, 512)]
+               (1, 128, 64), (5, 256, 192), (17, 384, 1024), (32, 128, 64), (8, 4096, 512), (200, 304, 128), (129, 136, 256), (1000, 1000, 256)]
 
 
 def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
