@@ -31,10 +31,10 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # measured yet.
 TRAFFIC_BYTES = {
     # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes)
-    "gemm_f16_8192": int((792204 * 2.0 + 134918) * 1024),
-    "decode_bf16": int((1048959 * 2.0 + 1088) * 1024),
-    "attn_f16_prefill": int((98762 * 2.0 + 132098) * 1024),
-    "attn_bf16_prefill": int((98443 * 2.0 + 132096) * 1024),
+    "gemm_f16_8192": int((799260 * 2.0 + 139212) * 1024),
+    "decode_bf16": int((1048908 * 2.0 + 1088) * 1024),
+    "attn_f16_prefill": int((98519 * 2.0 + 132099) * 1024),
+    "attn_bf16_prefill": int((98466 * 2.0 + 132097) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
