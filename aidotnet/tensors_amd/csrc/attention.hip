@@ -62,6 +62,40 @@ __device__ __forceinline__ u32x4 ld16(const typename Raw2<T>::type* p, int valid
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+// packed conversions of probabilities and pair sums (shared by both kernels)
+template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
+template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
+{
+    // one packed round-to-nearest-even convert (v_cvt_pk_f16_f32)
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    f2 x = {a, b};
+    h2 v = __builtin_convertvector(x, h2);
+    return __builtin_bit_cast(uint32_t, v);
+}
+// acc + lo + hi of a packed pair (one VALU operation)
+template <typename T> __device__ __forceinline__ float add_pair(uint32_t packed, float acc);
+template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t packed, float acc)
+{
+    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), ones, acc, false);
+}
+template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t packed, float acc)
+{
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    const bf2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, packed), ones, acc, false);
+}
+template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b)
+{
+    // probabilities are finite and non-negative: the hardware round-to-nearest-even convert equals the
+    // integer rule of float_to_bf16_bits on them
+    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+    bf2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
 template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB>
 __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 {
@@ -283,10 +317,13 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     psum += p;
                 }
             l_run = l_run * alpha + psum;
+            // alpha == 1 in every lane (no row maximum moved) is the common case once a few tiles have been seen
+            if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0ull) {
 #pragma unroll
-            for (int i = 0; i < DT; i++)
+                for (int i = 0; i < DT; i++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+                    for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+            }
 
             // ---- O^T += V^T * P^T
 #pragma unroll
@@ -296,8 +333,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     u32x4 pf;
                     if constexpr (E == 8) {
 #pragma unroll
-                        for (int w = 0; w < 4; w++)
-                            pf[w] = Elem<T>::narrow(st[kt][8 * ps + 2 * w]) | (Elem<T>::narrow(st[kt][8 * ps + 2 * w + 1]) << 16);
+                        for (int w = 0; w < 4; w++) pf[w] = pack2_p<T>(st[kt][8 * ps + 2 * w], st[kt][8 * ps + 2 * w + 1]);
                     } else {
 #pragma unroll
                         for (int w = 0; w < 4; w++) pf[w] = as_u32(st[kt][4 * ps + w]);
@@ -379,39 +415,6 @@ __device__ __forceinline__ void attn_dma16(const void* gptr, uint32_t lds_dst)
 __device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
-}
-
-template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
-template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
-{
-    // one packed round-to-nearest-even convert (v_cvt_pk_f16_f32)
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    typedef float f2 __attribute__((ext_vector_type(2)));
-    f2 x = {a, b};
-    h2 v = __builtin_convertvector(x, h2);
-    return __builtin_bit_cast(uint32_t, v);
-}
-// acc + lo + hi of a packed pair (one VALU operation)
-template <typename T> __device__ __forceinline__ float add_pair(uint32_t packed, float acc);
-template <> __device__ __forceinline__ float add_pair<f16_t>(uint32_t packed, float acc)
-{
-    typedef _Float16 h2 __attribute__((ext_vector_type(2)));
-    const h2 ones = {(_Float16)1.0f, (_Float16)1.0f};
-    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, packed), ones, acc, false);
-}
-template <> __device__ __forceinline__ float add_pair<bf16_t>(uint32_t packed, float acc)
-{
-    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-    const bf2 ones = {(__bf16)1.0f, (__bf16)1.0f};
-    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, packed), ones, acc, false);
-}
-template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b)
-{
-    // probabilities are finite and non-negative: the hardware round-to-nearest-even convert equals the
-    // integer rule of float_to_bf16_bits on them
-    typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
-    bf2 v = {(__bf16)a, (__bf16)b};
-    return __builtin_bit_cast(uint32_t, v);
 }
 
 template <typename T, typename OutT>
