@@ -133,6 +133,17 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
+        if (a.causal && nblk <= 768) {
+            // A grid that is resident all at once (at most three workgroups per CU) is not balanced by the order of
+            // dispatch: hand the query tiles out heaviest first across ALL heads, so the workgroups that end up sharing a
+            // CU are a heavy one and, later in the id order, a light one.
+            // (the first 256 ids, one per CU, in ascending weight, so that the ids after them -- which land on the same
+            // CUs in the same order -- pair the lightest of the first round with the heaviest of the second)
+            const int nbh = nblk / a.qtiles;
+            const int rank = (nblk > 256 && pid < 256) ? 255 - pid : pid;
+            qt = a.qtiles - 1 - rank / nbh;
+            bh = rank - (rank / nbh) * nbh;
+        }
     }
     const int b = bh / a.H, hd = bh - b * a.H;
     const int kvh = hd / (a.H / a.Hkv);
@@ -852,7 +863,12 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
         if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
         else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);
     } else
-    if (kind == 0) err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    if (kind == 0) {
+        // fp32: 64-key tiles while two workgroups still fit the LDS of a CU (head dimension up to 64), else 32-key tiles
+        if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
+                                  : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
+        else err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    }
     else if (kind == 1) err = p.out16 ? dispatch_attn_d<f16_t, f16_t, 64>(a, full, stream) : dispatch_attn_d<f16_t, float, 64>(a, full, stream);
     else err = p.out16 ? dispatch_attn_d<bf16_t, bf16_t, 64>(a, full, stream) : dispatch_attn_d<bf16_t, float, 64>(a, full, stream);
     if (err != hipSuccess) return err;
