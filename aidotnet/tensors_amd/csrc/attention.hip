@@ -448,6 +448,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
+        if (a.causal && rem == 0 && per % a.qtiles == 0) {
+            // every XCD owns whole heads: inside an XCD hand out the query tiles heaviest first across its heads
+            const int hx = per / a.qtiles;                    // heads per XCD
+            qt = a.qtiles - 1 - idx / hx;
+            bh = xcd * hx + idx % hx;
+        }
     }
     const int b = bh / a.H, hd = bh - b * a.H;
     const int kvh = hd / (a.H / a.Hkv);
