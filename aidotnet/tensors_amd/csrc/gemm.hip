@@ -9,11 +9,13 @@
 // BFloat16Kernels.cs:144-211): products of the stored values, fp32 accumulation, one
 // round-to-nearest-even narrow at the end for 16-bit outputs.
 //
-// Data movement per workgroup and K-tile (128 bytes of K per row: 64 halves / 32 floats):
-//   global --16 B/lane--> registers --(B[K,N]: E x E register transpose)--> LDS [row][k], 144 B
-//   row pitch (128 + 16 pad: conflict-free ds_read_b128 / ds_write_b128) --> 16-byte MFMA
-//   fragments.  Two LDS stages: the next tile's global loads are issued before the current
-//   tile's MFMAs and stored to the other stage after them; one barrier per K-tile.
+// Data movement per workgroup and K-tile of the general kernel (128 bytes of K per row, 256 for the 64 x 64 tile):
+//   global --16 B/lane--> registers --(B[K,N]: E x E register transpose)--> LDS [row][k], row pitch
+//   = row + 16 bytes of padding (conflict-free ds_read_b128 / ds_write_b128) --> 16-byte MFMA
+//   fragments.  Two LDS stages: the next tile's global loads are issued at the top of an iteration and
+//   stored to the other stage before its last k-step; one barrier per K-tile.
+// The 16-bit 256 x 256 kernel further down loads global -> LDS directly; the skinny (M <= 32, 16-bit) and
+// small-M (M <= 8, fp32) kernels are bandwidth-bound split-K streams of B.
 #include "common.hpp"
 #include "launch.hpp"
 #include <type_traits>
@@ -1009,8 +1011,9 @@ static int choose_tile(long long tiles128, long long tiles64, double rel64)
     return fill(tiles128, 256) >= rel64 * fill(tiles64, 512) ? 128 : 64;
 }
 
-// Tile choice: the largest tile that still gives the 256 CUs roughly a full wave of
-// workgroups; the unchecked 256x256 instance only for shapes it divides exactly.
+// Kernel and tile choice: the 256 x 256 direct-to-LDS kernel for 16-bit B[K,N] problems with at least 128 such tiles,
+// otherwise the general kernel with the 128 x 128 or 64 x 64 tile (choose_tile), in its branch-free instance when the
+// operands are 16-byte aligned and the K-tile divides K.
 template <typename T, typename OutT, bool TRANSB>
 static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream, int force_tile)
 {
