@@ -482,9 +482,17 @@ __device__ __forceinline__ void dma16_base(const void* base_uniform, uint32_t la
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
 }
 
-// EDGE: M and N need not be multiples of 256 (N still a multiple of 8, K of 64): loads of rows / column chunks past the end
-// are redirected to the last valid one (their products land in accumulator elements that are never stored) and the stores
-// are guarded.
+// EDGE: M, N and K need not be multiples of the tile (N and K still multiples of 8): loads of rows / column chunks past the
+// end are redirected to the last valid one (their products land in accumulator elements that are never stored), the stores
+// are guarded, and in the last, partial K-tile every 16-byte chunk at or past K is fetched from a block of zeros instead.
+__device__ __attribute__((aligned(16))) const uint32_t g_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+// direct global -> LDS load with a full per-lane address (the form for lanes that do not share a base)
+__device__ __forceinline__ void dma16_addr(const void* gptr, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_dst), "v"(gptr) : "memory");
+}
+
 template <typename T, typename OutT, bool EDGE = false>
 __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 {
@@ -535,11 +543,32 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda);
     const unsigned char* b_base = (const unsigned char*)(B + (long long)(2 * LB * wave_s) * g.ldb + n0);
     const long long a_step = 8LL * g.lda * 2, b_step = 2LL * g.ldb * 2;        // bytes between consecutive wave-loads
+    const int KT = (g.K + BK - 1) / BK;
+    const int ktail = EDGE ? g.K - (KT - 1) * BK : BK;                        // k-rows of the last tile (BK when K % BK == 0)
     auto issue_loads = [&](int kt, int stage) {
         const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
         const uint32_t bs = lds0 + stage * STAGE + ABYTES + wave_s * (LB * 1024);
         const unsigned char* a_src = a_base + (long long)kt * (BK * 2);
         const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * 2;
+        if constexpr (EDGE) {
+            if (kt == KT - 1 && ktail < BK) {
+                // partial last tile: chunks at or past K come from the zero block (a product with zero adds nothing)
+#pragma unroll
+                for (int i = 0; i < LA; i++) {
+                    const int ra = lane >> 3, pos_a = lane & 7;
+                    const int chunk = pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7);               // the chunk this lane fetches
+                    const void* src = chunk * 8 < ktail ? (const void*)(a_src + a_lane_off[i]) : (const void*)g_zero_chunk;
+                    dma16_addr(src, as + i * 1024);
+                }
+#pragma unroll
+                for (int i = 0; i < LB; i++) {
+                    const int row = 2 * (LB * wave + i) + (lane >> 5);                       // k-row inside the tile
+                    const void* src = row < ktail ? (const void*)(b_src + i * b_step + b_lane_off[i & 1]) : (const void*)g_zero_chunk;
+                    dma16_addr(src, bs + i * 1024);
+                }
+                return;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < LA; i++) {
             if constexpr (EDGE) dma16_base(a_src, a_lane_off[i], as + i * 1024);
@@ -590,7 +619,6 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    const int KT = g.K / BK;
     issue_loads(0, 0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
@@ -1024,18 +1052,18 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     int tile = force_tile;
     if (tile == 0) {
         if constexpr (E == 8 && !TRANSB) {
-            // the 256 x 256 kernel: K a multiple of 64, rows of B in whole 16-byte chunks, leading dimensions within the 32-bit
-            // lane offsets of its loads; M and N may be ragged
-            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldb < (1 << 22) &&
+            // the 256 x 256 kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane offsets
+            // of its loads; M, N and K may be ragged
+            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 22) && g.ldb < (1 << 22) &&
                 tiles(256, 256) >= 128) tile = 256;
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 256) {
-            if (!(vec && g.K % 64 == 0 && g.lda < (1 << 22) && g.ldb < (1 << 22))) return hipErrorInvalidValue;
+            if (!(vec && g.lda < (1 << 22) && g.ldb < (1 << 22))) return hipErrorInvalidValue;
             if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
-            if (g.M % 256 == 0 && g.N % 256 == 0) return launch_gemm_dl<T, OutT>(g, stream);
+            if (g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0) return launch_gemm_dl<T, OutT>(g, stream);
             return launch_gemm_dl<T, OutT, true>(g, stream);
         }
     }

@@ -221,18 +221,19 @@ def test_half_gemm_large_tile_direct_to_lds_path(be, kind, M, N, K):
         truth = oracle.gemm_f64(aw, bw, M, K, N)
         got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
         assert mixed_err(got32, truth) <= 1e-4
-        # a K the kernel's 64-wide K-tile does not divide is refused rather than mis-computed
+        # rows that are not whole 16-byte chunks are outside the kernel's contract: refused rather than mis-computed
         from aidotnet.tensors_amd import HipException
         with pytest.raises(HipException):
-            _half_gemm(be, kind, ab.reshape(M, K)[:, :K - 8].copy(), bb.reshape(K, N)[:K - 8].copy(), M, N, K - 8, True)
+            _half_gemm(be, kind, ab.reshape(M, K)[:, :K - 1].copy(), bb.reshape(K, N)[:K - 1].copy(), M, N, K - 1, True)
     finally:
         be.SetGemmTile(0)
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
-@pytest.mark.parametrize("M,N,K", [(257, 264, 64), (300, 520, 128), (1, 8, 64), (255, 248, 192), (511, 1000, 256), (700, 72, 64)])
+@pytest.mark.parametrize("M,N,K", [(257, 264, 64), (300, 520, 128), (1, 8, 64), (255, 248, 192), (511, 1000, 256), (700, 72, 64),
+                                   (257, 264, 72), (300, 520, 200), (255, 248, 8), (511, 1000, 264), (256, 256, 120)])
 def test_half_gemm_large_tile_ragged_edges(be, kind, M, N, K):
-    # the 256 x 256 tile kernel on M and N it does not divide (clamped loads, guarded stores); C is pre-filled so a store
+    # the 256 x 256 tile kernel on M, N and K it does not divide (clamped loads, zero-filled K tail, guarded stores); C is pre-filled so a store
     # outside the matrix or a missing one shows
     be.SetGemmTile(256)
     try:
