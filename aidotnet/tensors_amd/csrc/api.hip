@@ -183,7 +183,7 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
         if (e != hipSuccess) return hip_status(c, e, "mha: weight gather");
     }
     const int M = (int)rows, N3 = 3 * dModel;
-    const int tile32 = c->force_tile == 256 ? 0 : c->force_tile;
+    const int tile32 = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
     hipError_t e;
     if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)wf, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
     else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)wf, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
@@ -315,7 +315,8 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
-    if (tile != 0 && tile != 64 && tile != 128 && tile != 256) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "tile must be 0, 64, 128 or 256");
+    if (tile != 0 && tile != 64 && tile != 128 && tile != 129 && tile != 256)
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "tile must be 0, 64, 128, 129 (128, direct-to-LDS kernel) or 256");
     c->force_tile = tile;
     return AIDN_OK;
 }
@@ -347,7 +348,7 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
-    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    int tile = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
     void* ws = nullptr;
     if (int st = smallm_ws(c, M, N, K, transB, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),
@@ -363,7 +364,7 @@ AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, c
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: dimensions must be positive");
     if (batch <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: batch count must be positive");
     if (batch > 65535) return fail(c, AIDN_ERR_UNSUPPORTED, "sgemm_batched: more than 65535 batches");
-    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    int tile = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, 0, batch,
                                         (long long)M * K, (long long)K * N, (long long)M * N, tile), "gemm_f32 (batched)");
 }
@@ -376,7 +377,7 @@ AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, 
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: unknown activation");
-    int tile = c->force_tile == 256 ? 0 : c->force_tile;
+    int tile = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
     void* ws = nullptr;
     if (int st = smallm_ws(c, M, N, K, 0, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param, ws),

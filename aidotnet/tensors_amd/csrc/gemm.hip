@@ -493,16 +493,21 @@ __device__ __forceinline__ void dma16_addr(const void* gptr, uint32_t lds_dst)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_dst), "v"(gptr) : "memory");
 }
 
-template <typename T, typename OutT, bool EDGE = false>
-__global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
+// TILE = 256: 8 waves (2 x 4), wave tile 128 x 64, one workgroup per CU.  TILE = 128: 4 waves (2 x 2), wave tile 64 x 64, two
+// workgroups per CU (for problems with too few 256 x 256 tiles to occupy the chip).
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
+__global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
     typedef uint16_t raw_t;
-    constexpr int WM = 2, WN = 4;
-    constexpr int BM = 256, BN = 256, BK = 64;
+    constexpr int WM = 2, WN = TILE == 256 ? 4 : 2;
+    constexpr int BM = TILE, BN = TILE, BK = 64;
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int ABYTES = BM * 128, BBYTES = BK * 512, STAGE = ABYTES + BBYTES;
-    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (32 + 32 per workgroup)
+    constexpr int BROW = BN * 2;                  // bytes of one k-row of the B tile
+    constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
+    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (both tile sizes: 32 + 32 resp. 16 + 16 per workgroup)
+    constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load (2 resp. 4)
+    constexpr int LPR = 64 / RPL;                 // lanes (16-byte chunks) per B row
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -518,7 +523,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
 
     // Sources of this wave's loads: a wave-uniform base (scalar registers, advanced per tile by scalar adds) plus a per-lane
     // 32-bit byte offset that never changes, so issuing a load costs no vector instruction.  Wave-load w = 4 wave + i covers
-    // A rows 8w .. 8w+7 resp. B k-rows 2w, 2w+1; the swizzle of a lane depends on w only through its parity, i.e. on i & 1.
+    // A rows 8w .. 8w+7 resp. B k-rows RPL w .. RPL w + RPL-1; the swizzle of a lane depends on w only through its parity, i.e.
+    // on i & 1.
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     uint32_t a_lane_off[EDGE ? LA : 2], b_lane_off[2];
@@ -526,8 +532,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     for (int par = 0; par < 2; par++) {
         const int ra = lane >> 3, pos_a = lane & 7;           // row inside the wave-load, 16-byte chunk
         if constexpr (!EDGE) a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * 8) * 2u;
-        const int rb = lane >> 5, pos_b = lane & 31;
-        int chunk = pos_b ^ (((2 * par + rb) & 3) << 2);
+        const int rb = lane / LPR, pos_b = lane % LPR;
+        int chunk = pos_b ^ (((RPL * par + rb) & 3) << 2);
         if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / 8 - 1);          // N % 8 == 0 and n0 < N: at least one chunk
         b_lane_off[par] = (uint32_t)(rb * g.ldb + chunk * 8) * 2u;
     }
@@ -541,8 +547,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
     }
     // (EDGE: the A offsets are relative to the tile's first row, since a clamped row may lie before the wave's own rows)
     const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda);
-    const unsigned char* b_base = (const unsigned char*)(B + (long long)(2 * LB * wave_s) * g.ldb + n0);
-    const long long a_step = 8LL * g.lda * 2, b_step = 2LL * g.ldb * 2;        // bytes between consecutive wave-loads
+    const unsigned char* b_base = (const unsigned char*)(B + (long long)(RPL * LB * wave_s) * g.ldb + n0);
+    const long long a_step = 8LL * g.lda * 2, b_step = (long long)RPL * g.ldb * 2;   // bytes between consecutive wave-loads
     const int KT = (g.K + BK - 1) / BK;
     const int ktail = EDGE ? g.K - (KT - 1) * BK : BK;                        // k-rows of the last tile (BK when K % BK == 0)
     auto issue_loads = [&](int kt, int stage) {
@@ -562,7 +568,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
                 }
 #pragma unroll
                 for (int i = 0; i < LB; i++) {
-                    const int row = 2 * (LB * wave + i) + (lane >> 5);                       // k-row inside the tile
+                    const int row = RPL * (LB * wave + i) + lane / LPR;                      // k-row inside the tile
                     const void* src = row < ktail ? (const void*)(b_src + i * b_step + b_lane_off[i & 1]) : (const void*)g_zero_chunk;
                     dma16_addr(src, bs + i * 1024);
                 }
@@ -603,7 +609,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
                 int row = 16 * s + 4 * q + b_rowl;
                 int pos = b_chunk[j] ^ ((row & 3) << 2);
                 s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(bs + row * 512 + pos * 16 + b_half));
+                    (__attribute__((address_space(3))) s16x4*)(bs + row * BROW + pos * 16 + b_half));
                 u32x2 w = __builtin_bit_cast(u32x2, v);
                 fb[j][2 * q] = w[0];
                 fb[j][2 * q + 1] = w[1];
@@ -684,20 +690,20 @@ __global__ __launch_bounds__(512, 1) void gemm_dl_kernel(const GemmArgs g)
         }
 }
 
-template <typename T, typename OutT, bool EDGE = false>
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
 static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
 {
-    auto kern = gemm_dl_kernel<T, OutT, EDGE>;
-    constexpr int smem = 2 * (256 * 128 + 64 * 512);
+    auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE>;
+    constexpr int smem = 2 * (TILE * 128 + 64 * TILE * 2);
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    g.tiles_m = (g.M + 255) / 256;
-    g.tiles_n = (g.N + 255) / 256;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(512), smem, stream, g);
+    g.tiles_m = (g.M + TILE - 1) / TILE;
+    g.tiles_n = (g.N + TILE - 1) / TILE;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(TILE == 256 ? 512 : 256), smem, stream, g);
     return hipGetLastError();
 }
 
@@ -1054,19 +1060,24 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         if constexpr (E == 8 && !TRANSB) {
             // the 256 x 256 kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane offsets
             // of its loads; M, N and K may be ragged
-            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 22) && g.ldb < (1 << 22) &&
-                tiles(256, 256) >= 128) tile = 256;
+            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 22) && g.ldb < (1 << 22)) {
+                if (tiles(256, 256) >= 128) tile = 256;
+                else if (tiles(128, 128) >= 128) tile = 129;          // the same kernel with 128 x 128 tiles, two workgroups per CU
+            }
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
     if constexpr (E == 8 && !TRANSB) {
-        if (tile == 256) {
+        if (tile == 256 || tile == 129) {
             if (!(vec && g.lda < (1 << 22) && g.ldb < (1 << 22))) return hipErrorInvalidValue;
             if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
-            if (g.M % 256 == 0 && g.N % 256 == 0 && g.K % 64 == 0) return launch_gemm_dl<T, OutT>(g, stream);
-            return launch_gemm_dl<T, OutT, true>(g, stream);
+            const int edge = tile == 256 ? 256 : 128;
+            const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % 64 == 0;
+            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256>(g, stream) : launch_gemm_dl<T, OutT, true, 256>(g, stream);
+            return exact_fit ? launch_gemm_dl<T, OutT, false, 128>(g, stream) : launch_gemm_dl<T, OutT, true, 128>(g, stream);
         }
     }
+    if (tile == 129) tile = 128;
     // 16-byte aligned operands whose K the K-tile divides take the instance without bounds checks in its loop (no zero fill
     // is needed; rows and column blocks past the end are clamped loads whose products are never stored)
     auto exact = [&](int bt) { return vec && g.N >= E && g.K % (gemm_k_chunks(bt, bt) * E) == 0; };
