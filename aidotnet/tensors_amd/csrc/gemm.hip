@@ -498,16 +498,17 @@ __device__ __forceinline__ void dma16_addr(const void* gptr, uint32_t lds_dst)
 template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
 __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
-    typedef uint16_t raw_t;
+    constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     constexpr int WM = 2, WN = TILE == 256 ? 4 : 2;
-    constexpr int BM = TILE, BN = TILE, BK = 64;
+    constexpr int BM = TILE, BN = TILE, BK = 128 / EB;          // 128 bytes of K per tile row: 64 halves / 32 floats
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int BROW = BN * 2;                  // bytes of one k-row of the B tile
+    constexpr int BROW = BN * EB;                 // bytes of one k-row of the B tile
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
-    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (both tile sizes: 32 + 32 resp. 16 + 16 per workgroup)
-    constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load (2 resp. 4)
+    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (every instance: 32 + 32 resp. 16 + 16 per workgroup)
+    constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load
     constexpr int LPR = 64 / RPL;                 // lanes (16-byte chunks) per B row
+    static_assert(BK * BROW / 1024 == LB * WM * WN, "B tile = four wave-loads per wave");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -518,44 +519,51 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const raw_t* __restrict__ A = (const raw_t*)g.A;
-    const raw_t* __restrict__ B = (const raw_t*)g.B;
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B;
+
+    // Chunk swizzle of the B tile (which 16-byte chunk position of its LDS row a chunk of k-row `row` occupies):
+    //   16-bit: c ^ ((row & 3) << 2)  -- the four rows one transposing read touches go to different bank groups;
+    //   fp32:   c ^ (((row >> 2) & 1) << 3)  -- the two lane halves of a b32 fragment read (rows 4 apart) use different bank halves.
+    auto b_swz = [](int row) -> int { return E == 8 ? ((row & 3) << 2) : (((row >> 2) & 1) << 3); };
 
     // Sources of this wave's loads: a wave-uniform base (scalar registers, advanced per tile by scalar adds) plus a per-lane
     // 32-bit byte offset that never changes, so issuing a load costs no vector instruction.  Wave-load w = 4 wave + i covers
-    // A rows 8w .. 8w+7 resp. B k-rows RPL w .. RPL w + RPL-1; the swizzle of a lane depends on w only through its parity, i.e.
-    // on i & 1.
+    // A rows 8w .. 8w+7 resp. B k-rows RPL w .. RPL w + RPL-1.
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
-    uint32_t a_lane_off[EDGE ? LA : 2], b_lane_off[2];
+    uint32_t a_lane_off[EDGE ? LA : 2], b_lane_off[LB];
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         const int ra = lane >> 3, pos_a = lane & 7;           // row inside the wave-load, 16-byte chunk
-        if constexpr (!EDGE) a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * 8) * 2u;
+        if constexpr (!EDGE) a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
         const int rb = lane / LPR, pos_b = lane % LPR;
-        int chunk = pos_b ^ (((RPL * par + rb) & 3) << 2);
-        if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / 8 - 1);          // N % 8 == 0 and n0 < N: at least one chunk
-        b_lane_off[par] = (uint32_t)(rb * g.ldb + chunk * 8) * 2u;
+        int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
+        if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / E - 1);          // N % E == 0 and n0 < N: at least one chunk
+        b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
     }
     if constexpr (EDGE) {
 #pragma unroll
         for (int i = 0; i < LA; i++) {
             const int ra = lane >> 3, pos_a = lane & 7;
             const int row = min(8 * (LA * wave + i) + ra, g.M - 1 - m0);      // source row inside the tile (m0 < M)
-            a_lane_off[i] = (uint32_t)(row * g.lda + (pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7)) * 8) * 2u;
+            a_lane_off[i] = (uint32_t)(row * g.lda + (pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
         }
     }
     // (EDGE: the A offsets are relative to the tile's first row, since a clamped row may lie before the wave's own rows)
-    const unsigned char* a_base = (const unsigned char*)(A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda);
-    const unsigned char* b_base = (const unsigned char*)(B + (long long)(RPL * LB * wave_s) * g.ldb + n0);
-    const long long a_step = 8LL * g.lda * 2, b_step = (long long)RPL * g.ldb * 2;   // bytes between consecutive wave-loads
+    const unsigned char* a_base = A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda * EB;
+    const unsigned char* b_base = B + ((long long)(RPL * LB * wave_s) * g.ldb + n0) * EB;
+    const long long a_step = 8LL * g.lda * EB, b_step = (long long)RPL * g.ldb * EB;   // bytes between consecutive wave-loads
     const int KT = (g.K + BK - 1) / BK;
     const int ktail = EDGE ? g.K - (KT - 1) * BK : BK;                        // k-rows of the last tile (BK when K % BK == 0)
     auto issue_loads = [&](int kt, int stage) {
         const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
         const uint32_t bs = lds0 + stage * STAGE + ABYTES + wave_s * (LB * 1024);
-        const unsigned char* a_src = a_base + (long long)kt * (BK * 2);
-        const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * 2;
+        const unsigned char* a_src = a_base + (long long)kt * 128;
+        const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * EB;
         if constexpr (EDGE) {
             if (kt == KT - 1 && ktail < BK) {
                 // partial last tile: chunks at or past K come from the zero block (a product with zero adds nothing)
@@ -563,13 +571,13 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
                 for (int i = 0; i < LA; i++) {
                     const int ra = lane >> 3, pos_a = lane & 7;
                     const int chunk = pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7);               // the chunk this lane fetches
-                    const void* src = chunk * 8 < ktail ? (const void*)(a_src + a_lane_off[i]) : (const void*)g_zero_chunk;
+                    const void* src = chunk * E < ktail ? (const void*)(a_src + a_lane_off[i]) : (const void*)g_zero_chunk;
                     dma16_addr(src, as + i * 1024);
                 }
 #pragma unroll
                 for (int i = 0; i < LB; i++) {
                     const int row = RPL * (LB * wave + i) + lane / LPR;                      // k-row inside the tile
-                    const void* src = row < ktail ? (const void*)(b_src + i * b_step + b_lane_off[i & 1]) : (const void*)g_zero_chunk;
+                    const void* src = row < ktail ? (const void*)(b_src + i * b_step + b_lane_off[i]) : (const void*)g_zero_chunk;
                     dma16_addr(src, bs + i * 1024);
                 }
                 return;
@@ -581,7 +589,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
             else dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
         }
 #pragma unroll
-        for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i & 1], bs + i * 1024);
+        for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i], bs + i * 1024);
     };
 
     // per-lane LDS read offsets
@@ -592,27 +600,40 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         a_off[i] = row * 128;
         a_sw[i] = (row >> 1) & 7;
     }
+    // 16-bit B fragments (transposing reads): lane j of a 16-lane group addresses k-row (base + j / 4), 8 bytes
     const int jl = lane & 15;
     const int b_rowl = 8 * h + (jl >> 2);                     // + 16 s + 4 q
     const int b_half = (jl & 1) * 8;
     int b_chunk[TN];
 #pragma unroll
     for (int j = 0; j < TN; j++) b_chunk[j] = (wn * WTN + j * 32 + 16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;
+    // fp32 B fragments (b32 reads): lane (h, l32) reads column l32 of k-rows 8 s + 4 h + (0..3); (row >> 2) & 1 == h there
+    int b_col32[TN];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int col = wn * WTN + j * 32 + l32;
+        b_col32[j] = (((col >> 2) ^ (h << 3)) << 4) + (col & 3) * 4 + 4 * h * BROW;
+    }
 
     auto read_frags = [&](const unsigned char* as, const unsigned char* bs, int s, u32x4 (&fa)[TM], u32x4 (&fb)[TN]) {
 #pragma unroll
         for (int i = 0; i < TM; i++) fa[i] = *(const u32x4*)(as + a_off[i] + (((2 * s + h) ^ a_sw[i]) << 4));
 #pragma unroll
         for (int j = 0; j < TN; j++) {
+            if constexpr (E == 4) {
 #pragma unroll
-            for (int q = 0; q < 2; q++) {
-                int row = 16 * s + 4 * q + b_rowl;
-                int pos = b_chunk[j] ^ ((row & 3) << 2);
-                s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (__attribute__((address_space(3))) s16x4*)(bs + row * BROW + pos * 16 + b_half));
-                u32x2 w = __builtin_bit_cast(u32x2, v);
-                fb[j][2 * q] = w[0];
-                fb[j][2 * q + 1] = w[1];
+                for (int q = 0; q < 4; q++) fb[j][q] = *(const uint32_t*)(bs + (8 * s + q) * BROW + b_col32[j]);
+            } else {
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    int row = 16 * s + 4 * q + b_rowl;
+                    int pos = b_chunk[j] ^ ((row & 3) << 2);
+                    s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                        (__attribute__((address_space(3))) s16x4*)(bs + row * BROW + pos * 16 + b_half));
+                    u32x2 w = __builtin_bit_cast(u32x2, v);
+                    fb[j][2 * q] = w[0];
+                    fb[j][2 * q + 1] = w[1];
+                }
             }
         }
     };
@@ -659,8 +680,9 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
                 for (int j = 0; j < TN; j++) Mma32<T>::run(acc[i][j], fa[s & 1][i], fb[s & 1][j]);
             // the next step's fragment reads go behind the first half of this step's MFMAs (two each), so the matrix pipe does
             // not wait behind a burst of reads and the last read still has half a step to complete
-            spread_schedule<TM * TN / 2, TM + 2 * TN, 0, 0>();
-            __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM * TN / 2, 0);
+            constexpr int NMF = TM * TN * (E == 4 ? 4 : 1);             // MFMA instructions per step
+            spread_schedule<NMF / 2, TM + (E == 4 ? 4 : 2) * TN, 0, 0>();
+            __builtin_amdgcn_sched_group_barrier(0x008, NMF - NMF / 2, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -694,7 +716,7 @@ template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
 static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
 {
     auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE>;
-    constexpr int smem = 2 * (TILE * 128 + 64 * TILE * 2);
+    constexpr int smem = 2 * (TILE * 128 + 128 * TILE);         // A tile + B tile (128 bytes of K each), two stages
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -1035,14 +1057,15 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
-// 128 x 128 or 64 x 64 tile, by how evenly the workgroups load the 256 CUs (a CU works through 128 x 128 tiles at about
-// the same rate whether it holds one or two, so rounds of 256; two 64 x 64 tiles at a time, so rounds of 512); rel64 =
-// efficiency per flop of the smaller tile relative to the larger one when both fill their rounds equally well (measured:
-// about 0.85 for fp32, 0.55 for the 16-bit types).
+// How evenly `tiles` workgroups load the 256 CUs: a CU works through its tiles at about the same rate whether it holds one or
+// several at a time, so what counts is the largest number of tiles any CU gets.
+static double cu_fill(long long tiles) { return (double)tiles / (double)(((tiles + 255) / 256) * 256); }
+
+// 128 x 128 or 64 x 64 tile; rel64 = efficiency per flop of the smaller tile relative to the larger one when both load the
+// CUs equally well (measured: about 0.85 for fp32, 0.55 for the 16-bit types).
 static int choose_tile(long long tiles128, long long tiles64, double rel64)
 {
-    auto fill = [](long long t, long long slots) { return (double)t / (double)(((t + slots - 1) / slots) * slots); };
-    return fill(tiles128, 256) >= rel64 * fill(tiles64, 512) ? 128 : 64;
+    return cu_fill(tiles128) >= rel64 * cu_fill(tiles64) ? 128 : 64;
 }
 
 // Kernel and tile choice: the 256 x 256 direct-to-LDS kernel for 16-bit B[K,N] problems with at least 128 such tiles,
@@ -1057,22 +1080,26 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     auto tiles = [&](int bm, int bn) { return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * batch; };
     int tile = force_tile;
     if (tile == 0) {
-        if constexpr (E == 8 && !TRANSB) {
-            // the 256 x 256 kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane offsets
-            // of its loads; M, N and K may be ragged
-            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 22) && g.ldb < (1 << 22)) {
-                if (tiles(256, 256) >= 128) tile = 256;
-                else if (tiles(128, 128) >= 128) tile = 129;          // the same kernel with 128 x 128 tiles, two workgroups per CU
+        if constexpr (!TRANSB) {
+            // the direct-to-LDS kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane
+            // offsets of its loads; M, N and K may be ragged
+            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 21) && g.ldb < (1 << 21)) {
+                // 16-bit: the 256 x 256 tile moves half the bytes per flop of the 128 x 128 one and wins from half a chip of
+                // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
+                const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
+                const bool big = E == 8 ? t256 >= 128 : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
+                if (big) tile = 256;
+                else if (t128 >= 128 && choose_tile(t128, tiles(64, 64), E == 4 ? 0.85 : 0.55) == 128) tile = 129;   // same kernel, 128 x 128 tiles
             }
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
-    if constexpr (E == 8 && !TRANSB) {
+    if constexpr (!TRANSB) {
         if (tile == 256 || tile == 129) {
-            if (!(vec && g.lda < (1 << 22) && g.ldb < (1 << 22))) return hipErrorInvalidValue;
+            if (!(vec && g.N >= E && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
-            const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % 64 == 0;
+            const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
             if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256>(g, stream) : launch_gemm_dl<T, OutT, true, 256>(g, stream);
             return exact_fit ? launch_gemm_dl<T, OutT, false, 128>(g, stream) : launch_gemm_dl<T, OutT, true, 128>(g, stream);
         }

@@ -380,3 +380,28 @@ def test_conversions_bit_exact(be, n):
     assert np.array_equal(back_b.cpu().numpy().view(np.uint32), oracle.bf16_to_f32(got_b).view(np.uint32))
     ok = ~np.isnan(oracle.f16_to_f32(got_h))
     assert np.array_equal(back_h.cpu().numpy()[ok], oracle.f16_to_f32(got_h)[ok])
+
+
+# ---------------------------------------------------------------- fp32 on the direct global->LDS kernel
+@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 256, 128), (512, 256, 96), (768, 1024, 160), (256, 512, 2048),
+                                   (257, 260, 32), (300, 516, 100), (1, 4, 32), (255, 248, 4), (511, 1000, 132), (700, 36, 36)])
+def test_fp32_gemm_direct_to_lds_path(be, tile, M, N, K):
+    # exact on dyadic inputs (every summation order is exact), 1e-4 against the float64 truth otherwise; ragged M, N, K
+    be.SetGemmTile(tile)
+    try:
+        rng = np.random.default_rng(M + 2 * N + 3 * K + tile)
+        a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+        assert np.array_equal(_gemm(be, a, b, M, N, K).astype(np.float64), a.astype(np.float64) @ b.astype(np.float64))
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        got = _gemm(be, a, b, M, N, K)
+        assert mixed_err(got, oracle.gemm_f64(a, b, M, K, N)) <= FP32_TOL
+        if M * N * K <= 1 << 24:
+            assert mixed_err(got, oracle.sgemm(a, b, M, K, N)) <= FP32_TOL
+        # guard band: one extra row of C must stay untouched
+        c = torch.full(((M + 1) * N,), -7.0, device="cuda")
+        be.Gemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), M, N, K, 1.0, 0.0)
+        assert bool((c[M * N:] == -7.0).all())
+        assert mixed_err(c[:M * N].cpu().numpy().reshape(M, N), oracle.gemm_f64(a, b, M, K, N)) <= FP32_TOL
+    finally:
+        be.SetGemmTile(0)

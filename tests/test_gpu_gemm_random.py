@@ -61,6 +61,22 @@ def test_random_fp32_gemm(be, tile):
         be.SetGemmTile(0)
 
 
+@pytest.mark.parametrize("tile", [256, 129])
+def test_random_fp32_gemm_direct_kernel(be, tile):
+    be.SetGemmTile(tile)
+    try:
+        rng = np.random.default_rng(300 + tile)
+        for (m, n, k) in shapes(70 + tile, 40):
+            if n % 4 or k % 4:
+                continue                                     # rows must be whole 16-byte chunks for this kernel
+            a = rng.uniform(-1, 1, (m, k)).astype(np.float32); b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+            c = torch.full((m, n), float("nan"), device="cuda")
+            be.Gemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), m, n, k, 1.0, 0.0)
+            assert mixed_err(c.cpu().numpy(), a.astype(np.float64) @ b.astype(np.float64)) <= 1e-4, (tile, m, n, k)
+    finally:
+        be.SetGemmTile(0)
+
+
 def test_random_fp32_batched_gemm(be):
     rng = np.random.default_rng(5)
     for (m, n, k) in shapes(9, 12):
