@@ -348,8 +348,7 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
-    // the direct-to-LDS instances (256, 129) exist for B stored [K,N] only
-    int tile = ((c->force_tile == 256 || c->force_tile == 129) && transB) ? 0 : c->force_tile;
+    int tile = c->force_tile;
     void* ws = nullptr;
     if (int st = smallm_ws(c, M, N, K, transB, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),

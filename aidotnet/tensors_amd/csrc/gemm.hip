@@ -495,7 +495,8 @@ __device__ __forceinline__ void dma16_addr(const void* gptr, uint32_t lds_dst)
 
 // TILE = 256: 8 waves (2 x 4), wave tile 128 x 64, one workgroup per CU.  TILE = 128: 4 waves (2 x 2), wave tile 64 x 64, two
 // workgroups per CU (for problems with too few 256 x 256 tiles to occupy the chip).
-template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
+// TRANSB: B is stored [N,K]; its tile is then loaded and read exactly like the A tile (rows of 128 bytes of K, b128 fragments).
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false>
 __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
@@ -508,7 +509,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (every instance: 32 + 32 resp. 16 + 16 per workgroup)
     constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load
     constexpr int LPR = 64 / RPL;                 // lanes (16-byte chunks) per B row
-    static_assert(BK * BROW / 1024 == LB * WM * WN, "B tile = four wave-loads per wave");
+    static_assert(BK * BROW / 1024 == LB * WM * WN && BN / 8 == LB * WM * WN, "B tile = four wave-loads per wave");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -540,10 +541,19 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
-        const int rb = lane / LPR, pos_b = lane % LPR;
-        int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
-        if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / E - 1);          // N % E == 0 and n0 < N: at least one chunk
-        b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
+        if constexpr (TRANSB) {
+            const int rn = lane >> 3, pos = lane & 7;             // like A: wave-load w covers tile rows (n) 8w .. 8w+7
+            int row = 8 * (LB * wave + i) + rn;
+            const int sw = (row >> 1) & 7;
+            if constexpr (EDGE) row = min(row, g.N - 1 - n0);
+            else row = rn;                                        // relative to the wave-load's first row (scalar base)
+            b_lane_off[i] = (uint32_t)(row * g.ldb + (pos ^ sw) * E) * (uint32_t)EB;
+        } else {
+            const int rb = lane / LPR, pos_b = lane % LPR;
+            int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
+            if constexpr (EDGE) chunk = min(chunk, (g.N - n0) / E - 1);      // N % E == 0 and n0 < N: at least one chunk
+            b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
+        }
     }
     if constexpr (EDGE) {
 #pragma unroll
@@ -555,15 +565,17 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     }
     // (EDGE: the A offsets are relative to the tile's first row, since a clamped row may lie before the wave's own rows)
     const unsigned char* a_base = A + (long long)(m0 + (EDGE ? 0 : 8 * LA * wave_s)) * g.lda * EB;
-    const unsigned char* b_base = B + ((long long)(RPL * LB * wave_s) * g.ldb + n0) * EB;
-    const long long a_step = 8LL * g.lda * EB, b_step = (long long)RPL * g.ldb * EB;   // bytes between consecutive wave-loads
+    const unsigned char* b_base = TRANSB ? B + (long long)(n0 + (EDGE ? 0 : 8 * LB * wave_s)) * g.ldb * EB
+                                         : B + ((long long)(RPL * LB * wave_s) * g.ldb + n0) * EB;
+    // bytes between consecutive wave-loads
+    const long long a_step = 8LL * g.lda * EB, b_step = TRANSB ? (EDGE ? 0LL : 8LL * g.ldb * EB) : (long long)RPL * g.ldb * EB;
     const int KT = (g.K + BK - 1) / BK;
     const int ktail = EDGE ? g.K - (KT - 1) * BK : BK;                        // k-rows of the last tile (BK when K % BK == 0)
     auto issue_loads = [&](int kt, int stage) {
         const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
         const uint32_t bs = lds0 + stage * STAGE + ABYTES + wave_s * (LB * 1024);
         const unsigned char* a_src = a_base + (long long)kt * 128;
-        const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * EB;
+        const unsigned char* b_src = TRANSB ? b_base + (long long)kt * 128 : b_base + (long long)kt * BK * g.ldb * EB;
         if constexpr (EDGE) {
             if (kt == KT - 1 && ktail < BK) {
                 // partial last tile: chunks at or past K come from the zero block (a product with zero adds nothing)
@@ -576,8 +588,14 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
                 }
 #pragma unroll
                 for (int i = 0; i < LB; i++) {
-                    const int row = RPL * (LB * wave + i) + lane / LPR;                      // k-row inside the tile
-                    const void* src = row < ktail ? (const void*)(b_src + i * b_step + b_lane_off[i]) : (const void*)g_zero_chunk;
+                    bool valid;
+                    if constexpr (TRANSB) {
+                        const int rn = lane >> 3, pos = lane & 7;
+                        valid = (pos ^ (((8 * (LB * wave + i) + rn) >> 1) & 7)) * E < ktail;  // the chunk of K this lane fetches
+                    } else {
+                        valid = RPL * (LB * wave + i) + lane / LPR < ktail;                  // k-row inside the tile
+                    }
+                    const void* src = valid ? (const void*)(b_src + i * b_step + b_lane_off[i]) : (const void*)g_zero_chunk;
                     dma16_addr(src, bs + i * 1024);
                 }
                 return;
@@ -615,12 +633,22 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         b_col32[j] = (((col >> 2) ^ (h << 3)) << 4) + (col & 3) * 4 + 4 * h * BROW;
     }
 
+    int bt_off[TN], bt_sw[TN];                               // B stored [N,K]: like the A fragments
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        int row = wn * WTN + j * 32 + l32;
+        bt_off[j] = row * 128;
+        bt_sw[j] = (row >> 1) & 7;
+    }
+
     auto read_frags = [&](const unsigned char* as, const unsigned char* bs, int s, u32x4 (&fa)[TM], u32x4 (&fb)[TN]) {
 #pragma unroll
         for (int i = 0; i < TM; i++) fa[i] = *(const u32x4*)(as + a_off[i] + (((2 * s + h) ^ a_sw[i]) << 4));
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            if constexpr (E == 4) {
+            if constexpr (TRANSB) {
+                fb[j] = *(const u32x4*)(bs + bt_off[j] + (((2 * s + h) ^ bt_sw[j]) << 4));
+            } else if constexpr (E == 4) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) fb[j][q] = *(const uint32_t*)(bs + (8 * s + q) * BROW + b_col32[j]);
             } else {
@@ -681,7 +709,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
             // the next step's fragment reads go behind the first half of this step's MFMAs (two each), so the matrix pipe does
             // not wait behind a burst of reads and the last read still has half a step to complete
             constexpr int NMF = TM * TN * (E == 4 ? 4 : 1);             // MFMA instructions per step
-            spread_schedule<NMF / 2, TM + (E == 4 ? 4 : 2) * TN, 0, 0>();
+            spread_schedule<NMF / 2, TM + (TRANSB ? 1 : E == 4 ? 4 : 2) * TN, 0, 0>();
             __builtin_amdgcn_sched_group_barrier(0x008, NMF - NMF / 2, 0);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -712,10 +740,10 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         }
 }
 
-template <typename T, typename OutT, bool EDGE = false, int TILE = 256>
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false>
 static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
 {
-    auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE>;
+    auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE, TRANSB>;
     constexpr int smem = 2 * (TILE * 128 + 128 * TILE);         // A tile + B tile (128 bytes of K each), two stages
     static bool attr_set = false;
     if (!attr_set) {
@@ -1080,7 +1108,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     auto tiles = [&](int bm, int bn) { return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * batch; };
     int tile = force_tile;
     if (tile == 0) {
-        if constexpr (!TRANSB) {
+        if constexpr (!TRANSB || E == 4) {
             // the direct-to-LDS kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane
             // offsets of its loads; M, N and K may be ragged
             if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 21) && g.ldb < (1 << 21)) {
@@ -1094,14 +1122,14 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
-    if constexpr (!TRANSB) {
+    if constexpr (!TRANSB || E == 4) {
         if (tile == 256 || tile == 129) {
-            if (!(vec && g.N >= E && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
+            if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
             const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
-            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256>(g, stream) : launch_gemm_dl<T, OutT, true, 256>(g, stream);
-            return exact_fit ? launch_gemm_dl<T, OutT, false, 128>(g, stream) : launch_gemm_dl<T, OutT, true, 128>(g, stream);
+            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, stream) : launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, stream);
+            return exact_fit ? launch_gemm_dl<T, OutT, false, 128, TRANSB>(g, stream) : launch_gemm_dl<T, OutT, true, 128, TRANSB>(g, stream);
         }
     }
     if (tile == 129) tile = 128;

@@ -403,5 +403,17 @@ def test_fp32_gemm_direct_to_lds_path(be, tile, M, N, K):
         be.Gemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), M, N, K, 1.0, 0.0)
         assert bool((c[M * N:] == -7.0).all())
         assert mixed_err(c[:M * N].cpu().numpy().reshape(M, N), oracle.gemm_f64(a, b, M, K, N)) <= FP32_TOL
+        # B stored [N, K] (MatMulTransposed) on the same kernel; here N need not be a multiple of 4
+        bt = np.ascontiguousarray(b.T)
+        c = torch.full(((M + 1) * N,), -7.0, device="cuda")
+        be.MatMulTransposed(be.WrapTensor(dev(a)), be.WrapTensor(dev(bt)), be.WrapTensor(c), M, N, K, 1.0, 0.0)
+        assert bool((c[M * N:] == -7.0).all())
+        assert mixed_err(c[:M * N].cpu().numpy().reshape(M, N), oracle.gemm_f64(a, b, M, K, N)) <= FP32_TOL
+        if N > 3:
+            n2 = N - 3                                   # ragged, odd N
+            c = torch.full(((M + 1) * n2,), -7.0, device="cuda")
+            be.MatMulTransposed(be.WrapTensor(dev(a)), be.WrapTensor(dev(np.ascontiguousarray(bt[:n2]))), be.WrapTensor(c), M, n2, K, 1.0, 0.0)
+            assert bool((c[M * n2:] == -7.0).all())
+            assert mixed_err(c[:M * n2].cpu().numpy().reshape(M, n2), oracle.gemm_f64(a, np.ascontiguousarray(b[:, :n2]), M, K, n2)) <= FP32_TOL
     finally:
         be.SetGemmTile(0)

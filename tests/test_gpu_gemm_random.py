@@ -73,6 +73,9 @@ def test_random_fp32_gemm_direct_kernel(be, tile):
             c = torch.full((m, n), float("nan"), device="cuda")
             be.Gemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), m, n, k, 1.0, 0.0)
             assert mixed_err(c.cpu().numpy(), a.astype(np.float64) @ b.astype(np.float64)) <= 1e-4, (tile, m, n, k)
+            c = torch.full((m, n), float("nan"), device="cuda")
+            be.MatMulTransposed(be.WrapTensor(dev(a)), be.WrapTensor(dev(np.ascontiguousarray(b.T))), be.WrapTensor(c), m, n, k, 1.0, 0.0)
+            assert mixed_err(c.cpu().numpy(), a.astype(np.float64) @ b.astype(np.float64)) <= 1e-4, ("transposed", tile, m, n, k)
     finally:
         be.SetGemmTile(0)
 
