@@ -183,7 +183,7 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
         if (e != hipSuccess) return hip_status(c, e, "mha: weight gather");
     }
     const int M = (int)rows, N3 = 3 * dModel;
-    const int tile32 = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
+    const int tile32 = c->force_tile;
     hipError_t e;
     if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)wf, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
     else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)wf, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
@@ -364,7 +364,7 @@ AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, c
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: dimensions must be positive");
     if (batch <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_batched: batch count must be positive");
     if (batch > 65535) return fail(c, AIDN_ERR_UNSUPPORTED, "sgemm_batched: more than 65535 batches");
-    int tile = (c->force_tile == 256 || c->force_tile == 129) ? 0 : c->force_tile;
+    int tile = c->force_tile;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, 0, batch,
                                         (long long)M * K, (long long)K * N, (long long)M * N, tile), "gemm_f32 (batched)");
 }

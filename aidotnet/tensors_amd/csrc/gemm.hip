@@ -520,8 +520,9 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const unsigned char* __restrict__ A = (const unsigned char*)g.A;
-    const unsigned char* __restrict__ B = (const unsigned char*)g.B;
+    const long long bz = blockIdx.z;                                         // batch index (strides in elements)
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A + bz * g.sA * EB;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B + bz * g.sB * EB;
 
     // Chunk swizzle of the B tile (which 16-byte chunk position of its LDS row a chunk of k-row `row` occupies):
     //   16-bit: c ^ ((row & 3) << 2)  -- the four rows one transposing read touches go to different bank groups;
@@ -716,14 +717,28 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     }
 
     typedef typename Raw<OutT>::type out_t;
-    out_t* __restrict__ C = (out_t*)g.C;
+    out_t* __restrict__ C = (out_t*)g.C + bz * g.sC;
     const bool fused = g.bias != nullptr || g.act != 0;
+    const bool scaled = g.alpha != 1.0f || g.beta != 0.0f;
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
             if (EDGE && col >= g.N) continue;
+            if (scaled) {                                 // C = alpha A B + beta C
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                    float v = g.alpha * acc[i][j][r];
+                    if (g.beta != 0.0f && (!EDGE || row < g.M)) {
+                        const out_t old = C[(long long)row * g.ldc + col];
+                        if constexpr (Elem<OutT>::BYTES == 4) v += g.beta * as_f32(old);
+                        else v += g.beta * Elem<OutT>::widen(old);
+                    }
+                    acc[i][j][r] = v;
+                }
+            }
             if (fused) {                                  // bias and / or activation folded into the store
                 const float bias = g.bias ? g.bias[col] : 0.0f;
 #pragma unroll
@@ -741,7 +756,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 }
 
 template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false>
-static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
+static hipError_t launch_gemm_dl(GemmArgs g, int batch, hipStream_t stream)
 {
     auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE, TRANSB>;
     constexpr int smem = 2 * (TILE * 128 + 128 * TILE);         // A tile + B tile (128 bytes of K each), two stages
@@ -753,7 +768,7 @@ static hipError_t launch_gemm_dl(GemmArgs g, hipStream_t stream)
     }
     g.tiles_m = (g.M + TILE - 1) / TILE;
     g.tiles_n = (g.N + TILE - 1) / TILE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n)), dim3(TILE == 256 ? 512 : 256), smem, stream, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(TILE == 256 ? 512 : 256), smem, stream, g);
     return hipGetLastError();
 }
 
@@ -1111,7 +1126,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         if constexpr (!TRANSB || E == 4) {
             // the direct-to-LDS kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane
             // offsets of its loads; M, N and K may be ragged
-            if (vec && batch == 1 && g.alpha == 1.0f && g.beta == 0.0f && g.lda < (1 << 21) && g.ldb < (1 << 21)) {
+            if (vec && g.lda < (1 << 21) && g.ldb < (1 << 21)) {
                 // 16-bit: the 256 x 256 tile moves half the bytes per flop of the 128 x 128 one and wins from half a chip of
                 // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
@@ -1125,11 +1140,10 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     if constexpr (!TRANSB || E == 4) {
         if (tile == 256 || tile == 129) {
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
-            if (batch != 1 || g.alpha != 1.0f || g.beta != 0.0f) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
             const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
-            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, stream) : launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, stream);
-            return exact_fit ? launch_gemm_dl<T, OutT, false, 128, TRANSB>(g, stream) : launch_gemm_dl<T, OutT, true, 128, TRANSB>(g, stream);
+            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, batch, stream);
+            return exact_fit ? launch_gemm_dl<T, OutT, false, 128, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 128, TRANSB>(g, batch, stream);
         }
     }
     if (tile == 129) tile = 128;

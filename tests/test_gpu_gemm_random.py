@@ -62,6 +62,26 @@ def test_random_fp32_gemm(be, tile):
 
 
 @pytest.mark.parametrize("tile", [256, 129])
+def test_random_fp32_direct_kernel_alpha_beta_and_batches(be, tile):
+    be.SetGemmTile(tile)
+    try:
+        rng = np.random.default_rng(400 + tile)
+        for (m, n, k) in shapes(90 + tile, 24):
+            if n % 4 or k % 4 or m % 4:                     # batch strides m*k, k*n must keep 16-byte alignment
+                continue
+            batch = int(rng.integers(1, 5))
+            a = rng.uniform(-1, 1, (batch, m, k)).astype(np.float32); b = rng.uniform(-1, 1, (batch, k, n)).astype(np.float32)
+            c0 = rng.uniform(-1, 1, (batch, m, n)).astype(np.float32)
+            alpha, beta = float(rng.uniform(-2, 2)), float(rng.uniform(-2, 2))
+            c = dev(c0.copy())
+            be.BatchedGemm(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(c), m, n, k, batch, alpha, beta)
+            truth = alpha * np.einsum("bmk,bkn->bmn", a.astype(np.float64), b.astype(np.float64)) + beta * c0.astype(np.float64)
+            assert mixed_err(c.cpu().numpy(), truth) <= 1e-4, (tile, m, n, k, batch, alpha, beta)
+    finally:
+        be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("tile", [256, 129])
 def test_random_fp32_gemm_direct_kernel(be, tile):
     be.SetGemmTile(tile)
     try:
