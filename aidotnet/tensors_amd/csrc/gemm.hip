@@ -500,16 +500,17 @@ template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRA
 __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
+    static_assert(TILE == 256 || TILE == 128 || (TILE == 64 && E == 4), "64 x 64 tiles: fp32 only (the 16-bit B swizzle needs 16 chunks per row)");
     constexpr int WM = 2, WN = TILE == 256 ? 4 : 2;
     constexpr int BM = TILE, BN = TILE, BK = 128 / EB;          // 128 bytes of K per tile row: 64 halves / 32 floats
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int BROW = BN * EB;                 // bytes of one k-row of the B tile
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
-    constexpr int LA = 4, LB = 4;                 // 1 KiB wave-loads per wave per tile (every instance: 32 + 32 resp. 16 + 16 per workgroup)
+    constexpr int LA = BM / 8 / (WM * WN), LB = LA;   // 1 KiB wave-loads per wave per tile (4 + 4; 2 + 2 for the 64 x 64 tile)
     constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load
     constexpr int LPR = 64 / RPL;                 // lanes (16-byte chunks) per B row
-    static_assert(BK * BROW / 1024 == LB * WM * WN && BN / 8 == LB * WM * WN, "B tile = four wave-loads per wave");
+    static_assert(BK * BROW / 1024 == LB * WM * WN && BN / 8 == LB * WM * WN && LA % 2 == 0, "B tile = as many wave-loads as the A tile");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -719,38 +720,55 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     typedef typename Raw<OutT>::type out_t;
     out_t* __restrict__ C = (out_t*)g.C + bz * g.sC;
     const bool fused = g.bias != nullptr || g.act != 0;
-    const bool scaled = g.alpha != 1.0f || g.beta != 0.0f;
+    if (Elem<OutT>::BYTES == 4 && (g.alpha != 1.0f || g.beta != 0.0f)) {
+        // C = act(alpha A B + beta C + bias), fp32 output only: the uncommon form, kept apart so the plain stores below stay lean
+#pragma unroll 1
+        for (int ij = 0; ij < TM * TN; ij++) {
+            const int i = ij / TN, j = ij - i * TN;
+            const int col = n0 + wn * WTN + j * 32 + l32;
+            if (EDGE && col >= g.N) continue;
+            const float bias = g.bias ? g.bias[col] : 0.0f;
+            f32x16 v = acc[0][0];
+#pragma unroll
+            for (int ii = 0; ii < TM; ii++)
+#pragma unroll
+                for (int jj = 0; jj < TN; jj++) if (ii == i && jj == j) v = acc[ii][jj];
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                if (EDGE && row >= g.M) continue;
+                out_t* p = C + (long long)row * g.ldc + col;
+                float x = g.alpha * v[r];
+                if (g.beta != 0.0f) {
+                    if constexpr (Elem<OutT>::BYTES == 4) x += g.beta * as_f32(*p);
+                    else x += g.beta * Elem<OutT>::widen(*p);
+                }
+                if (fused) x = apply_activation(x + bias, g.act, g.act_param);
+                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(x);
+                else *p = (out_t)Elem<OutT>::narrow(x);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
-            if (EDGE && col >= g.N) continue;
-            if (scaled) {                                 // C = alpha A B + beta C
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
-                    float v = g.alpha * acc[i][j][r];
-                    if (g.beta != 0.0f && (!EDGE || row < g.M)) {
-                        const out_t old = C[(long long)row * g.ldc + col];
-                        if constexpr (Elem<OutT>::BYTES == 4) v += g.beta * as_f32(old);
-                        else v += g.beta * Elem<OutT>::widen(old);
-                    }
-                    acc[i][j][r] = v;
-                }
-            }
+            const bool col_ok = !EDGE || col < g.N;
             if (fused) {                                  // bias and / or activation folded into the store
-                const float bias = g.bias ? g.bias[col] : 0.0f;
+                const float bias = (g.bias && col_ok) ? g.bias[col] : 0.0f;
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = apply_activation(acc[i][j][r] + bias, g.act, g.act_param);
             }
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
-                if (EDGE && row >= g.M) continue;
                 out_t* p = C + (long long)row * g.ldc + col;
-                if constexpr (Elem<OutT>::BYTES == 4) *p = as_u32(acc[i][j][r]);
-                else *p = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
+                out_t v;
+                if constexpr (Elem<OutT>::BYTES == 4) v = as_u32(acc[i][j][r]);
+                else v = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
+                if (col_ok && (!EDGE || row < g.M)) *p = v;
             }
         }
 }
@@ -1126,23 +1144,39 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         if constexpr (!TRANSB || E == 4) {
             // the direct-to-LDS kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane
             // offsets of its loads; M, N and K may be ragged
-            if (vec && g.lda < (1 << 21) && g.ldb < (1 << 21)) {
+            if (vec && g.lda < (1 << 21) && g.ldb < (1 << 21) && (Elem<OutT>::BYTES == 4 || (g.alpha == 1.0f && g.beta == 0.0f))) {
                 // 16-bit: the 256 x 256 tile moves half the bytes per flop of the 128 x 128 one and wins from half a chip of
                 // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
                 const bool big = E == 8 ? t256 >= 128 : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
                 if (big) tile = 256;
                 else if (t128 >= 128 && choose_tile(t128, tiles(64, 64), E == 4 ? 0.85 : 0.55) == 128) tile = 129;   // same kernel, 128 x 128 tiles
+                else if (E == 4 && choose_tile(t128, tiles(64, 64), 0.85) == 64) tile = 65;                         // fp32: and 64 x 64 tiles
             }
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
+    if constexpr (E == 4) {
+        if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel (fp32)
+            if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
+            const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % 32 == 0;
+            return exact_fit ? launch_gemm_dl<T, OutT, false, 64, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 64, TRANSB>(g, batch, stream);
+        }
+    }
+    if (tile == 65) tile = 64;
     if constexpr (!TRANSB || E == 4) {
         if (tile == 256 || tile == 129) {
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
+            if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
             const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
-            if (tile == 256) return exact_fit ? launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, batch, stream);
+            // (bf16 output with ragged edges on the 256 x 256 tile: that one instance does not fit the register file -- the
+            // compiler moves accumulators to scratch memory -- so such problems take the 128 x 128 tile)
+            constexpr bool kSpills256Edge = std::is_same<T, bf16_t>::value && std::is_same<OutT, bf16_t>::value;
+            if (tile == 256 && exact_fit) return launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, batch, stream);
+            if constexpr (!kSpills256Edge) {
+                if (tile == 256) return launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, batch, stream);
+            }
             return exact_fit ? launch_gemm_dl<T, OutT, false, 128, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 128, TRANSB>(g, batch, stream);
         }
     }

@@ -251,8 +251,9 @@ AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* in
                             const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
 
 /* ---- test / tuning hook --------------------------------------------------------------------------------
- * Forces the GEMM tile edge (64, 128 or 256; 129 = 128 with the 16-bit direct-to-LDS kernel; 0 = automatic choice) for
- * subsequent calls on this context, so the parity suite can exercise every kernel instance.  No counterpart in the reference. */
+ * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel, 65 for fp32 only; 0 = automatic
+ * choice) for subsequent calls on this context, so the parity suite can exercise every kernel instance.  No counterpart in the
+ * reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
 /* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast
  * path is then not taken), so the parity suite can hold the two kernels against each other.  Process-wide.

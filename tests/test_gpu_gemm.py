@@ -383,7 +383,7 @@ def test_conversions_bit_exact(be, n):
 
 
 # ---------------------------------------------------------------- fp32 on the direct global->LDS kernel
-@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("tile", [256, 129, 65])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 32), (256, 256, 128), (512, 256, 96), (768, 1024, 160), (256, 512, 2048),
                                    (257, 260, 32), (300, 516, 100), (1, 4, 32), (255, 248, 4), (511, 1000, 132), (700, 36, 36)])
 def test_fp32_gemm_direct_to_lds_path(be, tile, M, N, K):

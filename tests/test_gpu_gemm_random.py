@@ -61,7 +61,7 @@ def test_random_fp32_gemm(be, tile):
         be.SetGemmTile(0)
 
 
-@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("tile", [256, 129, 65])
 def test_random_fp32_direct_kernel_alpha_beta_and_batches(be, tile):
     be.SetGemmTile(tile)
     try:
@@ -81,7 +81,7 @@ def test_random_fp32_direct_kernel_alpha_beta_and_batches(be, tile):
         be.SetGemmTile(0)
 
 
-@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("tile", [256, 129, 65])
 def test_random_fp32_gemm_direct_kernel(be, tile):
     be.SetGemmTile(tile)
     try:
