@@ -6,6 +6,7 @@ Run as ``python -m aidotnet.tensors_amd.build``; ``__graft_entry__.build()`` cal
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -28,10 +29,34 @@ def _hipcc() -> str:
 
 
 def _compile(src: str, obj: str) -> None:
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
+    # the resource-usage remarks name every kernel with its register and scratch use: a kernel that needs scratch memory has
+    # spilled registers (for the GEMM kernels that means accumulators in memory and a 30-fold slowdown), so the build refuses it
+    cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, r.stderr[-4000:]))
+    spilled = [kv for kv in kernels_with_scratch(r.stderr) if not _KNOWN_SCRATCH.search(kv[0])]
+    if spilled:
+        raise RuntimeError("%s: kernels that spill registers to scratch memory:\n  %s"
+                           % (src, "\n  ".join("%s (%d bytes/lane)" % kv for kv in spilled)))
+
+
+# The general attention kernel at head dimension 256 (its largest instance, one workgroup per CU) keeps 48-200 bytes per lane
+# in scratch; it is correct and rarely used, so it is tolerated.  Nothing else may spill.
+_KNOWN_SCRATCH = re.compile(r"attn_fwd_kernelI\w*?Li256ELi(32|64)E")
+
+
+def kernels_with_scratch(remarks: str):
+    """(kernel name, scratch bytes per lane) of every kernel in hipcc's kernel-resource-usage remarks that uses scratch."""
+    out, name = [], None
+    for line in remarks.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split("[")[0].strip()
+        elif "ScratchSize [bytes/lane]:" in line and name is not None:
+            n = int(line.split("ScratchSize [bytes/lane]:")[1].split("[")[0].strip())
+            if n > 0:
+                out.append((name, n))
+    return out
 
 
 def build_library(verbose: bool = False, jobs: int = 5) -> str:

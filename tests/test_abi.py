@@ -73,3 +73,16 @@ def test_no_product_module_imports_the_oracle():
             if f.endswith((".py", ".hip", ".hpp", ".cpp", ".h")):
                 src = open(os.path.join(dp, f), errors="replace").read()
                 assert "import oracle" not in src and "liboracle" not in src and "from oracle" not in src, f
+
+
+def test_build_rejects_kernels_that_spill():
+    """The build parses hipcc's resource-usage remarks and refuses a kernel that needs scratch memory."""
+    from aidotnet.tensors_amd.build import kernels_with_scratch
+    remarks = """a.hip:1:1: remark: Function Name: _ZN4aidn3fooEv [-Rpass-analysis=kernel-resource-usage]
+a.hip:1:1: remark:     VGPRs: 17 [-Rpass-analysis=kernel-resource-usage]
+a.hip:1:1: remark:     ScratchSize [bytes/lane]: 0 [-Rpass-analysis=kernel-resource-usage]
+a.hip:9:1: remark: Function Name: _ZN4aidn3barEv [-Rpass-analysis=kernel-resource-usage]
+a.hip:9:1: remark:     ScratchSize [bytes/lane]: 576 [-Rpass-analysis=kernel-resource-usage]
+"""
+    assert kernels_with_scratch(remarks) == [("_ZN4aidn3barEv", 576)]
+    assert kernels_with_scratch("") == []
