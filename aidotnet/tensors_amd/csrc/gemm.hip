@@ -500,7 +500,7 @@ template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRA
 __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
-    static_assert(TILE == 256 || TILE == 128 || (TILE == 64 && E == 4), "64 x 64 tiles: fp32 only (the 16-bit B swizzle needs 16 chunks per row)");
+    static_assert(TILE == 256 || TILE == 128 || TILE == 64, "tile edge");
     constexpr int WM = 2, WN = TILE == 256 ? 4 : 2;
     constexpr int BM = TILE, BN = TILE, BK = 128 / EB;          // 128 bytes of K per tile row: 64 halves / 32 floats
     constexpr int WTM = BM / WM, WTN = BN / WN;
@@ -526,9 +526,12 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     const unsigned char* __restrict__ B = (const unsigned char*)g.B + bz * g.sB * EB;
 
     // Chunk swizzle of the B tile (which 16-byte chunk position of its LDS row a chunk of k-row `row` occupies):
-    //   16-bit: c ^ ((row & 3) << 2)  -- the four rows one transposing read touches go to different bank groups;
+    //   16-bit: c ^ ((row & 3) << 2)  -- the four rows one transposing read touches go to different bank groups (rows of 256
+    //           bytes and more; 128-byte rows, which alternate between the bank halves by themselves: c ^ (((row >> 1) & 1) << 2));
     //   fp32:   c ^ (((row >> 2) & 1) << 3)  -- the two lane halves of a b32 fragment read (rows 4 apart) use different bank halves.
-    auto b_swz = [](int row) -> int { return E == 8 ? ((row & 3) << 2) : (((row >> 2) & 1) << 3); };
+    auto b_swz = [](int row) -> int {
+        return E == 8 ? (BROW >= 256 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2)) : (((row >> 2) & 1) << 3);
+    };
 
     // Sources of this wave's loads: a wave-uniform base (scalar registers, advanced per tile by scalar adds) plus a per-lane
     // 32-bit byte offset that never changes, so issuing a load costs no vector instruction.  Wave-load w = 4 wave + i covers
@@ -657,7 +660,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 #pragma unroll
                 for (int q = 0; q < 2; q++) {
                     int row = 16 * s + 4 * q + b_rowl;
-                    int pos = b_chunk[j] ^ ((row & 3) << 2);
+                    int pos = b_chunk[j] ^ b_swz(row);
                     s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                         (__attribute__((address_space(3))) s16x4*)(bs + row * BROW + pos * 16 + b_half));
                     u32x2 w = __builtin_bit_cast(u32x2, v);
@@ -1149,17 +1152,19 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
                 // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
                 const bool big = E == 8 ? t256 >= 128 : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
+                // otherwise the same kernel with 128 x 128 or 64 x 64 tiles (codes 129, 65), whichever loads the CUs better; per
+                // flop the 64 x 64 instance runs at about 0.85 (fp32) resp. 0.8 (16-bit) of the 128 x 128 one
                 if (big) tile = 256;
-                else if (t128 >= 128 && choose_tile(t128, tiles(64, 64), E == 4 ? 0.85 : 0.55) == 128) tile = 129;   // same kernel, 128 x 128 tiles
-                else if (E == 4 && choose_tile(t128, tiles(64, 64), 0.85) == 64) tile = 65;                         // fp32: and 64 x 64 tiles
+                else tile = choose_tile(t128, tiles(64, 64), E == 4 ? 0.85 : 0.8) == 128 ? 129 : 65;
             }
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
-    if constexpr (E == 4) {
-        if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel (fp32)
+    if constexpr (E == 4 || !TRANSB) {
+        if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
-            const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % 32 == 0;
+            if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
+            const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % (8 * E) == 0;
             return exact_fit ? launch_gemm_dl<T, OutT, false, 64, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 64, TRANSB>(g, batch, stream);
         }
     }

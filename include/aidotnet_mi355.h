@@ -251,7 +251,7 @@ AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* in
                             const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
 
 /* ---- test / tuning hook --------------------------------------------------------------------------------
- * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel, 65 for fp32 only; 0 = automatic
+ * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel; 0 = automatic
  * choice) for subsequent calls on this context, so the parity suite can exercise every kernel instance.  No counterpart in the
  * reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);

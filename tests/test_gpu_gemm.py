@@ -204,7 +204,7 @@ def test_half_gemm_random_within_tolerance(be, kind, M, N, K):
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
-@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("tile", [256, 129, 65])
 @pytest.mark.parametrize("M,N,K", [(256, 256, 64), (256, 256, 128), (512, 256, 192), (768, 1024, 320), (256, 512, 4096)])
 def test_half_gemm_large_tile_direct_to_lds_path(be, kind, tile, M, N, K):
     # the direct global->LDS kernel (256 x 256 tiles, or 128 x 128 as tile code 129) forced on small shapes
@@ -233,7 +233,7 @@ def test_half_gemm_large_tile_direct_to_lds_path(be, kind, tile, M, N, K):
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("M,N,K", [(257, 264, 64), (300, 520, 128), (1, 8, 64), (255, 248, 192), (511, 1000, 256), (700, 72, 64),
                                    (257, 264, 72), (300, 520, 200), (255, 248, 8), (511, 1000, 264), (256, 256, 120)])
-@pytest.mark.parametrize("tile", [256, 129])
+@pytest.mark.parametrize("tile", [256, 129, 65])
 def test_half_gemm_large_tile_ragged_edges(be, kind, tile, M, N, K):
     # the 256 x 256 tile kernel on M, N and K it does not divide (clamped loads, zero-filled K tail, guarded stores); C is pre-filled so a store
     # outside the matrix or a missing one shows
