@@ -62,6 +62,19 @@ __device__ __forceinline__ u32x4 ld16(const typename Raw2<T>::type* p, int valid
 constexpr float LOG2E = 1.4426950408889634f;
 constexpr float LN2 = 0.6931471805599453f;
 
+// Direct global -> LDS load of 16 bytes per lane: lane i's data lands at LDS address lds_dst + 16 i (lds_dst wave
+// uniform).  Issued from inline asm so the compiler does not order later LDS reads behind it; completion is
+// awaited explicitly (s_waitcnt vmcnt(0) + barrier) before the tile is read.
+__device__ __forceinline__ void attn_dma16(const void* gptr, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_dst), "v"(gptr) : "memory");
+}
+// same, source = wave-uniform base (SGPR pair) + per-lane unsigned 32-bit byte offset
+__device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
+}
+
 // packed conversions of probabilities and pair sums (shared by both kernels)
 template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
@@ -96,9 +109,14 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
     return __builtin_bit_cast(uint32_t, v);
 }
 
-template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB>
+// DMA (fp32, plain / causal, aligned contiguous K/V): the K and V tiles go global -> LDS directly, unpadded [key][d] rows with
+// XOR-swizzled 16-byte chunks (K: c ^ (key & 15) for the b128 fragment reads; V: c ^ (((key >> 2) & 1) << 3), read as the
+// A operand of O^T += V^T P^T with 32-bit LDS reads, the two lane halves -- keys 4 apart -- in different bank halves).  This
+// removes the register -> LDS store path (and the V transpose in registers) of the general form.
+template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB, bool DMA = false>
 __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 {
+    static_assert(!DMA || (Elem<T>::BYTES == 4 && !FULL && DP * 4 == 256), "DMA form: fp32, 256-byte rows");
     typedef typename Raw2<T>::type raw_t;
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     constexpr int NT = 256, BR = 128;
@@ -106,7 +124,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     constexpr int DSTEPS = DP / KS;            // fragment steps over the head dim (QK^T)
     constexpr int KPITCH = DP * EB + 16;       // K tile [key][d] row pitch, bytes
     constexpr int VPITCH = BC * EB + 16;       // V^T tile [d][key] row pitch, bytes
-    constexpr int KBYTES = BC * KPITCH, VBYTES = DP * VPITCH;
+    constexpr int KBYTES = DMA ? BC * DP * EB : BC * KPITCH, VBYTES = DMA ? BC * DP * EB : DP * VPITCH;
     constexpr int KT = BC / 32;                // 32-key sub-tiles per tile
     constexpr int DT = DP / 32;                // 32-row tiles of O^T
     constexpr int PSTEPS = 32 / KS;            // PV fragment steps per key sub-tile
@@ -252,16 +270,37 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
     const float sl2 = a.scale * LOG2E;
 
-    if (ntiles > 0) {
-        load_tile(0);
-        store_tile(0);
+    // DMA form: this wave's loads of a tile are K and V wave-loads 4 wave .. 4 wave + 3 (4 keys x 256 bytes each); rows past
+    // the end of the sequence repeat the last key (masked below)
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    auto issue_tile = [&](int tile, int stage) {
+        const int ld_key = lane >> 4, ld_pos = lane & 15;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int key = 4 * (4 * wave + i) + ld_key;                   // key inside the tile
+            const long long gkey = min(tile * BC + key, a.Sk - 1);
+            attn_dma16(K + gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 4, lds0 + stage * KBYTES + (4 * wave_s + i) * 1024);
+            attn_dma16(V + gkey * a.vs[2] + (ld_pos ^ (((key >> 2) & 1) << 3)) * 4,
+                       lds0 + 2 * KBYTES + stage * VBYTES + (4 * wave_s + i) * 1024);
+        }
+    };
+    if constexpr (DMA) {
+        if (ntiles > 0) issue_tile(0, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+    } else {
+        if (ntiles > 0) {
+            load_tile(0);
+            store_tile(0);
+        }
     }
     __syncthreads();
 
     for (int j = 0; j < ntiles; j++) {
         const int stage = j & 1;
         const int kv0 = j * BC;
-        if (j + 1 < ntiles) load_tile(kv0 + BC);
+        if constexpr (DMA) { if (j + 1 < ntiles) issue_tile(j + 1, stage ^ 1); }
+        else if (j + 1 < ntiles) load_tile(kv0 + BC);
 
         // a wave whose 32 rows are all above the causal diagonal of this tile only helps with the copies
         const bool active = !(a.causal && (long long)kv0 > (long long)wq_max + a.qoff);
@@ -278,7 +317,9 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             for (int s = 0; s < DSTEPS; s++) {
 #pragma unroll
                 for (int kt = 0; kt < KT; kt++) {
-                    u32x4 kf = *(const u32x4*)(ks + kt * 32 * KPITCH + s * 32);
+                    u32x4 kf;
+                    if constexpr (DMA) kf = *(const u32x4*)(Ks + stage * KBYTES + (kt * 32 + l32) * 256 + (((2 * s + h) ^ (l32 & 15)) << 4));
+                    else kf = *(const u32x4*)(ks + kt * 32 * KPITCH + s * 32);
                     Mma32<T>::run(st[kt], kf, qf[s]);
                 }
             }
@@ -351,13 +392,23 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     }
 #pragma unroll
                     for (int i = 0; i < DT; i++) {
-                        u32x4 vf = *(const u32x4*)(vs + i * 32 * VPITCH + kt * 32 * EB + ps * 32);
+                        u32x4 vf;
+                        if constexpr (DMA) {
+                            // V[key = 32 kt + 8 ps + 4 h + q][d = 32 i + l32]; (key >> 2) & 1 == h
+                            const int d = i * 32 + l32;
+                            const unsigned char* vp = Vs + stage * VBYTES + (kt * 32 + 8 * ps + 4 * h) * 256 + ((((d >> 2) ^ (h << 3)) << 4) + (d & 3) * 4);
+#pragma unroll
+                            for (int q = 0; q < 4; q++) vf[q] = *(const uint32_t*)(vp + q * 256);
+                        } else {
+                            vf = *(const u32x4*)(vs + i * 32 * VPITCH + kt * 32 * EB + ps * 32);
+                        }
                         Mma32<T>::run(oacc[i], vf, pf);
                     }
                 }
             }
         }
-        if (j + 1 < ntiles) store_tile(stage ^ 1);
+        if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0);      // this wave's loads of tile j + 1 have landed
+        else if (j + 1 < ntiles) store_tile(stage ^ 1);
         __syncthreads();
     }
 
@@ -415,18 +466,6 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 // for any reference point m.
 typedef short s16x4a __attribute__((ext_vector_type(4)));
 
-// Direct global -> LDS load of 16 bytes per lane: lane i's data lands at LDS address lds_dst + 16 i (lds_dst wave
-// uniform).  Issued from inline asm so the compiler does not order later LDS reads behind it; completion is
-// awaited explicitly (s_waitcnt vmcnt(0) + barrier) before the tile is read.
-__device__ __forceinline__ void attn_dma16(const void* gptr, uint32_t lds_dst)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_dst), "v"(gptr) : "memory");
-}
-// same, source = wave-uniform base (SGPR pair) + per-lane unsigned 32-bit byte offset
-__device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
-{
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
-}
 
 template <typename T, typename OutT>
 __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
@@ -806,12 +845,12 @@ __global__ __launch_bounds__(256) void attn_weights_kernel(const AttnArgs a, flo
 }
 
 // ------------------------------------------------------------------ host side
-template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB>
+template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB, bool DMA = false>
 static hipError_t launch_attn(AttnArgs a, hipStream_t stream)
 {
-    auto kern = attn_fwd_kernel<T, OutT, DP, BC, FULL, MINB>;
+    auto kern = attn_fwd_kernel<T, OutT, DP, BC, FULL, MINB, DMA>;
     constexpr int EB = Elem<T>::BYTES;
-    constexpr int smem = 2 * (BC * (DP * EB + 16) + DP * (BC * EB + 16));
+    constexpr int smem = DMA ? 4 * BC * DP * EB : 2 * (BC * (DP * EB + 16) + DP * (BC * EB + 16));
     static bool attr_set = false;
     if (!attr_set) {
         hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -871,7 +910,8 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     } else
     if (kind == 0) {
         // fp32: 64-key tiles while two workgroups still fit the LDS of a CU (head dimension up to 64), else 32-key tiles
-        if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
+        if (p.D == 64 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) err = launch_attn<float, float, 64, 64, false, 2, true>(a, stream);
+        else if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
                                   : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
         else err = dispatch_attn_d<float, float, 32>(a, full, stream);
     }

@@ -327,3 +327,25 @@ def test_fast_path_all_masked_rows_and_large_logits(be):
     assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
     assert mixed_err(o, o64) <= HALF_TOL
     assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
+
+
+# --------------------------------------------------------------- fp32 head-dim-64 direct-to-LDS form of the general kernel
+@pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
+                                                                   (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
+def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, B, H, Hkv, Sq, Sk, causal, offset):
+    D = 64
+    rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + 64)
+    q, k, v = _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
+    scale = 1.0 / math.sqrt(D)
+    o64, lse64 = oracle.attention_f64(q, k, v, scale, causal, offset)
+    outs = {}
+    try:
+        for direct in (True, False):
+            be.SetAttentionFastPath(direct)
+            o, lse = eng.FlashAttention(dev(q), dev(k), dev(v), scale, causal, queryOffset=offset)
+            outs[direct] = (o.cpu().numpy(), lse.cpu().numpy())
+            assert mixed_err(outs[direct][0], o64) <= FP32_TOL and mixed_err(outs[direct][1], lse64) <= FP32_TOL
+    finally:
+        be.SetAttentionFastPath(True)
+    # the two forms multiply and sum the same values in the same order: identical results
+    assert np.array_equal(outs[True][0], outs[False][0]) and np.array_equal(outs[True][1], outs[False][1])
