@@ -75,6 +75,8 @@ __device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
 }
 
+typedef short s16x4a __attribute__((ext_vector_type(4)));
+
 // packed conversions of probabilities and pair sums (shared by both kernels)
 template <typename T> __device__ __forceinline__ uint32_t pack2_p(float a, float b);
 template <> __device__ __forceinline__ uint32_t pack2_p<f16_t>(float a, float b)
@@ -116,7 +118,7 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
 template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB, bool DMA = false>
 __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 {
-    static_assert(!DMA || (Elem<T>::BYTES == 4 && !FULL && DP * 4 == 256), "DMA form: fp32, 256-byte rows");
+    static_assert(!DMA || (!FULL && DP == 64 && BC == 64), "DMA form: head dimension 64, 64-key tiles, plain / causal");
     typedef typename Raw2<T>::type raw_t;
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     constexpr int NT = 256, BR = 128;
@@ -274,15 +276,24 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     // the end of the sequence repeat the last key (masked below)
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    // swizzles of the DMA form (chunk position of 16-byte chunk c of key row `key`):
+    //   fp32 (256-byte rows):   K  c ^ (key & 15);         V  c ^ (((key >> 2) & 1) << 3)   (32-bit reads, lane halves 4 keys apart)
+    //   16-bit (128-byte rows): K  c ^ ((key >> 1) & 7);   V  c ^ (((key >> 1) & 1) << 2)   (transposing reads of 4 consecutive keys)
+    auto k_swz = [](int key) -> int { return EB == 4 ? (key & 15) : ((key >> 1) & 7); };
+    auto v_swz = [](int key) -> int { return EB == 4 ? (((key >> 2) & 1) << 3) : (((key >> 1) & 1) << 2); };
     auto issue_tile = [&](int tile, int stage) {
-        const int ld_key = lane >> 4, ld_pos = lane & 15;
+        constexpr int ROWB = DP * EB;                      // 256 / 128 bytes per key row
+        constexpr int KPL = 1024 / ROWB;                   // keys per 1 KiB wave-load
+        constexpr int LPW = BC / KPL / 4;                  // wave-loads per wave and tile (K and V each)
+        constexpr int CPRW = ROWB / 16;                    // chunks per row
+        const int ld_key = lane / CPRW, ld_pos = lane % CPRW;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const int key = 4 * (4 * wave + i) + ld_key;                   // key inside the tile
+        for (int i = 0; i < LPW; i++) {
+            const int key = KPL * (LPW * wave + i) + ld_key;               // key inside the tile
             const long long gkey = min(tile * BC + key, a.Sk - 1);
-            attn_dma16(K + gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 4, lds0 + stage * KBYTES + (4 * wave_s + i) * 1024);
-            attn_dma16(V + gkey * a.vs[2] + (ld_pos ^ (((key >> 2) & 1) << 3)) * 4,
-                       lds0 + 2 * KBYTES + stage * VBYTES + (4 * wave_s + i) * 1024);
+            attn_dma16(K + gkey * a.ks[2] + (ld_pos ^ k_swz(key)) * E, lds0 + stage * KBYTES + (LPW * wave_s + i) * 1024);
+            attn_dma16(V + gkey * a.vs[2] + (ld_pos ^ v_swz(key)) * E,
+                       lds0 + 2 * KBYTES + stage * VBYTES + (LPW * wave_s + i) * 1024);
         }
     };
     if constexpr (DMA) {
@@ -318,7 +329,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
                 for (int kt = 0; kt < KT; kt++) {
                     u32x4 kf;
-                    if constexpr (DMA) kf = *(const u32x4*)(Ks + stage * KBYTES + (kt * 32 + l32) * 256 + (((2 * s + h) ^ (l32 & 15)) << 4));
+                    if constexpr (DMA) kf = *(const u32x4*)(Ks + stage * KBYTES + (kt * 32 + l32) * (DP * EB) + (((2 * s + h) ^ k_swz(l32)) << 4));
                     else kf = *(const u32x4*)(ks + kt * 32 * KPITCH + s * 32);
                     Mma32<T>::run(st[kt], kf, qf[s]);
                 }
@@ -393,12 +404,26 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
                     for (int i = 0; i < DT; i++) {
                         u32x4 vf;
-                        if constexpr (DMA) {
+                        if constexpr (DMA && EB == 4) {
                             // V[key = 32 kt + 8 ps + 4 h + q][d = 32 i + l32]; (key >> 2) & 1 == h
                             const int d = i * 32 + l32;
                             const unsigned char* vp = Vs + stage * VBYTES + (kt * 32 + 8 * ps + 4 * h) * 256 + ((((d >> 2) ^ (h << 3)) << 4) + (d & 3) * 4);
 #pragma unroll
                             for (int q = 0; q < 4; q++) vf[q] = *(const uint32_t*)(vp + q * 256);
+                        } else if constexpr (DMA) {
+                            // 16-bit: the lane's eight k-slots are keys 16 ps + 4 h + (0..3) and 16 ps + 8 + 4 h + (0..3) (the order of
+                            // the accumulator rows its P values come from); one transposing read per group of four: in a
+                            // 16-lane group lane j addresses key (base + j / 4), 8 bytes at head-dim 4 (j % 4) of the 16-wide block
+                            const int jl = lane & 15;
+                            const int chunk = (i * 32 + 16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3;
+#pragma unroll
+                            for (int q = 0; q < 2; q++) {
+                                const int row = kt * 32 + 16 * ps + 8 * q + 4 * h + (jl >> 2);
+                                u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                                    (__attribute__((address_space(3))) s16x4a*)(Vs + stage * VBYTES + row * 128 + ((chunk ^ v_swz(row)) << 4) + (jl & 1) * 8)));
+                                vf[2 * q] = w[0];
+                                vf[2 * q + 1] = w[1];
+                            }
                         } else {
                             vf = *(const u32x4*)(vs + i * 32 * VPITCH + kt * 32 * EB + ps * 32);
                         }
@@ -464,7 +489,6 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 // the exponent is only raised when the true max has grown by more than 8 (log2 units), so the O
 // accumulator is rescaled rarely and P never exceeds 2^8 -- exact mathematics, LSE = m + log2(l) holds
 // for any reference point m.
-typedef short s16x4a __attribute__((ext_vector_type(4)));
 
 
 template <typename T, typename OutT>
@@ -914,6 +938,11 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
         else if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
                                   : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
         else err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    }
+    else if (p.D == 64 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) {
+        // head dimension 64, plain / causal, aligned contiguous K/V: the direct-to-LDS form of the general kernel
+        if (kind == 1) err = p.out16 ? launch_attn<f16_t, f16_t, 64, 64, false, 2, true>(a, stream) : launch_attn<f16_t, float, 64, 64, false, 2, true>(a, stream);
+        else err = p.out16 ? launch_attn<bf16_t, bf16_t, 64, 64, false, 2, true>(a, stream) : launch_attn<bf16_t, float, 64, 64, false, 2, true>(a, stream);
     }
     else if (kind == 1) err = p.out16 ? dispatch_attn_d<f16_t, f16_t, 64>(a, full, stream) : dispatch_attn_d<f16_t, float, 64>(a, full, stream);
     else err = p.out16 ? dispatch_attn_d<bf16_t, bf16_t, 64>(a, full, stream) : dispatch_attn_d<bf16_t, float, 64>(a, full, stream);

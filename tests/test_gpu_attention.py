@@ -349,3 +349,35 @@ def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, B, H
         be.SetAttentionFastPath(True)
     # the two forms multiply and sum the same values in the same order: identical results
     assert np.array_equal(outs[True][0], outs[False][0]) and np.array_equal(outs[True][1], outs[False][1])
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
+                                                                   (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
+def test_half_d64_direct_load_form_matches_oracle_and_general_form(be, kind, B, H, Hkv, Sq, Sk, causal, offset):
+    D = 64
+    rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + len(kind) + 64)
+    q, k, v = _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+    scale = 1.0 / math.sqrt(D)
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale, causal, offset)
+    dt = TORCH16[kind]
+    args = (be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)))
+    outs = {}
+    try:
+        for direct in (True, False):
+            be.SetAttentionFastPath(direct)
+            out = torch.full((B, H, Sq, D), float("nan"), device="cuda")
+            lse = torch.full((B, H, Sq), float("nan"), device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out), be.WrapTensor(lse), B, H, Sq, Sk, D, scale, causal, offset, Hkv)
+            outs[direct] = (out.cpu().numpy(), lse.cpu().numpy())
+            assert mixed_err(outs[direct][0], o64) <= HALF_TOL
+            assert mixed_err(outs[direct][1], lse64) <= 1e-3
+        be.SetAttentionFastPath(True)
+        out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
+        be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
+        assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
+    finally:
+        be.SetAttentionFastPath(True)
+    # same values multiplied and summed in the same order by both forms
+    assert np.array_equal(outs[True][0], outs[False][0]) and np.array_equal(outs[True][1], outs[False][1])
