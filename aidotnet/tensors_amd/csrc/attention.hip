@@ -118,7 +118,8 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
 template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB, bool DMA = false>
 __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 {
-    static_assert(!DMA || (!FULL && DP == 64 && BC == 64), "DMA form: head dimension 64, 64-key tiles, plain / causal");
+    static_assert(!DMA || (!FULL && ((DP == 64 && BC == 64) || (Elem<T>::BYTES == 4 && DP == 128 && BC == 32))),
+                  "DMA form: head dimension 64 with 64-key tiles (or fp32 128 with 32-key tiles), plain / causal");
     typedef typename Raw2<T>::type raw_t;
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     constexpr int NT = 256, BR = 128;
@@ -407,9 +408,9 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                         if constexpr (DMA && EB == 4) {
                             // V[key = 32 kt + 8 ps + 4 h + q][d = 32 i + l32]; (key >> 2) & 1 == h
                             const int d = i * 32 + l32;
-                            const unsigned char* vp = Vs + stage * VBYTES + (kt * 32 + 8 * ps + 4 * h) * 256 + ((((d >> 2) ^ (h << 3)) << 4) + (d & 3) * 4);
+                            const unsigned char* vp = Vs + stage * VBYTES + (kt * 32 + 8 * ps + 4 * h) * (DP * 4) + ((((d >> 2) ^ (h << 3)) << 4) + (d & 3) * 4);
 #pragma unroll
-                            for (int q = 0; q < 4; q++) vf[q] = *(const uint32_t*)(vp + q * 256);
+                            for (int q = 0; q < 4; q++) vf[q] = *(const uint32_t*)(vp + q * (DP * 4));
                         } else if constexpr (DMA) {
                             // 16-bit: the lane's eight k-slots are keys 16 ps + 4 h + (0..3) and 16 ps + 8 + 4 h + (0..3) (the order of
                             // the accumulator rows its P values come from); one transposing read per group of four: in a
@@ -935,6 +936,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     if (kind == 0) {
         // fp32: 64-key tiles while two workgroups still fit the LDS of a CU (head dimension up to 64), else 32-key tiles
         if (p.D == 64 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) err = launch_attn<float, float, 64, 64, false, 2, true>(a, stream);
+        else if (p.D == 128 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) err = launch_attn<float, float, 128, 32, false, 2, true>(a, stream);
         else if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
                                   : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
         else err = dispatch_attn_d<float, float, 32>(a, full, stream);

@@ -332,8 +332,8 @@ def test_fast_path_all_masked_rows_and_large_logits(be):
 # --------------------------------------------------------------- fp32 head-dim-64 direct-to-LDS form of the general kernel
 @pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
                                                                    (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
-def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, B, H, Hkv, Sq, Sk, causal, offset):
-    D = 64
+@pytest.mark.parametrize("D", [64, 128])
+def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, D, B, H, Hkv, Sq, Sk, causal, offset):
     rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + 64)
     q, k, v = _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
     scale = 1.0 / math.sqrt(D)
