@@ -259,6 +259,25 @@ def test_half_gemm_large_tile_ragged_edges(be, kind, tile, M, N, K):
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(256, 256, 64), (300, 520, 128), (130, 72, 64), (512, 768, 192)])
+def test_half_gemm_16bit_output_guard_band_and_odd_offset(be, kind, M, N, K):
+    # 16-bit results leave the direct-to-LDS kernel as 32-bit column pairs: elements around the matrix must stay untouched, and
+    # an output that starts on an odd element (not 4-byte aligned) must take a kernel with element stores -- same bits either way
+    rng = np.random.default_rng(5 * M + N + K)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+    ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+    want16, _ = (oracle.hgemm if kind == "f16" else oracle.bf16gemm)(ab, bb, M, K, N)
+    A = be.WrapTensor(from_bits16(ab, TORCH16[kind])); B = be.WrapTensor(from_bits16(bb, TORCH16[kind]))
+    run = be.Hgemm if kind == "f16" else be.Bf16Gemm
+    for lead in (0, 1, 2):
+        flat = torch.full((lead + (M + 1) * N,), -7.0, device="cuda").to(TORCH16[kind])
+        run(A, B, be.WrapTensor(flat[lead:]), M, N, K)
+        torch.cuda.synchronize()
+        assert np.array_equal(bits16(flat[lead:lead + M * N]).reshape(M, N), want16.reshape(M, N)), lead
+        assert bool((flat[:lead].float() == -7.0).all()) and bool((flat[lead + M * N:].float() == -7.0).all()), lead
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
 def test_half_gemm_ragged_large_shape_takes_the_large_tile(be, kind):
     # 3000 x 3080 x 512: 156 tiles of 256 x 256, chosen automatically; sampled rows against the float64 truth
     M, N, K = 3000, 3080, 512
