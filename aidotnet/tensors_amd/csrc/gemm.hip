@@ -753,8 +753,6 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         }
         return;
     }
-    // (16-bit output: the dispatcher admits only C whose rows start on 4-byte boundaries; N is a multiple of 8 on this path, so
-    // a column pair lies inside or outside the matrix together)
 #pragma unroll
     for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -766,27 +764,14 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = apply_activation(acc[i][j][r] + bias, g.act, g.act_param);
             }
-            if constexpr (Elem<OutT>::BYTES == 2) {
-                // 16-bit output: neighbouring lanes (columns c, c + 1) trade halves of their row pairs, so every lane stores
-                // one 32-bit word (two columns of one row) -- half the store instructions of element-wise stores
-                {
-                    const bool odd = lane & 1;
-                    const uint32_t sel = odd ? 0x03020706u : 0x05040100u;
 #pragma unroll
-                    for (int u = 0; u < 8; u++) {
-                        const uint32_t w = Elem<OutT>::narrow(acc[i][j][2 * u]) | (Elem<OutT>::narrow(acc[i][j][2 * u + 1]) << 16);
-                        const uint32_t x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w, 0xB1, 0xF, 0xF, false);   // lane ^ 1
-                        const uint32_t o = __builtin_amdgcn_perm(x, w, sel);
-                        const int row = m0 + wm * WTM + i * 32 + acc_row(2 * u, h) + (odd ? 1 : 0);
-                        if (col_ok && (!EDGE || row < g.M)) *(uint32_t*)(C + (long long)row * g.ldc + (col & ~1)) = o;
-                    }
-                }
-            } else {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
-                    if (col_ok && (!EDGE || row < g.M)) C[(long long)row * g.ldc + col] = as_u32(acc[i][j][r]);
-                }
+            for (int r = 0; r < 16; r++) {
+                const int row = m0 + wm * WTM + i * 32 + acc_row(r, h);
+                out_t* p = C + (long long)row * g.ldc + col;
+                out_t v;
+                if constexpr (Elem<OutT>::BYTES == 4) v = as_u32(acc[i][j][r]);
+                else v = (out_t)Elem<OutT>::narrow(acc[i][j][r]);
+                if (col_ok && (!EDGE || row < g.M)) *p = v;
             }
         }
 }
@@ -1157,14 +1142,12 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     const bool vec = aligned16(g.A) && aligned16(g.B) && g.lda % E == 0 && g.ldb % E == 0 && g.K % E == 0 &&
                      (TRANSB || g.N % E == 0) && g.sA % E == 0 && g.sB % E == 0;
     auto tiles = [&](int bm, int bn) { return (long long)((g.M + bm - 1) / bm) * ((g.N + bn - 1) / bn) * batch; };
-    // the direct-to-LDS kernel stores 16-bit results as 32-bit column pairs
-    const bool pair_c = Elem<OutT>::BYTES == 4 || (((uintptr_t)g.C & 3) == 0 && g.ldc % 2 == 0 && g.sC % 2 == 0);
     int tile = force_tile;
     if (tile == 0) {
         if constexpr (!TRANSB || E == 4) {
             // the direct-to-LDS kernel: rows of A and B in whole 16-byte chunks, leading dimensions within the 32-bit lane
             // offsets of its loads; M, N and K may be ragged
-            if (vec && pair_c && g.lda < (1 << 21) && g.ldb < (1 << 21) && (Elem<OutT>::BYTES == 4 || (g.alpha == 1.0f && g.beta == 0.0f))) {
+            if (vec && g.lda < (1 << 21) && g.ldb < (1 << 21) && (Elem<OutT>::BYTES == 4 || (g.alpha == 1.0f && g.beta == 0.0f))) {
                 // 16-bit: the 256 x 256 tile moves half the bytes per flop of the 128 x 128 one and wins from half a chip of
                 // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
@@ -1179,7 +1162,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     }
     if constexpr (E == 4 || !TRANSB) {
         if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
-            if (!(vec && pair_c && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
+            if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
             const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % (8 * E) == 0;
             return exact_fit ? launch_gemm_dl<T, OutT, false, 64, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 64, TRANSB>(g, batch, stream);
@@ -1188,7 +1171,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     if (tile == 65) tile = 64;
     if constexpr (!TRANSB || E == 4) {
         if (tile == 256 || tile == 129) {
-            if (!(vec && pair_c && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
+            if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
             const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
