@@ -325,6 +325,9 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             for (int kt = 0; kt < KT; kt++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) st[kt][r] = 0.0f;
+            // fp32: the two MFMA phases run at a raised wave priority, ahead of the other workgroup's softmax on the SIMD (1-3 %
+            // measured; the 16-bit instances lose with it)
+            if constexpr (EB == 4) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int s = 0; s < DSTEPS; s++) {
 #pragma unroll
@@ -335,6 +338,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     Mma32<T>::run(st[kt], kf, qf[s]);
                 }
             }
+            if constexpr (EB == 4) __builtin_amdgcn_s_setprio(0);
 
             // ---- logits in the log2 domain, masks
             const bool need_mask = (kv0 + BC > a.Sk) || (a.causal && (long long)kv0 + BC - 1 > (long long)wq_min + a.qoff);
@@ -390,6 +394,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             }
 
             // ---- O^T += V^T * P^T
+            if constexpr (EB == 4) __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int kt = 0; kt < KT; kt++) {
 #pragma unroll
@@ -432,6 +437,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                     }
                 }
             }
+            if constexpr (EB == 4) __builtin_amdgcn_s_setprio(0);
         }
         if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0);      // this wave's loads of tile j + 1 have landed
         else if (j + 1 < ntiles) store_tile(stage ^ 1);
