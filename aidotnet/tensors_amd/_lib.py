@@ -17,6 +17,7 @@ AIDN_ERR_INVALID_ARGUMENT = 1001
 AIDN_ERR_UNSUPPORTED = 1002
 AIDN_ERR_NO_DEVICE = 1003
 AIDN_ERR_OUT_OF_MEMORY = 1004
+AIDN_ERR_WORKSPACE = 1005
 
 
 class AttnDesc(ctypes.Structure):
@@ -42,6 +43,7 @@ _vp = ctypes.c_void_p
 _i = ctypes.c_int
 _f = ctypes.c_float
 _i64 = ctypes.c_int64
+_u64 = ctypes.c_uint64
 _descp = ctypes.POINTER(AttnDesc)
 
 # name -> (restype, argtypes); every symbol include/aidotnet_mi355.h declares
@@ -83,6 +85,12 @@ SIGNATURES = {
     "aidn_mi355_attn_decode_f32": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_attn_decode_f16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_attn_decode_bf16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
+    "aidn_mi355_mha_pack_qkv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i]),
+    "aidn_mi355_mha_fwd_packed_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_mha_fwd_packed_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_mha_fwd_packed_bf16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_reserve_workspace": (_i, [_vp, _vp, _u64]),
+    "aidn_mi355_workspace_bytes": (_u64, [_vp, _vp]),
     "aidn_mi355_set_gemm_tile": (_i, [_vp, _i]),
     "aidn_mi355_set_attention_fast_path": (_i, [_vp, _i]),
 }

@@ -88,7 +88,11 @@ class Mi355Backend:
 
     BackendName = "HIP-MI355X"
 
-    def __init__(self, device: int = 0, synchronous: bool = True):
+    def __init__(self, device: int = 0, synchronous: bool = True, validate_block_tables: bool = False):
+        # validate_block_tables: read every block table back to the host and check its ids against the pool before a paged
+        # call (a device-to-host copy and a stream synchronisation per call; the reference's guard checks capacities only,
+        # GpuKernelGuards.cs:83-100).  Off by default so that paged calls stay launch-only and can be captured into a graph.
+        self.ValidateBlockTables = validate_block_tables
         self._lib = _lib.load()
         if not torch.cuda.is_available():
             raise InvalidOperationException("no HIP device visible")
@@ -125,6 +129,8 @@ class Mi355Backend:
                 raise ArgumentException(msg)
             if status == _lib.AIDN_ERR_UNSUPPORTED:
                 raise NotSupportedException(msg)
+            if status == _lib.AIDN_ERR_WORKSPACE:
+                raise InvalidOperationException(msg)
             raise HipException(status, msg)
 
     def _done(self) -> None:
@@ -141,6 +147,17 @@ class Mi355Backend:
     def SetAttentionFastPath(self, enabled: bool) -> None:
         """Test hook: False routes every attention shape through the general kernel."""
         self._check(self._lib.aidn_mi355_set_attention_fast_path(self._ctx, 1 if enabled else 0))
+
+    def ReserveWorkspace(self, size_in_bytes: int) -> None:
+        """Grow the library workspace of the current stream now, so that later calls on it allocate nothing (needed before a
+        call sequence is captured into a HIP graph).  No counterpart in the reference."""
+        if size_in_bytes < 0:
+            raise ArgumentOutOfRangeException("size must not be negative")
+        self._check(self._lib.aidn_mi355_reserve_workspace(self._ctx, self._stream(), int(size_in_bytes)))
+
+    def WorkspaceBytes(self) -> int:
+        """Current size of the library workspace of the current stream."""
+        return int(self._lib.aidn_mi355_workspace_bytes(self._ctx, self._stream()))
 
     # buffers -- AllocateBuffer zero-fills (HipBackend.cs:1251-1273)
     def AllocateBuffer(self, data_or_size) -> GpuBuffer:
@@ -369,7 +386,7 @@ class Mi355Backend:
         bt = blockTable.tensor.reshape(-1)[:blocks]
         if bt.dtype != torch.int32:
             raise ArgumentException("%s: blockTable must hold 32-bit block ids." % op)
-        if int(bt.min()) < 0 or int(bt.max()) >= kcache.SizeInBytes // per_block:
+        if self.ValidateBlockTables and (int(bt.min()) < 0 or int(bt.max()) >= kcache.SizeInBytes // per_block):
             raise ArgumentException("%s: blockTable names a block outside the pool." % op)
         out = self.AllocateBuffer(numQueries * heads * headDim)
         if decode:
@@ -455,6 +472,55 @@ class Mi355Backend:
             else:
                 raise ArgumentException("mask must hold seqLen*seqLen or batch*numHeads*seqLen*seqLen floats")
         self._check(fn(self._ctx, self._stream(), input.Handle, qWeight.Handle, kWeight.Handle, vWeight.Handle, outWeight.Handle,
+                       mask.Handle if mask is not None else None, mode, output.Handle, batch, seqLen, dModel, numHeads))
+        self._done()
+
+    def PackQkvWeights(self, kind: str, qWeight: GpuBuffer, kWeight: GpuBuffer, vWeight: GpuBuffer, dModel: int) -> GpuBuffer:
+        """[Wq|Wk|Wv] side by side in one new [dModel, 3 dModel] buffer: the constant operand of the fused QKV projection,
+        packed once instead of on every forward call."""
+        if kind not in ("f32", "f16", "bf16"):
+            raise NotSupportedException("PackQkvWeights: kind must be 'f32', 'f16' or 'bf16'")
+        self._positive(dModel=dModel)
+        es = 4 if kind == "f32" else 2
+        for b, n in ((qWeight, "qWeight"), (kWeight, "kWeight"), (vWeight, "vWeight")):
+            self._capacity(self._need(b, n), dModel * dModel * es, n, "PackQkvWeights")
+        packed = self.AllocateByteBuffer(3 * dModel * dModel * es)
+        self._check(self._lib.aidn_mi355_mha_pack_qkv(self._ctx, self._stream(), qWeight.Handle, kWeight.Handle, vWeight.Handle,
+                                                       packed.Handle, dModel, es))
+        self._done()
+        return packed
+
+    def MultiHeadAttentionForwardPacked(self, kind: str, input: GpuBuffer, qkvWeight: GpuBuffer, outWeight: GpuBuffer,
+                                        mask: Optional[GpuBuffer], output: GpuBuffer,
+                                        batch: int, seqLen: int, dModel: int, numHeads: int) -> None:
+        """MultiHeadAttentionForward on a weight packed by PackQkvWeights (no per-call weight gather)."""
+        fn = {"f32": self._lib.aidn_mi355_mha_fwd_packed_f32, "f16": self._lib.aidn_mi355_mha_fwd_packed_f16,
+              "bf16": self._lib.aidn_mi355_mha_fwd_packed_bf16}.get(kind)
+        if fn is None:
+            raise NotSupportedException("MultiHeadAttentionForwardPacked: kind must be 'f32', 'f16' or 'bf16'")
+        op = "MultiHeadAttentionForwardPacked"
+        for b, n in ((input, "input"), (qkvWeight, "qkvWeight"), (outWeight, "outWeight"), (output, "output")):
+            self._need(b, n)
+        self._positive(batch=batch, seqLen=seqLen, dModel=dModel, numHeads=numHeads)
+        if dModel % numHeads != 0:
+            raise ArgumentException("dModel (%d) must be divisible by numHeads (%d)." % (dModel, numHeads))
+        if dModel // numHeads > 256:
+            raise ArgumentException("head dimension %d exceeds 256" % (dModel // numHeads))
+        es = 4 if kind == "f32" else 2
+        self._capacity(input, batch * seqLen * dModel * es, "input", op)
+        self._capacity(output, batch * seqLen * dModel * es, "output", op)
+        self._capacity(qkvWeight, 3 * dModel * dModel * es, "qkvWeight", op)
+        self._capacity(outWeight, dModel * dModel * es, "outWeight", op)
+        mode = 0
+        if mask is not None:
+            plane = seqLen * seqLen
+            if mask.SizeInBytes == plane * 4:
+                mode = 1
+            elif mask.SizeInBytes == batch * numHeads * plane * 4:
+                mode = 2
+            else:
+                raise ArgumentException("mask must hold seqLen*seqLen or batch*numHeads*seqLen*seqLen floats")
+        self._check(fn(self._ctx, self._stream(), input.Handle, qkvWeight.Handle, outWeight.Handle,
                        mask.Handle if mask is not None else None, mode, output.Handle, batch, seqLen, dModel, numHeads))
         self._done()
 

@@ -59,12 +59,23 @@ def kernels_with_scratch(remarks: str):
     return out
 
 
-def build_library(verbose: bool = False, jobs: int = 5) -> str:
+def _stale(src: str, obj: str) -> bool:
+    """True when `obj` is older than its source or than any header the sources share."""
+    if not os.path.exists(obj):
+        return True
+    deps = [src] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith((".hpp", ".h"))]
+    deps.append(os.path.join(os.path.dirname(os.path.dirname(HERE)), "include", "aidotnet_mi355.h"))
+    return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps if os.path.exists(d))
+
+
+def build_library(verbose: bool = False, jobs: int = 5, incremental: bool = False) -> str:
+    """Compiles every source (always, unless `incremental`: then only those newer than their object file) and links."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
     pairs = [(os.path.join(CSRC, s), os.path.join(objdir, s.replace(".hip", ".o"))) for s in SOURCES]
+    todo = [p for p in pairs if not incremental or _stale(*p)]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        list(ex.map(lambda p: _compile(*p), pairs))
+        list(ex.map(lambda p: _compile(*p), todo))
     tmp = LIB_PATH + ".tmp"
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + [o for _, o in pairs]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -77,4 +88,4 @@ def build_library(verbose: bool = False, jobs: int = 5) -> str:
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv[1:]))

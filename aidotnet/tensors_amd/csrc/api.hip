@@ -6,21 +6,31 @@
 #include "../../../include/aidotnet_mi355.h"
 #include "launch.hpp"
 
+#include <map>
 #include <mutex>
 #include <math.h>
 #include <string>
+#include <vector>
 #include <cstdio>
 #include <cstring>
 
 namespace {
 
+// Library-owned workspace of one stream.  Blocks are never freed before aidn_mi355_destroy: a kernel that is still queued,
+// or a captured graph that holds the address, keeps a valid block when a later call needs a larger one.
+struct WsSlot {
+    void* cur = nullptr;
+    size_t bytes = 0;
+    std::vector<void*> retired;
+};
+
 struct Ctx {
     int device = 0;
     std::mutex mu;
     std::string last_error;
-    void* ws = nullptr;          // library-owned workspace (decode split partials, LSE for weights)
-    size_t ws_bytes = 0;
+    std::map<void*, WsSlot> ws;  // keyed by stream: calls on different streams never share split partials or intermediates
     int force_tile = 0;
+    int attn_fast_path = 1;      // 0: every attention shape takes the general kernel (parity tests hold the two against each other)
 };
 
 int fail(Ctx* c, int code, const char* what)
@@ -44,21 +54,33 @@ int hip_status(Ctx* c, hipError_t e, const char* where)
     return (int)e;
 }
 
-// Grow-only workspace.  Replacing it first drains the device so no queued kernel still uses the old block.
-int ensure_ws(Ctx* c, size_t bytes)
+// Workspace of `stream`, at least `bytes` large.  Growing allocates a new block and keeps the old one until destroy (no
+// synchronisation, nothing queued or captured is invalidated).  While `stream` is being captured into a graph nothing may be
+// allocated: the call fails with AIDN_ERR_WORKSPACE and the caller reserves beforehand (aidn_mi355_reserve_workspace, or one
+// eager call of the same sequence).
+int acquire_ws(Ctx* c, void* stream, size_t bytes, void** out)
 {
     std::lock_guard<std::mutex> g(c->mu);
-    if (bytes <= c->ws_bytes) return AIDN_OK;
-    if (c->ws) {
-        hipError_t e = hipDeviceSynchronize();
-        if (e != hipSuccess) { c->last_error = "workspace: hipDeviceSynchronize failed"; return (int)e; }
-        (void)hipFree(c->ws);
-        c->ws = nullptr; c->ws_bytes = 0;
+    WsSlot& slot = c->ws[stream];
+    if (bytes > slot.bytes) {
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            c->last_error = "workspace: the stream is being captured and its workspace would have to grow; reserve it before the capture";
+            return AIDN_ERR_WORKSPACE;
+        }
+        size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
+        if (want < 2 * slot.bytes) want = 2 * slot.bytes;           // geometric growth bounds what the retired blocks hold
+        want = (want + 255) & ~(size_t)255;
+        void* p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) {
+            (void)hipGetLastError();
+            c->last_error = "workspace: hipMalloc failed";
+            return AIDN_ERR_OUT_OF_MEMORY;
+        }
+        if (slot.cur) slot.retired.push_back(slot.cur);
+        slot.cur = p; slot.bytes = want;
     }
-    size_t want = bytes < (1u << 20) ? (1u << 20) : bytes;
-    void* p = nullptr;
-    if (hipMalloc(&p, want) != hipSuccess) { c->last_error = "workspace: hipMalloc failed"; return AIDN_ERR_OUT_OF_MEMORY; }
-    c->ws = p; c->ws_bytes = want;
+    *out = slot.cur;
     return AIDN_OK;
 }
 
@@ -103,10 +125,12 @@ int attn_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, cons
     if (weights && !lse) {
         // the probabilities are rebuilt from the saved log-sum-exp: borrow the workspace for it
         size_t need = (size_t)p.B * p.H * p.Sq * sizeof(float);
-        st = ensure_ws(c, need);
+        void* ws = nullptr;
+        st = acquire_ws(c, stream, need, &ws);
         if (st) return st;
-        p.lse = (float*)c->ws;
+        p.lse = (float*)ws;
     }
+    p.allow_fast_path = c->attn_fast_path;
     return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "attn_fwd");
 }
 
@@ -121,11 +145,17 @@ int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, co
     if (st) return st;
     if (p.Sq != 1) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "decode: Sq must be 1");
     if (kind == 0 && p.out16) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "decode: fp32 kernel has no 16-bit output");
+    if (p.softcap > 0.0f || p.mask_mode != 0)
+        return fail(c, AIDN_ERR_UNSUPPORTED, "decode: soft-cap and masks are not available here; use aidn_mi355_attn_fwd_* with Sq = 1");
     p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.bias = nullptr; p.mask = nullptr; p.weights = nullptr;
     int eff = aidn::attn_decode_splits(p, splits);
     size_t need = aidn::attn_decode_workspace_bytes(p, eff);
-    if (need) { st = ensure_ws(c, need); if (st) return st; }
-    return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, c->ws), "attn_decode");
+    void* ws = nullptr;
+    if (need) {
+        st = acquire_ws(c, stream, need, &ws);
+        if (st) return st;
+    }
+    return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, ws), "attn_decode");
 }
 
 bool valid_activation(int act) { return act >= 0 && act <= 6; }
@@ -140,23 +170,37 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
     void* ws = nullptr;
     size_t need = c->force_tile == 0 ? aidn::gemm_16_workspace_bytes(M, N, K) : 0;
     if (need) {
-        int st = ensure_ws(c, need);
+        int st = acquire_ws(c, stream, need, &ws);
         if (st) return st;
-        ws = c->ws;
     }
     if (!valid_activation(act)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: unknown activation");
     return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, bias, act, act_param), "gemm_16");
 }
 
+// [Wq|Wk|Wv] side by side in one [dModel, 3 dModel] matrix (three strided device copies), the weight operand of the fused
+// QKV projection.
+hipError_t gather_qkv(hipStream_t sm, const void* wq, const void* wk, const void* wv, void* packed, int dModel, size_t es)
+{
+    const void* w3[3] = {wq, wk, wv};
+    for (int j = 0; j < 3; j++) {
+        hipError_t e = hipMemcpy2DAsync((unsigned char*)packed + (size_t)j * dModel * es, (size_t)3 * dModel * es, w3[j], (size_t)dModel * es,
+                                        (size_t)dModel * es, (size_t)dModel, hipMemcpyDeviceToDevice, sm);
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 // Multi-head attention forward as three launches and no permutes: fused [Wq|Wk|Wv] projection into a packed
 // [B*S, 3*dModel] activation, attention reading it through strides and writing [B, S, H, d], output projection.
 // kind: 0 fp32, 1 fp16, 2 bf16 (16-bit: every intermediate stays in the input type, accumulation in fp32).
-int mha_common(void* ctx, void* stream, int kind, const void* input, const void* wq, const void* wk, const void* wv, const void* wo,
-               const float* mask, int mask_mode, void* output, int B, int S, int dModel, int heads)
+// wqkv non-null: the caller's pre-packed [dModel, 3 dModel] weight (nothing is gathered); else wq, wk, wv are gathered into the
+// workspace on every call.
+int mha_common(void* ctx, void* stream, int kind, const void* input, const void* wq, const void* wk, const void* wv, const void* wqkv,
+               const void* wo, const float* mask, int mask_mode, void* output, int B, int S, int dModel, int heads)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
-    if (!input || !wq || !wk || !wv || !wo || !output)
+    if (!input || !wo || !output || (!wqkv && (!wq || !wk || !wv)))
         return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: input, weights and output must not be null");
     if (B <= 0 || S <= 0 || dModel <= 0 || heads <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: dimensions must be positive");
     if (dModel % heads != 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha: dModel must be divisible by the number of heads");
@@ -168,25 +212,25 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
     if (rows > 0x7FFFFFFFLL || 3LL * dModel > 0x7FFFFFFFLL) return fail(c, AIDN_ERR_UNSUPPORTED, "mha: B*S or 3*dModel exceeds 2^31");
     const size_t es = kind == 0 ? 4 : 2;
     auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
-    const size_t wf_bytes = up((size_t)dModel * 3 * dModel * es), qkv_bytes = up((size_t)rows * 3 * dModel * es);
+    const size_t wf_bytes = wqkv ? 0 : up((size_t)dModel * 3 * dModel * es), qkv_bytes = up((size_t)rows * 3 * dModel * es);
     const size_t cc_bytes = up((size_t)rows * dModel * es);
-    int st = ensure_ws(c, wf_bytes + qkv_bytes + cc_bytes);
+    void* ws = nullptr;
+    int st = acquire_ws(c, stream, wf_bytes + qkv_bytes + cc_bytes, &ws);
     if (st) return st;
-    unsigned char* wf = (unsigned char*)c->ws;
+    unsigned char* wf = (unsigned char*)ws;
     unsigned char* qkv = wf + wf_bytes;
     unsigned char* cc = qkv + qkv_bytes;
     hipStream_t sm = (hipStream_t)stream;
-    const void* w3[3] = {wq, wk, wv};
-    for (int j = 0; j < 3; j++) {
-        hipError_t e = hipMemcpy2DAsync(wf + (size_t)j * dModel * es, (size_t)3 * dModel * es, w3[j], (size_t)dModel * es,
-                                        (size_t)dModel * es, (size_t)dModel, hipMemcpyDeviceToDevice, sm);
+    hipError_t e;
+    if (!wqkv) {
+        e = gather_qkv(sm, wq, wk, wv, wf, dModel, es);
         if (e != hipSuccess) return hip_status(c, e, "mha: weight gather");
     }
+    const void* w3 = wqkv ? wqkv : (const void*)wf;
     const int M = (int)rows, N3 = 3 * dModel;
     const int tile32 = c->force_tile;
-    hipError_t e;
-    if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)wf, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
-    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)wf, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
+    if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)w3, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
+    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)w3, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
     if (e != hipSuccess) return hip_status(c, e, "mha: QKV projection");
 
     aidn::AttnParams p{};
@@ -195,6 +239,7 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
     p.B = B; p.H = heads; p.Hkv = heads; p.Sq = S; p.Sk = S; p.D = dHead;
     p.scale = 1.0f / sqrtf((float)dHead); p.causal = 0; p.qoff = 0; p.softcap = 0.0f; p.mask_mode = mask_mode; p.out16 = kind != 0;
     p.bias_bs = 0;
+    p.allow_fast_path = c->attn_fast_path;
     for (int i = 0; i < 3; i++) { long long v = i == 0 ? (long long)S * N3 : (i == 1 ? dHead : N3); p.qs[i] = v; p.ks[i] = v; p.vs[i] = v; }
     p.os[0] = (long long)S * dModel; p.os[1] = dHead; p.os[2] = dModel;
     e = aidn::attn_fwd(sm, kind, p);
@@ -236,9 +281,11 @@ int paged_common(void* ctx, void* stream, int kind, const void* q, const void* k
     if (decode) {
         int eff = aidn::attn_decode_splits(p, splits);
         size_t need = aidn::attn_decode_workspace_bytes(p, eff);
-        if (need) { int st = ensure_ws(c, need); if (st) return st; }
-        return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, c->ws), "paged attn_decode");
+        void* ws = nullptr;
+        if (need) { int st = acquire_ws(c, stream, need, &ws); if (st) return st; }
+        return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, ws), "paged attn_decode");
     }
+    p.allow_fast_path = c->attn_fast_path;
     return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "paged attn_fwd");
 }
 
@@ -289,7 +336,16 @@ AIDN_API int aidn_mi355_destroy(void* ctx)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_OK;
-    if (c->ws) { (void)hipDeviceSynchronize(); (void)hipFree(c->ws); }
+    bool any = false;
+    for (auto& kv : c->ws) any = any || kv.second.cur;
+    if (any) {
+        (void)hipSetDevice(c->device);
+        (void)hipDeviceSynchronize();
+        for (auto& kv : c->ws) {
+            if (kv.second.cur) (void)hipFree(kv.second.cur);
+            for (void* r : kv.second.retired) (void)hipFree(r);
+        }
+    }
     delete c;
     return AIDN_OK;
 }
@@ -324,21 +380,18 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
 {
     if (!ctx) return AIDN_ERR_INVALID_ARGUMENT;
-    aidn::attn_set_fast_path(enabled);
+    ((Ctx*)ctx)->attn_fast_path = enabled != 0;
     return AIDN_OK;
 }
 
 // workspace of the small-M fp32 path (M <= 8, B [K,N]); *ws stays null when the path does not apply or a tile size is forced
-static int smallm_ws(Ctx* c, int M, int N, int K, int transB, void** ws)
+static int smallm_ws(Ctx* c, void* stream, int M, int N, int K, int transB, void** ws)
 {
     *ws = nullptr;
     if (c->force_tile != 0 || transB) return 0;
     size_t need = aidn::gemm_f32_workspace_bytes(M, N, K);
     if (!need) return 0;
-    int st = ensure_ws(c, need);
-    if (st) return st;
-    *ws = c->ws;
-    return 0;
+    return acquire_ws(c, stream, need, ws);
 }
 
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
@@ -350,7 +403,7 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
     int tile = c->force_tile;
     void* ws = nullptr;
-    if (int st = smallm_ws(c, M, N, K, transB, &ws)) return st;
+    if (int st = smallm_ws(c, stream, M, N, K, transB, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),
                       "gemm_f32");
 }
@@ -379,7 +432,7 @@ AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, 
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: unknown activation");
     int tile = c->force_tile;
     void* ws = nullptr;
-    if (int st = smallm_ws(c, M, N, K, 0, &ws)) return st;
+    if (int st = smallm_ws(c, stream, M, N, K, 0, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param, ws),
                       "gemm_f32 (bias + activation)");
 }
@@ -392,7 +445,7 @@ AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A,
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: unknown activation");
     void* ws = nullptr;
-    if (int st = smallm_ws(c, M, N, K, 0, &ws)) return st;
+    if (int st = smallm_ws(c, stream, M, N, K, 0, &ws)) return st;
     return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param, ws),
                       "gemm_f32_f16weight");
 }
@@ -483,13 +536,58 @@ AIDN_API int aidn_mi355_rope_interleaved_bf16(void* ctx, void* stream, const uin
 
 AIDN_API int aidn_mi355_mha_fwd_f32(void* ctx, void* stream, const float* input, const float* wq, const float* wk, const float* wv,
                            const float* wo, const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads)
-{ return mha_common(ctx, stream, 0, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
+{ return mha_common(ctx, stream, 0, input, wq, wk, wv, nullptr, wo, mask, mask_mode, output, B, S, dModel, heads); }
 AIDN_API int aidn_mi355_mha_fwd_f16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
                            const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
-{ return mha_common(ctx, stream, 1, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
+{ return mha_common(ctx, stream, 1, input, wq, wk, wv, nullptr, wo, mask, mask_mode, output, B, S, dModel, heads); }
 AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
                             const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
-{ return mha_common(ctx, stream, 2, input, wq, wk, wv, wo, mask, mask_mode, output, B, S, dModel, heads); }
+{ return mha_common(ctx, stream, 2, input, wq, wk, wv, nullptr, wo, mask, mask_mode, output, B, S, dModel, heads); }
+
+AIDN_API int aidn_mi355_mha_pack_qkv(void* ctx, void* stream, const void* wq, const void* wk, const void* wv, void* packed,
+                                     int dModel, int elem_bytes)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!wq || !wk || !wv || !packed) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha_pack_qkv: buffers must not be null");
+    if (dModel <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha_pack_qkv: dModel must be positive");
+    if (elem_bytes != 2 && elem_bytes != 4) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "mha_pack_qkv: elem_bytes must be 2 or 4");
+    return hip_status(c, gather_qkv((hipStream_t)stream, wq, wk, wv, packed, dModel, (size_t)elem_bytes), "mha_pack_qkv");
+}
+AIDN_API int aidn_mi355_mha_fwd_packed_f32(void* ctx, void* stream, const float* input, const float* wqkv, const float* wo,
+                                           const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads)
+{
+    if (ctx && !wqkv) return fail((Ctx*)ctx, AIDN_ERR_INVALID_ARGUMENT, "mha (packed): the packed weight must not be null");
+    return mha_common(ctx, stream, 0, input, nullptr, nullptr, nullptr, wqkv, wo, mask, mask_mode, output, B, S, dModel, heads);
+}
+AIDN_API int aidn_mi355_mha_fwd_packed_f16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wqkv, const uint16_t* wo,
+                                           const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
+{
+    if (ctx && !wqkv) return fail((Ctx*)ctx, AIDN_ERR_INVALID_ARGUMENT, "mha (packed): the packed weight must not be null");
+    return mha_common(ctx, stream, 1, input, nullptr, nullptr, nullptr, wqkv, wo, mask, mask_mode, output, B, S, dModel, heads);
+}
+AIDN_API int aidn_mi355_mha_fwd_packed_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wqkv, const uint16_t* wo,
+                                            const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads)
+{
+    if (ctx && !wqkv) return fail((Ctx*)ctx, AIDN_ERR_INVALID_ARGUMENT, "mha (packed): the packed weight must not be null");
+    return mha_common(ctx, stream, 2, input, nullptr, nullptr, nullptr, wqkv, wo, mask, mask_mode, output, B, S, dModel, heads);
+}
+
+AIDN_API int aidn_mi355_reserve_workspace(void* ctx, void* stream, uint64_t bytes)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    void* ws = nullptr;
+    return acquire_ws(c, stream, (size_t)bytes, &ws);
+}
+AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return 0;
+    std::lock_guard<std::mutex> g(c->mu);
+    auto it = c->ws.find(stream);
+    return it == c->ws.end() ? 0 : (uint64_t)it->second.bytes;
+}
 
 AIDN_API int aidn_mi355_attn_decode_f32(void* ctx, void* stream, const aidn_attn_desc* desc, const float* q, const float* k, const float* v,
                                float* o, float* lse, int splits)
@@ -500,5 +598,6 @@ AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn
 AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                 void* o, float* lse, int splits)
 { return decode_common(ctx, stream, 2, desc, q, k, v, o, lse, splits); }
+
 
 }  // extern "C"

@@ -829,12 +829,8 @@ static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
 {
     auto kern = attn_fwd_dl_kernel<T, OutT>;
     constexpr int smem = 2 * (64 * 256 + 64 * 256);
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
     long long nblk = (long long)a.qtiles * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
@@ -888,12 +884,8 @@ static hipError_t launch_attn(AttnArgs a, hipStream_t stream)
     auto kern = attn_fwd_kernel<T, OutT, DP, BC, FULL, MINB, DMA>;
     constexpr int EB = Elem<T>::BYTES;
     constexpr int smem = DMA ? 4 * BC * DP * EB : 2 * (BC * (DP * EB + 16) + DP * (BC * EB + 16));
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
     long long nblk = (long long)a.qtiles * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
@@ -912,13 +904,11 @@ static hipError_t dispatch_attn_d(const AttnArgs& a, bool full, hipStream_t stre
     return hipErrorInvalidValue;
 }
 
-// Test hook: 0 routes every shape through the general kernel.
-bool g_attn_allow_dl = true;
-void attn_set_fast_path(int enabled) { g_attn_allow_dl = enabled != 0; }
 
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
 {
+    const bool g_attn_allow_dl = p.allow_fast_path != 0;      // 0 (test hook of the context): every shape takes the general kernel
     AttnArgs a;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;

@@ -35,6 +35,17 @@ struct GemmArgs {
     float act_param;
 };
 
+hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long* done_mask)
+{
+    int dev = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    const unsigned long long bit = 1ULL << (dev & 63);
+    if (__atomic_load_n(done_mask, __ATOMIC_ACQUIRE) & bit) return hipSuccess;
+    if (hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes)) return e;
+    __atomic_fetch_or(done_mask, bit, __ATOMIC_RELEASE);
+    return hipSuccess;
+}
+
 // Pointwise activations of the fused projection epilogues, numbered like the reference's FusedActivationType
 // (src/AiDotNet.Tensors/Engines/FusedActivationType.cs:23-70) and computed like its HIP activation kernels
 // (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/Kernels/HipActivationKernels.cs:19-70).
@@ -781,12 +792,8 @@ static hipError_t launch_gemm_dl(GemmArgs g, int batch, hipStream_t stream)
 {
     auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE, TRANSB>;
     constexpr int smem = 2 * (TILE * 128 + 128 * TILE);         // A tile + B tile (128 bytes of K each), two stages
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     g.tiles_m = (g.M + TILE - 1) / TILE;
     g.tiles_n = (g.N + TILE - 1) / TILE;
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(TILE == 256 ? 512 : 256), smem, stream, g);
@@ -1106,12 +1113,8 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
     auto kern = gemm_kernel<T, OutT, BM, BN, WM, WN, TRANSB, VEC, CHECK, KS, B16>;
     constexpr int tiles_smem = 2 * (BM + BN) * gemm_row_pitch(BM, BN), merge_smem = KS == 2 ? BM * BN * 4 : 0;
     constexpr int smem = tiles_smem > merge_smem ? tiles_smem : merge_smem;
-    static bool attr_set = false;
-    if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        attr_set = true;
-    }
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch);

@@ -42,11 +42,16 @@ struct AttnParams {
     const int* block_table = nullptr;
     int block_size = 0;
     long long block_table_stride = 0;
+    // 0: every shape takes the general kernel (the direct-to-LDS instances are not used); set per call from the context
+    int allow_fast_path = 1;
 };
+
+// Raises a kernel's dynamic shared-memory limit once per device (the attribute belongs to the device's copy of the function).
+// Safe to call from several threads: the attribute call is idempotent and the done-mask is atomic.
+hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long* done_mask);
 
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p);
-void attn_set_fast_path(int enabled);
 
 // Decode (Sq == 1).  eff_splits: the split count actually used for `splits` requested (<= 0 = auto).
 int attn_decode_splits(const AttnParams& p, int splits);

@@ -39,31 +39,50 @@ TRAFFIC_BYTES = {
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PEAK_HBM_GBS = 8000.0
-# untimed warm-up of every secondary configuration lasts at least this long (their steps are tens of microseconds)
-OTHERS_MIN_WARM_MS = 60.0
+# the untimed warm-up of every configuration lasts at least this long, whatever --warmup says (outside the timed region)
+MIN_WARM_MS = 60.0
 
 
-def _events_time(torch, fn, steps, warmup, min_warm_ms=0.0):
-    """`warmup` untimed steps, continued until `min_warm_ms` of wall time has passed (short kernels need some tens of
-    milliseconds of their own load before the clock management of the device settles), then exactly `steps` timed steps."""
+def _sclk_mhz():
+    """Engine clock the driver reports right now (MHz), or None: the line of pp_dpm_sclk marked with '*'."""
+    import glob
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+        try:
+            for line in open(path):
+                if "*" in line:
+                    return int(line.split(":")[1].strip().lower().split("mhz")[0])
+        except (OSError, ValueError, IndexError):
+            continue
+    return None
+
+
+def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
+    """`warmup` untimed steps, continued until `min_warm_ms` of wall time has passed (a launch sequence needs some tens of
+    milliseconds of its own load before the clock management of the device settles), then exactly `steps` timed steps.
+    Every step is bracketed by its own pair of events on the launch stream: returns the mean over the whole timed region
+    (first event to last), the wall-clock mean, and the median / 95th percentile / spread of the single steps."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
     t_warm = time.perf_counter()
     while (time.perf_counter() - t_warm) * 1e3 < min_warm_ms:
-        for _ in range(50):
+        for _ in range(10):
             fn()
         torch.cuda.synchronize()
-    start = torch.cuda.Event(enable_timing=True)
-    end = torch.cuda.Event(enable_timing=True)
+    clk0 = _sclk_mhz()
+    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
     t0 = time.perf_counter()
-    start.record()
-    for _ in range(steps):
+    evs[0].record()
+    for i in range(steps):
         fn()
-    end.record()
+        evs[i + 1].record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return start.elapsed_time(end) / steps, wall_ms
+    clk1 = _sclk_mhz()
+    per = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(steps))
+    stats = {"median_ms": round(per[len(per) // 2], 5), "p95_ms": round(per[min(len(per) - 1, int(math.ceil(0.95 * len(per))) - 1)], 5),
+             "min_ms": round(per[0], 5), "max_ms": round(per[-1], 5), "sclk_mhz_before_after": [clk0, clk1]}
+    return evs[0].elapsed_time(evs[steps]) / steps, wall_ms, stats
 
 
 def _roof_flops(kind, flops, ms, traffic=None):
@@ -116,7 +135,7 @@ def main() -> int:
     b = randn(n, n, std=0.02, kind="f16")
     c = torch.empty(n, n, device="cuda", dtype=torch.float16)
     A, B, C = W(a), W(b), W(c)
-    ms, wall_ms = _events_time(torch, lambda: be.Hgemm(A, B, C, n, n, n), steps, warmup)
+    ms, wall_ms, stats = _events_time(torch, lambda: be.Hgemm(A, B, C, n, n, n), steps, warmup)
     flops = 2.0 * n * n * n
     value = flops / (ms * 1e-3) / 1e12
     out = {
@@ -124,7 +143,8 @@ def main() -> int:
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "fp16 GEMM C=A*B, M=N=K=8192, fp32 accumulate, fp16 out (A~N(0,1), B~N(0,0.02^2), seeded)",
-                   "wall_ms_per_step": round(wall_ms, 5)},
+                   "wall_ms_per_step": round(wall_ms, 5), "min_warmup_ms": MIN_WARM_MS},
+        "step_stats": stats,
         "roofline": _roof_flops("f16", flops, ms, TRAFFIC_BYTES.get("gemm_f16_8192")),
     }
     del a, b, c
@@ -136,8 +156,9 @@ def main() -> int:
     def want(name):
         return not only or name in only
 
-    def add(name, kind, workload, ms, roof):
-        others.append({"name": name, "dtype": kind, "workload": workload, "ms_per_step": round(ms, 5), "roofline": roof})
+    def add(name, kind, workload, ms, roof, stats):
+        others.append({"name": name, "dtype": kind, "workload": workload, "ms_per_step": round(ms, 5), "roofline": roof,
+                       "step_stats": stats})
 
     def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02):
         if not want(name):
@@ -159,7 +180,7 @@ def main() -> int:
 
         def fn():
             fn1(Bs[it[0] % rotate]); it[0] += 1
-        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
+        ms_, _, st_ = _events_time(torch, fn, steps, warmup)
         fl = 2.0 * M * N * K
         if hbm:
             eb = a_.element_size()
@@ -169,7 +190,7 @@ def main() -> int:
             roof["note"] = "%d weight matrices rotated to defeat the last-level cache" % rotate
         else:
             roof = _roof_flops(kind, fl, ms_)
-        add(name, kind, "GEMM M=%d N=%d K=%d%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else ""), ms_, roof)
+        add(name, kind, "GEMM M=%d N=%d K=%d%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else ""), ms_, roof, st_)
 
     def attn_case(name, kind, Bn, H, S, D):
         if not want(name):
@@ -181,11 +202,11 @@ def main() -> int:
             fn = lambda: be.FlashAttentionV2(W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, sc, True)
         else:
             fn = lambda: be.FlashAttentionHalf(kind, W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, sc, True)
-        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
+        ms_, _, st_ = _events_time(torch, fn, steps, warmup)
         exact = 4.0 * Bn * H * D * (S * (S + 1) / 2)
         roof = _roof_flops(kind, exact, ms_, TRAFFIC_BYTES.get(name))
         roof["tflops_full_matrix_convention"] = round(4.0 * Bn * H * S * S * D / (ms_ * 1e-3) / 1e12, 3)
-        add(name, kind, "causal attention B=%d H=%d S=%d d=%d (fp32 softmax/accumulate, fp32 O + LSE)" % (Bn, H, S, D), ms_, roof)
+        add(name, kind, "causal attention B=%d H=%d S=%d d=%d (fp32 softmax/accumulate, fp32 O + LSE)" % (Bn, H, S, D), ms_, roof, st_)
 
     def decode_case(name, kind, Bn, H, S, D):
         if not want(name):
@@ -194,9 +215,9 @@ def main() -> int:
         o = torch.empty(Bn, H, 1, D, device="cuda")
         sc = 1.0 / math.sqrt(D)
         fn = lambda: be.DecodeAttention(kind, W(q), W(k), W(v), W(o), Bn, H, S, D, sc)
-        ms_, _ = _events_time(torch, fn, steps, warmup, OTHERS_MIN_WARM_MS)
+        ms_, _, st_ = _events_time(torch, fn, steps, warmup)
         nbytes = 2.0 * Bn * H * S * D * q.element_size()
-        add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)))
+        add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)), st_)
 
     gemm_case("gemm_f32_1024", "f32", 1024, 1024, 1024, wstd=1.0)
     gemm_case("gemm_f32_proj", "f32", 4096, 3072, 768)
@@ -218,28 +239,48 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    # ------------------------------------------------------------------ CPU baseline (bounded sample, about 20 s of host time)
     if not args.no_cpu:
         try:
             import numpy as np
             import oracle      # test infrastructure: used here only as the reported CPU baseline
             threads = min(oracle.max_threads(), os.cpu_count() or 1)
-            ms_rows = 8192     # the whole 8192^3 product, fp32 path on widened inputs (about 2 s per pass on 16 cores)
             rng = np.random.default_rng(0)
-            ah = rng.standard_normal((ms_rows, n)).astype(np.float16).astype(np.float32)
+
+            def median_time(fn, reps):
+                ts = []
+                for _ in range(reps):
+                    t0 = time.perf_counter(); fn(); ts.append(time.perf_counter() - t0)
+                return sorted(ts)[len(ts) // 2]
+
+            # headline workload, all host threads: the whole 8192^3 product, fp32 path on fp16-rounded inputs
+            ah = rng.standard_normal((n, n)).astype(np.float16).astype(np.float32)
             bh = (0.02 * rng.standard_normal((n, n))).astype(np.float16).astype(np.float32)
             oracle.sgemm(ah[:256], bh, 256, n, n, threads=threads)    # warm-up
-            times = []
-            for _ in range(5):
-                t0 = time.perf_counter()
-                oracle.sgemm(ah, bh, ms_rows, n, n, threads=threads)
-                times.append(time.perf_counter() - t0)
-            tsec = sorted(times)[len(times) // 2]
+            tsec = median_time(lambda: oracle.sgemm(ah, bh, n, n, n, threads=threads), 5)
+            # the same product on ONE thread, on a 256-row slab
+            rows1 = 256
+            oracle.sgemm(ah[:64], bh, 64, n, n, threads=1)
+            t1 = median_time(lambda: oracle.sgemm(ah[:rows1], bh, rows1, n, n, threads=1), 3)
+            # causal fp32 attention B8 H12 S512 d64 (the reference's per-(batch, head) loop of two SGEMMs around a softmax)
+            Bn, Hn, Sn, Dn = 8, 12, 512, 64
+            qa, ka, va = (rng.standard_normal((Bn, Hn, Sn, Dn)).astype(np.float32) for _ in range(3))
+            oracle.attention_f32(qa, ka, va, 1.0 / math.sqrt(Dn), True, threads=threads)
+            ta = median_time(lambda: oracle.attention_f32(qa, ka, va, 1.0 / math.sqrt(Dn), True, threads=threads), 5)
+            ta1 = median_time(lambda: oracle.attention_f32(qa[:1], ka[:1], va[:1], 1.0 / math.sqrt(Dn), True, threads=1), 3)
+            attn_flops = 4.0 * Bn * Hn * Dn * (Sn * (Sn + 1) / 2)
             out["cpu_baseline"] = {
-                "value": round(2.0 * ms_rows * n * n / tsec / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
-                "sample": "C restatement of the reference SimdGemm (6x16 AVX2 FMA tile, Kc=512, 2-D tile parallelism) on a "
-                          "%d-row slab of the 8192^3 product (%d x 8192 x 8192, fp32 path on fp16-rounded inputs), "
-                          "median of 5, %.2f s each" % (ms_rows, ms_rows, tsec),
+                "value": round(2.0 * n * n * n / tsec / 1e12, 4), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+                "sample": "C restatement of the reference SimdGemm (6x16 AVX2 FMA tile, Kc=512, 2-D tile parallelism) on the whole "
+                          "8192 x 8192 x 8192 product (fp32 path on fp16-rounded inputs), median of 5, %.2f s each" % tsec,
+                "one_thread": {"value": round(2.0 * rows1 * n * n / t1 / 1e12, 5), "unit": "TFLOP/s", "cores": 1,
+                               "sample": "%d-row slab of the same product, median of 3, %.2f s each" % (rows1, t1)},
+                "attention_f32_causal_B8_H12_S512_d64": {
+                    "value": round(attn_flops / ta / 1e12, 5), "unit": "TFLOP/s (causal-exact FLOPs)", "cores": threads,
+                    "ms": round(ta * 1e3, 3),
+                    "one_thread_value": round(attn_flops / Bn / ta1 / 1e12, 5),
+                    "sample": "C restatement of CpuEngine.FlashAttentionFloat (explicit K^T, two sequential SGEMMs per head around a "
+                              "scalar-expf softmax, parallel over batch x head), median of 5; one thread: batch 0 only, median of 3"},
             }
         except Exception as ex:     # the baseline is a reported extra, never the product path
             out["cpu_baseline"] = {"value": None, "unit": "TFLOP/s", "cores": 0, "kind": "port", "sample": "failed: %r" % (ex,)}

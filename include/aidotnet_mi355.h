@@ -38,13 +38,18 @@ enum {
     AIDN_ERR_INVALID_ARGUMENT = 1001,   /* null pointer, non-positive dimension, bad ratio */
     AIDN_ERR_UNSUPPORTED = 1002,        /* e.g. head dimension the kernels do not cover */
     AIDN_ERR_NO_DEVICE = 1003,          /* no gfx950 device */
-    AIDN_ERR_OUT_OF_MEMORY = 1004       /* library-owned workspace could not be allocated */
+    AIDN_ERR_OUT_OF_MEMORY = 1004,      /* library-owned workspace could not be allocated */
+    AIDN_ERR_WORKSPACE = 1005           /* the workspace would have to grow while the stream is being captured */
 };
 
 /* ---- lifetime ------------------------------------------------------------------------------
  * One context per backend instance (the reference creates one stream + one hipBLAS handle per
  * HipBackend, HipBackend.cs:246, 288, 371).  The context owns only the library's private
- * workspace (split-KV partials); it is released by aidn_mi355_destroy. */
+ * workspace (split-KV and split-K partials, intermediates of the fused MHA forward), one per stream
+ * the context has been called on, so calls on different streams never share it; it grows on demand
+ * (a block that has been handed to a kernel is never freed before aidn_mi355_destroy, so queued work
+ * and captured graphs keep valid addresses) and is released by aidn_mi355_destroy.  Calls on the SAME
+ * stream run in order and may share it.  The context may be used from several host threads. */
 AIDN_API int aidn_mi355_create(int device, void** ctx);
 AIDN_API int aidn_mi355_destroy(void* ctx);
 /* Text of the last failure on this context (never NULL; empty when none). */
@@ -52,6 +57,13 @@ AIDN_API const char* aidn_mi355_last_error(void* ctx);
 AIDN_API const char* aidn_mi355_version(void);
 /* hipStreamSynchronize(stream): replaces HipBackend.Synchronize (HipBackend.cs:1444-1446). */
 AIDN_API int aidn_mi355_sync(void* ctx, void* stream);
+/* Makes the workspace of `stream` at least `bytes` large now, so that later calls on it allocate nothing -- required before
+ * the calls are captured into a HIP graph (no allocation can happen during capture: such a call returns AIDN_ERR_WORKSPACE);
+ * one eager run of the same call sequence has the same effect.  aidn_mi355_workspace_bytes reads the current size (after a
+ * warm-up run: the amount to reserve on another stream or context).  No counterpart in the reference, whose backend allocates
+ * per call from its buffer pool (HipBackend.cs:12214-12270). */
+AIDN_API int aidn_mi355_reserve_workspace(void* ctx, void* stream, uint64_t bytes);
+AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream);
 
 /* ---- fp32 GEMM -------------------------------------------------------------------------------
  * C[M,N] = alpha * A[M,K] * op(B) + beta * C.  transB == 0: B is [K,N]; transB != 0: B is stored
@@ -150,8 +162,10 @@ AIDN_API int aidn_mi355_convert_bf16_to_f32(void* ctx, void* stream, const uint1
  * 16-bit variants: q, k, v are fp16 / bf16 patterns, softmax and accumulation are fp32, the output
  * is fp32 (out_is_16bit == 0; the reference's only reduced-precision attention contract: fp16 in,
  * fp32 O and LSE out, Engines/DirectGpuTensorEngine.cs:11143-11167) or the input type
- * (out_is_16bit != 0).  D must be a multiple of 16 (16-bit) / 8 (fp32) and at most 256
- * (GpuKernelGuards.MaxHeadDim, Engines/DirectGpu/GpuKernelGuards.cs:12), else AIDN_ERR_UNSUPPORTED.
+ * (out_is_16bit != 0).  Any 1 <= D <= 256 is accepted (GpuKernelGuards.MaxHeadDim,
+ * Engines/DirectGpu/GpuKernelGuards.cs:12; larger: AIDN_ERR_UNSUPPORTED); rows whose start and strides
+ * are multiples of 16 bytes take the vector loads, head dimensions 64 and 128 with such rows the
+ * direct-to-LDS kernels.
  */
 typedef struct aidn_attn_desc {
     int32_t B, H, Hkv, Sq, Sk, D;
@@ -183,7 +197,8 @@ AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_d
  * workgroups (coalesced 128-bit loads), partial (max, sum, acc) triples are merged by a second
  * kernel from a library-owned workspace.  Same descriptor (Sq must be 1; with causal != 0 keys
  * j > causal_query_offset are masked, so offset Sk - 1, the bottom-right rule, attends to the whole
- * cache; bias, mask and soft-cap are not available here); strides select the cache
+ * cache; bias, mask and soft-cap are not available here: a descriptor with softcap > 0 or
+ * mask_mode != 0 is refused with AIDN_ERR_UNSUPPORTED -- use aidn_mi355_attn_fwd_* with Sq = 1 for those); strides select the cache
  * layout: [B,Hkv,Sk,D] (dense), the reference's decode layout [Sk,Hkv,D]
  * (HipFlashDecodeKernels.cs:9-10; host FlashDecode HipBackend.cs:919-965) or its dense KVCache
  * [B,Sk,Hkv,D] (Engines/Autodiff/KVCache.cs:5-8).  splits <= 0 picks the split count
@@ -249,6 +264,18 @@ AIDN_API int aidn_mi355_mha_fwd_f16(void* ctx, void* stream, const uint16_t* inp
                            const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
 AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wq, const uint16_t* wk, const uint16_t* wv,
                             const uint16_t* wo, const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
+/* The forms above gather [Wq|Wk|Wv] into the workspace on every call (3 dModel^2 elements read and written).  For constant
+ * weights, pack once into a caller-owned [dModel, 3 dModel] buffer (elem_bytes 4 for fp32, 2 for fp16 / bf16) and call the
+ * *_packed forms, which read it in place: the concatenated weight of SimdGemm.SgemmConcatenatedProjections
+ * (Engines/Simd/SimdGemm.NParallelSmallM.cs:95-109) and of the fused QKV GEMM in CpuEngine.MultiHeadAttention.cs:358-420. */
+AIDN_API int aidn_mi355_mha_pack_qkv(void* ctx, void* stream, const void* wq, const void* wk, const void* wv, void* packed,
+                            int dModel, int elem_bytes);
+AIDN_API int aidn_mi355_mha_fwd_packed_f32(void* ctx, void* stream, const float* input, const float* wqkv, const float* wo,
+                                  const float* mask, int mask_mode, float* output, int B, int S, int dModel, int heads);
+AIDN_API int aidn_mi355_mha_fwd_packed_f16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wqkv, const uint16_t* wo,
+                                  const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
+AIDN_API int aidn_mi355_mha_fwd_packed_bf16(void* ctx, void* stream, const uint16_t* input, const uint16_t* wqkv, const uint16_t* wo,
+                                   const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
 
 /* ---- test / tuning hook --------------------------------------------------------------------------------
  * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel; 0 = automatic
@@ -256,7 +283,7 @@ AIDN_API int aidn_mi355_mha_fwd_bf16(void* ctx, void* stream, const uint16_t* in
  * reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
 /* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast
- * path is then not taken), so the parity suite can hold the two kernels against each other.  Process-wide.
+ * path is then not taken), so the parity suite can hold the two kernels against each other.  Per context.
  * No counterpart in the reference. */
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled);
 

@@ -17,7 +17,7 @@ HEADER = os.path.join(ROOT, "include", "aidotnet_mi355.h")
 
 def _declared():
     text = open(HEADER).read()
-    return sorted(set(re.findall(r"AIDN_API\s+(?:const\s+char\*|int)\s+(aidn_mi355_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"AIDN_API\s+(?:const\s+char\*|int|uint64_t)\s+(aidn_mi355_\w+)\s*\(", text)))
 
 
 def test_library_exists_in_tree():
