@@ -1,4 +1,4 @@
-"""The entry points are launch-only once the context workspace is sized: a decode step (three skinny projections, RoPE,
+"""The entry points are launch-only once the workspace of the stream is sized: a decode step (three skinny projections, RoPE,
 decode attention, output projection) is captured into a HIP graph and replayed; every replay must equal the eager result.
 Between replays the program does its own eager work and synchronises, and the inputs change, so stale-node effects show."""
 import math
@@ -33,12 +33,17 @@ def test_decode_step_under_hip_graph_matches_eager():
         be.DecodeAttention("bf16", W(q), W(kc), W(vc), W(att), B, H, S, D, 1 / math.sqrt(D), Hkv, 0, True)
         be.Bf16Gemm(W(att), W(wo), W(y), B, dM, H * D)                                      # output projection
 
-    step(); torch.cuda.synchronize()                      # sizes the context workspace; nothing allocates after this
+    step(); torch.cuda.synchronize()                      # an eager run: sizes the workspace of the stream it ran on
     eager = y.clone()
+    need = be.WorkspaceBytes()
+    assert need > 0
 
     side = torch.cuda.Stream()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
+        # the workspace is per stream: the capture stream gets its own, reserved before the capture (nothing may be
+        # allocated while capturing)
+        be.ReserveWorkspace(need)
         with torch.cuda.graph(graph, stream=side):
             step()
     for it in range(4):
