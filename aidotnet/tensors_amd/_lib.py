@@ -85,6 +85,7 @@ SIGNATURES = {
     "aidn_mi355_attn_decode_f32": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_attn_decode_f16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_attn_decode_bf16": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
+    "aidn_mi355_attn_decode_bf16_noalloc": (_i, [_vp, _vp, _descp, _vp, _vp, _vp, _vp, _vp, _i]),
     "aidn_mi355_mha_pack_qkv": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i]),
     "aidn_mi355_mha_fwd_packed_f32": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),
     "aidn_mi355_mha_fwd_packed_f16": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _i, _i, _i, _i]),

@@ -675,9 +675,14 @@ class Mi355Backend:
         self._attn(kind, query, key, value, output, softmaxStats, None, None, None, d)
 
     # ------------------------------------------------------------------ decode
-    def _decode(self, kind, q, k, v, o, lse, desc, splits):
-        fn = {"f32": self._lib.aidn_mi355_attn_decode_f32, "f16": self._lib.aidn_mi355_attn_decode_f16,
-              "bf16": self._lib.aidn_mi355_attn_decode_bf16}[kind]
+    def _decode(self, kind, q, k, v, o, lse, desc, splits, no_alloc=False):
+        if no_alloc:
+            if kind != "bf16":
+                raise NotSupportedException("the allocation-free decode entry point exists for bf16 only")
+            fn = self._lib.aidn_mi355_attn_decode_bf16_noalloc
+        else:
+            fn = {"f32": self._lib.aidn_mi355_attn_decode_f32, "f16": self._lib.aidn_mi355_attn_decode_f16,
+                  "bf16": self._lib.aidn_mi355_attn_decode_bf16}[kind]
         self._check(fn(self._ctx, self._stream(), ctypes.byref(desc), q.Handle, k.Handle, v.Handle, o.Handle,
                        lse.Handle if lse is not None else None, splits))
         self._done()
@@ -711,7 +716,7 @@ class Mi355Backend:
     def DecodeAttention(self, kind: str, q: GpuBuffer, k: GpuBuffer, v: GpuBuffer, output: GpuBuffer,
                         batch: int, numHeads: int, seqK: int, headDim: int, scale: float,
                         numKVHeads: int = 0, splits: int = 0, outputIs16Bit: bool = False,
-                        softmaxStats: Optional[GpuBuffer] = None, kvLayout: str = "bhsd") -> None:
+                        softmaxStats: Optional[GpuBuffer] = None, kvLayout: str = "bhsd", noAlloc: bool = False) -> None:
         """Batched decode: q [B,H,1,d]; the KV cache [B,Hkv,S,d] ("bhsd") or the reference's dense
         KVCache layout [B,S,Hkv,d] ("bshd", src/AiDotNet.Tensors/Engines/Autodiff/KVCache.cs:5-8).
         What ScaledDotProductAttention with seqQ = 1 computes (bottom-right causal = all keys);
@@ -739,4 +744,5 @@ class Mi355Backend:
             d.v_strides[:] = [seqK * kvHeads * headDim, headDim, kvHeads * headDim]
         elif kvLayout != "bhsd":
             raise ArgumentException("kvLayout must be 'bhsd' or 'bshd'")
-        self._decode(kind, q, k, v, output, softmaxStats, d, splits)
+        # noAlloc: the bf16 entry point whose split partials live in the library's static device array (never allocates)
+        self._decode(kind, q, k, v, output, softmaxStats, d, splits, no_alloc=noAlloc)

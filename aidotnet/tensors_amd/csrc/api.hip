@@ -16,6 +16,15 @@
 
 namespace {
 
+// Scratch memory of the allocation-free decode entry point (aidn_mi355_attn_decode_bf16_noalloc): the split-KV partials
+// (m, l, acc[D]) per (batch, head, split).  One copy per device, held until the process ends; its device address is looked
+// up once per device in aidn_mi355_create and only that address -- never the array's name -- is used by host code.
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};      // device address of `scratch` on each device (null = not looked up yet)
+std::mutex g_scratch_mu;
+
 // Library-owned workspace of one stream.  Blocks are never freed before aidn_mi355_destroy: a kernel that is still queued,
 // or a captured graph that holds the address, keeps a valid block when a later call needs a larger one.
 struct WsSlot {
@@ -134,8 +143,9 @@ int attn_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, cons
     return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "attn_fwd");
 }
 
+// scratch_override: non-null = split partials go there (capacity scratch_bytes) and nothing is allocated
 int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, const void* q, const void* k, const void* v,
-                  void* o, float* lse, int splits)
+                  void* o, float* lse, int splits, void* scratch_override = nullptr, size_t scratch_bytes = 0)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
@@ -151,7 +161,11 @@ int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, co
     int eff = aidn::attn_decode_splits(p, splits);
     size_t need = aidn::attn_decode_workspace_bytes(p, eff);
     void* ws = nullptr;
-    if (need) {
+    if (scratch_override) {
+        if (need > scratch_bytes)
+            return fail(c, AIDN_ERR_UNSUPPORTED, "decode (allocation-free): batch x heads x splits x head dimension exceeds the static scratch buffer");
+        ws = scratch_override;
+    } else if (need) {
         st = acquire_ws(c, stream, need, &ws);
         if (st) return st;
     }
@@ -326,6 +340,16 @@ AIDN_API int aidn_mi355_create(int device, void** ctx)
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return AIDN_ERR_NO_DEVICE;   // the code object holds gfx950 ISA only
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) return (int)e;
+    if (device < kMaxDevices) {
+        // device address of this device's copy of the static scratch array, looked up once with the device current
+        std::lock_guard<std::mutex> g(g_scratch_mu);
+        if (!g_scratch_ptr[device]) {
+            void* ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            g_scratch_ptr[device] = ptr;
+        }
+    }
     Ctx* c = new Ctx();
     c->device = device;
     *ctx = c;
@@ -599,5 +623,17 @@ AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_att
                                 void* o, float* lse, int splits)
 { return decode_common(ctx, stream, 2, desc, q, k, v, o, lse, splits); }
 
+
+// Allocation-free form of aidn_mi355_attn_decode_bf16: the split-KV partials live in the static device array `scratch`
+// (through its per-device address), so the call never touches hipMalloc / hipFree.
+AIDN_API int aidn_mi355_attn_decode_bf16_noalloc(void* ctx, void* stream, const aidn_attn_desc* desc, const uint16_t* q, const uint16_t* k,
+                                                 const uint16_t* v, void* o, float* lse, int splits)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    void* ptr = c->device < kMaxDevices ? g_scratch_ptr[c->device] : nullptr;
+    if (!ptr) return fail(c, AIDN_ERR_UNSUPPORTED, "decode (allocation-free): no static scratch buffer on this device");
+    return decode_common(ctx, stream, 2, desc, q, k, v, o, lse, splits, ptr, kStaticScratchBytes);
+}
 
 }  // extern "C"

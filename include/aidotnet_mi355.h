@@ -210,6 +210,15 @@ AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn
                                const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
 AIDN_API int aidn_mi355_attn_decode_bf16(void* ctx, void* stream, const aidn_attn_desc* desc,
                                 const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
+/* aidn_mi355_attn_decode_bf16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): same arguments and results, but the split-KV partials live in a static 8 MiB
+ * device array of the library instead of the context workspace, so the call never allocates or frees.  Problems whose partials
+ * (B * H * splits * (2 + head dimension padded to a power-of-two number of 16-byte chunks) floats) exceed 8 MiB are refused with
+ * AIDN_ERR_UNSUPPORTED.  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different
+ * streams) race; calls on one stream are ordered.  Nothing in the array has to start at zero.  No counterpart in the
+ * reference. */
+AIDN_API int aidn_mi355_attn_decode_bf16_noalloc(void* ctx, void* stream, const aidn_attn_desc* desc,
+                                        const uint16_t* q, const uint16_t* k, const uint16_t* v, void* o, float* lse, int splits);
 
 /* ---- attention over a paged K/V cache --------------------------------------------------------------------
  * K and V pools [numBlocks, blockSize, kvHeads, headDim]; block_table[i] = pool block of logical block i (int32, at least
