@@ -15,7 +15,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "libaidotnet_mi355.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["gemm.hip", "attention.hip", "decode.hip", "convert.hip", "api.hip"]
+# (source, object name, extra flags): gemm.hip is compiled in three parts so that its template instances build in parallel
+SOURCES = [("gemm.hip", "gemm.o", ["-DAIDN_GEMM_PART=0"]), ("gemm.hip", "gemm_f16.o", ["-DAIDN_GEMM_PART=1"]),
+           ("gemm.hip", "gemm_bf16.o", ["-DAIDN_GEMM_PART=2"]), ("attention.hip", "attention.o", []), ("decode.hip", "decode.o", []),
+           ("convert.hip", "convert.o", []), ("api.hip", "api.o", [])]
 # -packed-fp32-ops off: packed fp32 VALU forms are kept out of all device code.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
@@ -28,10 +31,10 @@ def _hipcc() -> str:
     return "hipcc"
 
 
-def _compile(src: str, obj: str) -> None:
+def _compile(src: str, obj: str, extra=()) -> None:
     # the resource-usage remarks name every kernel with its register and scratch use: a kernel that needs scratch memory has
     # spilled registers (for the GEMM kernels that means accumulators in memory and a 30-fold slowdown), so the build refuses it
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-Rpass-analysis=kernel-resource-usage", "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, r.stderr[-4000:]))
@@ -68,16 +71,16 @@ def _stale(src: str, obj: str) -> bool:
     return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps if os.path.exists(d))
 
 
-def build_library(verbose: bool = False, jobs: int = 5, incremental: bool = False) -> str:
+def build_library(verbose: bool = False, jobs: int = 7, incremental: bool = False) -> str:
     """Compiles every source (always, unless `incremental`: then only those newer than their object file) and links."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
-    pairs = [(os.path.join(CSRC, s), os.path.join(objdir, s.replace(".hip", ".o"))) for s in SOURCES]
-    todo = [p for p in pairs if not incremental or _stale(*p)]
+    pairs = [(os.path.join(CSRC, s), os.path.join(objdir, o), x) for s, o, x in SOURCES]
+    todo = [p for p in pairs if not incremental or _stale(p[0], p[1])]
     with ThreadPoolExecutor(max_workers=jobs) as ex:
         list(ex.map(lambda p: _compile(*p), todo))
     tmp = LIB_PATH + ".tmp"
-    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + [o for _, o in pairs]
+    cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp] + [o for _, o, _ in pairs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s" % r.stderr[-4000:])

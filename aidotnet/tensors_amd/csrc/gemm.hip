@@ -20,6 +20,12 @@
 #include "launch.hpp"
 #include <type_traits>
 
+// This file is compiled three times (the build passes -DAIDN_GEMM_PART=0/1/2) so that its template instances build in
+// parallel: part 0 holds the fp32 entry points and everything that exists once, part 1 the fp16 and part 2 the bf16 instances.
+#ifndef AIDN_GEMM_PART
+#define AIDN_GEMM_PART 0
+#endif
+
 namespace aidn {
 
 struct GemmArgs {
@@ -35,6 +41,7 @@ struct GemmArgs {
     float act_param;
 };
 
+#if AIDN_GEMM_PART == 0
 hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long* done_mask)
 {
     int dev = 0;
@@ -45,6 +52,7 @@ hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long
     __atomic_fetch_or(done_mask, bit, __ATOMIC_RELEASE);
     return hipSuccess;
 }
+#endif
 
 // Pointwise activations of the fused projection epilogues, numbered like the reference's FusedActivationType
 // (src/AiDotNet.Tensors/Engines/FusedActivationType.cs:23-70) and computed like its HIP activation kernels
@@ -801,6 +809,243 @@ static hipError_t launch_gemm_dl(GemmArgs g, int batch, hipStream_t stream)
 }
 
 // ---------------------------------------------------------------------------------------------
+// 256 x 256 x 64 direct-to-LDS kernel for 16-bit inputs on v_mfma_f32_16x16x32 (the form the large exact-fit problems take:
+// M % 256 == 0, N % 256 == 0, K % 64 == 0, B stored [K,N]).  Same tile, loads and LDS layout as gemm_dl_kernel<.., 256>; what
+// differs is the matrix instruction.  Under load this part runs at the clock its power limit allows, and per multiply-add the
+// 16 x 16 x 32 instruction moves 20 % fewer register bytes than 32 x 32 x 16 (half the accumulator traffic, twice the
+// operand traffic): with random fp16 operands and nothing else running it sustains 1.71 PFLOP/s against 1.52, and this kernel
+// 7-10 % more than the 32 x 32 x 16 one on the same box.
+//   * wave tile 128 x 64 = 8 x 4 blocks of 16 x 16, 128 accumulator registers; per 32 k: 8 A fragments (ds_read_b128: row
+//     16 i + lane % 16, 16-byte chunk lane / 16) and 4 B fragments (two transposing reads each), 32 MFMAs of 16 cycles.
+//   * a K-tile is four half-steps of 16 MFMAs (rows 64 hs .. 64 hs + 63 of the wave tile, k32-step s2); the fragments of the
+//     next half-step are read one LDS instruction behind each MFMA, the barrier that publishes the next tile sits before the
+//     last half-step, whose MFMAs cover the twelve reads of the next tile's first fragments.
+//   * the B fragment is the MFMA's first operand, so the accumulators hold C transposed: a lane owns 4 consecutive columns of
+//     one row, packs them to 8 bytes, and the wave stages its rows through its 8 KiB of the dead LDS stage so that C leaves as
+//     whole 128-byte lines (the 32 x 32 kernel stores 2 bytes per lane and instruction).
+//   * MFMA order: one operand changes between consecutive instructions (row-block outer, column-block inner, snaked).
+typedef float f32x4_acc __attribute__((ext_vector_type(4)));
+template <typename T> struct Mma16;
+template <> struct Mma16<f16_t> {
+    static __device__ __forceinline__ void run(f32x4_acc& acc, const u32x4& a, const u32x4& b)
+    { acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0); }
+};
+template <> struct Mma16<bf16_t> {
+    static __device__ __forceinline__ void run(f32x4_acc& acc, const u32x4& a, const u32x4& b)
+    { acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0); }
+};
+
+template <typename T, typename OutT>
+__global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
+{
+    constexpr int E = 8, EB = 2;
+    constexpr int WN = 4;
+    constexpr int BM = 256, BN = 256, BK = 64;
+    constexpr int WTM = 128, WTN = 64;
+    constexpr int TI = 8, TJ = 4;                 // 16 x 16 blocks of the wave tile
+    constexpr int BROW = BN * EB;
+    constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
+    constexpr int LA = 4, LB = 4, RPL = 2, LPR = 32;
+    constexpr int OB = Elem<OutT>::BYTES;
+
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+    const int t = threadIdx.x;
+    const int lane = t & 63, wave = t >> 6;
+    const int l16 = lane & 15, g4 = lane >> 4;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const long long bz = blockIdx.z;
+    const unsigned char* __restrict__ A = (const unsigned char*)g.A + bz * g.sA * EB;
+    const unsigned char* __restrict__ B = (const unsigned char*)g.B + bz * g.sB * EB;
+
+    // Chunk swizzle of a B k-row (position of 16-byte chunk c in its 512-byte LDS row: c ^ b_swz(row)): the four rows one
+    // transposing read touches go to different bank groups, and rows 8 apart -- the two 16-lane groups that share a cycle of
+    // that read -- are moved 32 bytes apart.
+    auto b_swz = [](int row) -> int { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
+    const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
+    uint32_t a_lane_off[2], b_lane_off[LB];
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+        const int ra = lane >> 3, pos_a = lane & 7;
+        a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+        const int rb = lane / LPR, pos_b = lane % LPR;
+        const int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
+        b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
+    }
+    const unsigned char* a_base = A + (long long)(m0 + 8 * LA * wave_s) * g.lda * EB;
+    const unsigned char* b_base = B + ((long long)(RPL * LB * wave_s) * g.ldb + n0) * EB;
+    const long long a_step = 8LL * g.lda * EB, b_step = (long long)RPL * g.ldb * EB;
+    const int KT = g.K / BK;
+    auto issue_loads = [&](int kt, int stage) {
+        const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
+        const uint32_t bs = lds0 + stage * STAGE + ABYTES + wave_s * (LB * 1024);
+        const unsigned char* a_src = a_base + (long long)kt * 128;
+        const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * EB;
+#pragma unroll
+        for (int i = 0; i < LA; i++) dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
+#pragma unroll
+        for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i], bs + i * 1024);
+    };
+
+    // A fragment of 16-row block i, k32-step s2: row 16 i + l16, chunk 4 s2 + g4, swizzled by (row >> 1) & 7 = (l16 >> 1) & 7
+    const int a_row0 = (wm * WTM + l16) * 128;
+    const int a_sw = (l16 >> 1) & 7;
+    // B fragment of 16-column block j, k32-step s2: two transposing reads (q = 0, 1); the lane addresses k-row
+    // 32 s2 + 8 g4 + 4 q + l16 / 4 and the 8 bytes at column 16 j + 4 (l16 % 4), and receives k 8 g4 + 4 q .. + 3 of column 16 j + l16
+    const int b_rowl = 8 * g4 + (l16 >> 2);
+    const int b_half = (l16 & 1) * 8;
+    const int b_chunk0 = wn * 8 + ((l16 & 3) >> 1);      // + 2 j
+
+    auto read_a = [&](const unsigned char* as, int s2, int i, u32x4& f) {
+        f = *(const u32x4*)(as + a_row0 + i * 2048 + (((4 * s2 + g4) ^ a_sw) << 4));
+    };
+    auto read_b = [&](const unsigned char* bs, int s2, int j, u32x4& f) {
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int row = 32 * s2 + 4 * q + b_rowl;
+            const int pos = (b_chunk0 + 2 * j) ^ b_swz(row);
+            s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                (__attribute__((address_space(3))) s16x4*)(bs + row * BROW + pos * 16 + b_half));
+            u32x2 w = __builtin_bit_cast(u32x2, v);
+            f[2 * q] = w[0];
+            f[2 * q + 1] = w[1];
+        }
+    };
+
+    f32x4_acc acc[TI][TJ];
+#pragma unroll
+    for (int i = 0; i < TI; i++)
+#pragma unroll
+        for (int j = 0; j < TJ; j++) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
+
+    issue_loads(0, 0);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    // fa[p]: the four A fragments of half-step parity p; fb[p]: the four B fragments of k32-step parity p
+    u32x4 fa[2][4], fb[2][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) read_a(smem, 0, i, fa[0][i]);
+#pragma unroll
+    for (int j = 0; j < 4; j++) read_b(smem + ABYTES, 0, j, fb[0][j]);
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int stage = kt & 1;
+        const unsigned char* as = smem + stage * STAGE;
+        const unsigned char* bs = as + ABYTES;
+        const unsigned char* an = smem + (stage ^ 1) * STAGE;
+        // the other stage was last read before the barrier inside the previous iteration
+        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+#pragma unroll
+        for (int u = 0; u < 4; u++) {              // half-step u = 2 s2 + hs
+            const int s2 = u >> 1, hs = u & 1;
+            if (u == 0) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) read_a(as, 0, 4 + i, fa[1][i]);
+                read_b(bs, 1, 0, fb[1][0]); read_b(bs, 1, 1, fb[1][1]);
+            } else if (u == 1) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) read_a(as, 1, i, fa[0][i]);
+                read_b(bs, 1, 2, fb[1][2]); read_b(bs, 1, 3, fb[1][3]);
+            } else if (u == 2) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) read_a(as, 1, 4 + i, fa[1][i]);
+            } else {
+                __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed and its LDS reads of this tile are done ...
+                __syncthreads();                    // ... and so have everyone else's
+                if (kt + 1 < KT) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) read_a(an, 0, i, fa[0][i]);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = (i & 1) ? 3 - jj : jj;
+                    Mma16<T>::run(acc[4 * hs + i][j], fb[s2][j], fa[hs][i]);
+                }
+            // one LDS read behind each of the first MFMAs, the remaining MFMAs after the reads have been issued
+            if (u < 2) { spread_schedule<8, 8, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 8, 0); }
+            else if (u == 2) { spread_schedule<4, 4, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 12, 0); }
+            else { spread_schedule<12, 12, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 4, 0); }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+
+    // ---- epilogue.  acc[i][j]: the lane holds C[row 16 i + l16][columns 16 j + 4 g4 .. + 3].  Staged through the wave's 8 KiB of
+    // the last stage (dead after the final barrier), 16-byte chunk c of a staged row at position c ^ ((row >> 1) & 7).
+    {
+        unsigned char* stg = smem + ((KT - 1) & 1) * STAGE + wave * 8192;
+        constexpr int ROWB = 64 * OB;
+        constexpr int RPR = 8192 / ROWB;              // rows per round: 64 (16-bit output) or 32 (fp32)
+        constexpr int IPR = RPR / 16;                 // 16-row blocks per round
+        constexpr int CPR = ROWB / 16;
+        const int sw = (l16 >> 1) & 7;
+        const bool fused = g.bias != nullptr || g.act != 0;
+        f32x4 bias4[TJ];
+#pragma unroll
+        for (int j = 0; j < TJ; j++) {
+            bias4[j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (g.bias) bias4[j] = *(const f32x4*)(g.bias + n0 + wn * WTN + 16 * j + 4 * g4);
+        }
+        unsigned char* Cw = (unsigned char*)g.C + (bz * g.sC + (long long)(m0 + wm * WTM) * g.ldc + n0 + wn * WTN) * OB;
+#pragma unroll
+        for (int ip = 0; ip < TI; ip += IPR) {
+#pragma unroll
+            for (int ii = 0; ii < IPR; ii++) {
+#pragma unroll
+                for (int j = 0; j < TJ; j++) {
+                    f32x4_acc v = acc[ip + ii][j];
+                    if (fused) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = apply_activation(v[e] + bias4[j][e], g.act, g.act_param);
+                    }
+                    const int row = ii * 16 + l16;
+                    if constexpr (OB == 2) {
+                        const uint32_t w0 = Elem<OutT>::narrow(v[0]) | (Elem<OutT>::narrow(v[1]) << 16);
+                        const uint32_t w1 = Elem<OutT>::narrow(v[2]) | (Elem<OutT>::narrow(v[3]) << 16);
+                        const int chunk = 2 * j + (g4 >> 1);
+                        *(u32x2*)(stg + row * ROWB + ((chunk ^ sw) << 4) + (g4 & 1) * 8) = u32x2{w0, w1};
+                    } else {
+                        const int chunk = 4 * j + g4;
+                        *(u32x4*)(stg + row * ROWB + ((chunk ^ sw) << 4)) = u32x4{as_u32(v[0]), as_u32(v[1]), as_u32(v[2]), as_u32(v[3])};
+                    }
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const int u = q * 64 + lane;
+                const int row = u / CPR, c = u % CPR;
+                const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ ((row >> 1) & 7)) << 4));
+                *(u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16) = v;
+            }
+        }
+    }
+}
+
+template <typename T, typename OutT>
+static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
+{
+    auto kern = gemm_dl16_kernel<T, OutT>;
+    constexpr int smem = 2 * (256 * 128 + 128 * 256);
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
+    g.tiles_m = g.M / 256;
+    g.tiles_n = g.N / 256;
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(512), smem, stream, g);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
 // Skinny-M path (decode projections): M <= 32, 16-bit, B stored [K,N], N % 128 == 0, K % 64 == 0.
 // HBM-bound: B (K x N) is read exactly once.  grid = (N / 128, KS): each workgroup streams a 128-column
 // slab of B over its K range with the direct global->LDS load (two 20 KB stages, several workgroups per
@@ -935,11 +1180,13 @@ static int skinny_ksplit(int N, int K)
     return ks;
 }
 
+#if AIDN_GEMM_PART == 0
 size_t gemm_16_workspace_bytes(int M, int N, int K)
 {
     if (!skinny_applies(M, N, K)) return 0;
     return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
 }
+#endif
 
 template <typename T, typename OutT>
 static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
@@ -1073,12 +1320,14 @@ static int smallm_kper(int N, int K)
     return kper;
 }
 
+#if AIDN_GEMM_PART == 0
 size_t gemm_f32_workspace_bytes(int M, int N, int K)
 {
     if (!smallm_applies(M, N, K)) return 0;
     const int kper = smallm_kper(N, K);
     return (size_t)((K + kper - 1) / kper) * M * N * sizeof(float);
 }
+#endif
 
 template <bool B16>
 static hipError_t launch_smallm(const GemmArgs& g, hipStream_t stream, float* ws)
@@ -1181,6 +1430,13 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             // (bf16 output with ragged edges on the 256 x 256 tile: that one instance does not fit the register file -- the
             // compiler moves accumulators to scratch memory -- so such problems take the 128 x 128 tile)
             constexpr bool kSpills256Edge = std::is_same<T, bf16_t>::value && std::is_same<OutT, bf16_t>::value;
+            if constexpr (E == 8 && !TRANSB) {
+                // 16-bit, whole tiles: the 16 x 16 x 32 kernel (its stores and bias loads are 16-byte vectors: C rows and the bias
+                // must be 16-byte aligned; it computes act(A B + bias), so alpha = 1 and beta = 0)
+                const bool rows16 = aligned16(g.C) && (g.ldc * Elem<OutT>::BYTES) % 16 == 0 && (g.sC * Elem<OutT>::BYTES) % 16 == 0 &&
+                                    (g.bias == nullptr || aligned16(g.bias));
+                if (tile == 256 && exact_fit && rows16 && g.alpha == 1.0f && g.beta == 0.0f) return launch_gemm_dl16<T, OutT>(g, batch, stream);
+            }
             if (tile == 256 && exact_fit) return launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, batch, stream);
             if constexpr (!kSpills256Edge) {
                 if (tile == 256) return launch_gemm_dl<T, OutT, true, 256, TRANSB>(g, batch, stream);
@@ -1210,6 +1466,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     return hipErrorInvalidValue;
 }
 
+#if AIDN_GEMM_PART == 0
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
                     int force_tile, const float* bias, int act, float act_param, void* workspace)
@@ -1239,22 +1496,42 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
     return launch_gemm<float, float, 64, 64, 2, 2, false, false, true, 1, true>(g, 1, stream);
 }
 
-// kind: 0 = fp16, 1 = bf16; out32: C is fp32 (else the same 16-bit type as the inputs)
-hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+#endif
+
+// one 16-bit type per part: T = f16_t in part 1, bf16_t in part 2; out32: C is fp32 (else the same 16-bit type as the inputs)
+template <typename T>
+static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                                int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
 {
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
     if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         float* ws = (float*)workspace;
-        if (kind == 0) return out32 ? launch_skinny<f16_t, float>(g, stream, ws) : launch_skinny<f16_t, f16_t>(g, stream, ws);
-        return out32 ? launch_skinny<bf16_t, float>(g, stream, ws) : launch_skinny<bf16_t, bf16_t>(g, stream, ws);
+        return out32 ? launch_skinny<T, float>(g, stream, ws) : launch_skinny<T, T>(g, stream, ws);
     }
-    if (kind == 0) {
-        if (out32) return dispatch_gemm<f16_t, float, false>(g, 1, stream, force_tile);
-        return dispatch_gemm<f16_t, f16_t, false>(g, 1, stream, force_tile);
-    }
-    if (out32) return dispatch_gemm<bf16_t, float, false>(g, 1, stream, force_tile);
-    return dispatch_gemm<bf16_t, bf16_t, false>(g, 1, stream, force_tile);
+    if (out32) return dispatch_gemm<T, float, false>(g, 1, stream, force_tile);
+    return dispatch_gemm<T, T, false>(g, 1, stream, force_tile);
 }
+
+hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param);
+hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param);
+#if AIDN_GEMM_PART == 1
+hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+{ return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param); }
+#elif AIDN_GEMM_PART == 2
+hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+{ return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param); }
+#else
+// kind: 0 = fp16, 1 = bf16
+hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
+                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+{
+    if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param);
+    return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param);
+}
+#endif
 
 }  // namespace aidn
