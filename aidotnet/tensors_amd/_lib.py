@@ -10,7 +10,8 @@ import ctypes
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libaidotnet_mi355.so")
+# the in-tree build; AIDOTNET_MI355_LIBRARY names another build of the same library (for comparing builds)
+LIB_PATH = os.environ.get("AIDOTNET_MI355_LIBRARY") or os.path.join(HERE, "libaidotnet_mi355.so")
 
 AIDN_OK = 0
 AIDN_ERR_INVALID_ARGUMENT = 1001

@@ -498,6 +498,9 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 // for any reference point m.
 
 
+#ifndef AIDN_ATTN_RING
+#define AIDN_ATTN_RING 4
+#endif
 template <typename T, typename OutT>
 __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 {
@@ -697,15 +700,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 return u32x4{w0[0], w0[1], w1[0], w1[1]};
             };
 
-            // LDS fragment reads run four ahead of the MFMAs that consume them (fr[] is a 4-deep ring);
-            // sched_barrier pins that order and the MFMA / exp interleave.
+            // LDS fragment reads run R ahead of the MFMAs that consume them (fr[] is an R-deep ring; an idle LDS read takes
+            // about 90 cycles, three MFMAs); sched_barrier pins that order and the MFMA / exp interleave.
             // ---- S0 = K[0:32] Q^T
             f32x16 s0, s1;
 #pragma unroll
             for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
-            u32x4 fr[4];
+            constexpr int R = AIDN_ATTN_RING;
+            u32x4 fr[R];
 #pragma unroll
-            for (int s = 0; s < 4; s++) fr[s] = k_frag(0, s);
+            for (int s = 0; s < R; s++) fr[s] = k_frag(0, s);
             // the phases that issue nothing but MFMAs (this one and the last) run at a raised wave priority: the matrix pipe then
             // takes them ahead of the other wave's instructions on the SIMD, whose exponentials fill the gaps (1-2 % measured)
             __builtin_amdgcn_s_setprio(2);
@@ -716,8 +720,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 const uint32_t vdst = lds0 + 2 * KBYTES + (stage ^ 1) * VBYTES + wave_s * 4096;
 #pragma unroll
                 for (int s = 0; s < DSTEPS; s++) {
-                    Mma32<T>::run(s0, fr[s & 3], qf[s]);
-                    fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
+                    Mma32<T>::run(s0, fr[s % R], qf[s]);
+                    fr[s % R] = s + R < DSTEPS ? k_frag(0, s + R) : k_frag(1, s + R - DSTEPS);
                     if (s < 4) attn_dma16_base(ksrc + 4 * s * k_row_bytes, k_lane_off[s], kdst + s * 1024);
                     else attn_dma16_base(vsrc + 4 * (s - 4) * v_row_bytes, v_lane_off, vdst + (s - 4) * 1024);
                     __builtin_amdgcn_sched_barrier(0);
@@ -725,8 +729,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             } else {
 #pragma unroll
                 for (int s = 0; s < DSTEPS; s++) {
-                    Mma32<T>::run(s0, fr[s & 3], qf[s]);
-                    fr[s & 3] = s + 4 < DSTEPS ? k_frag(0, s + 4) : k_frag(1, s + 4 - DSTEPS);
+                    Mma32<T>::run(s0, fr[s % R], qf[s]);
+                    fr[s % R] = s + R < DSTEPS ? k_frag(0, s + R) : k_frag(1, s + R - DSTEPS);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -740,8 +744,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             float psum = 0.0f;
 #pragma unroll
             for (int s = 0; s < DSTEPS; s++) {
-                Mma32<T>::run(s1, fr[s & 3], qf[s]);
-                fr[s & 3] = s + 4 < DSTEPS ? k_frag(1, s + 4) : v_frag8(0, s + 4 - DSTEPS);
+                Mma32<T>::run(s1, fr[s % R], qf[s]);
+                fr[s % R] = s + R < DSTEPS ? k_frag(1, s + R) : v_frag8(0, s + R - DSTEPS);
                 uint32_t pk;
                 exp_pair(s0[2 * s], s0[2 * s + 1], m_use, pk, psum);
                 asm volatile("" : "+v"(pk), "+v"(psum));       // keeps the exponentials here, between the MFMAs
@@ -754,8 +758,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             float psum1 = 0.0f;
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                Mma32<T>::run(oacc[s & 3], fr[s & 3], p0f[s >> 2]);
-                fr[s & 3] = s + 4 < 8 ? v_frag8(0, s + 4) : v_frag8(1, s + 4 - 8);
+                Mma32<T>::run(oacc[s & 3], fr[s % R], p0f[s >> 2]);
+                fr[s % R] = s + R < 8 ? v_frag8(0, s + R) : v_frag8(1, s + R - 8);
                 uint32_t pk;
                 exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk, psum1);
                 asm volatile("" : "+v"(pk), "+v"(psum1));
@@ -783,13 +787,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             __builtin_amdgcn_s_setprio(2);
 #pragma unroll
             for (int s = 0; s < 8; s++) {
-                Mma32<T>::run(oacc[s & 3], fr[s & 3], p1f[s >> 2]);
-                if (s + 4 < 8) fr[s & 3] = v_frag8(1, s + 4);
+                Mma32<T>::run(oacc[s & 3], fr[s % R], p1f[s >> 2]);
+                if (s + R < 8) fr[s % R] = v_frag8(1, s + R);
             }
             __builtin_amdgcn_s_setprio(0);
         }
+#if defined(AIDN_ATTN_ABL) && (AIDN_ATTN_ABL & 2)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#else
         __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA of tile j+1 has landed ...
+#endif
+#if !(defined(AIDN_ATTN_ABL) && (AIDN_ATTN_ABL & 1))
         __syncthreads();                    // ... everyone's has, and everyone is done with tile j
+#endif
     };
     for (int j = 0; j < ntiles; j += 2) {
         tile_body(j, std::integral_constant<int, 0>{});

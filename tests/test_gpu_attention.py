@@ -265,6 +265,22 @@ def test_config4_half_causal_b4_h32_s2048_d128(be, kind):
         o64, lse64 = oracle.attention_f64(qs, ks, vs, scale, True)
         assert mixed_err(out[b, h].cpu().numpy(), o64[0, 0]) <= HALF_TOL
         assert mixed_err(lse[b, h].cpu().numpy(), lse64[0, 0]) <= 1e-3
+    # every (batch, head) slice, so that a wrong head / workgroup remap cannot hide: the whole LSE column and eight sampled query
+    # rows per slice against a float64 softmax of the same rounded inputs (computed on the device; the arithmetic of
+    # oracle.attention_f64, which the three slices above tie it to)
+    rng = np.random.default_rng(5)
+    causal_mask = torch.ones(S, S, device="cuda", dtype=torch.bool).tril()
+    for b in range(B):
+        for h in range(H):
+            q64, k64, v64 = q[b, h].double(), k[b, h].double(), v[b, h].double()
+            logits = (q64 @ k64.T) * scale
+            logits = logits.masked_fill(~causal_mask, float("-inf"))
+            lse_ref = torch.logsumexp(logits, dim=1)
+            assert float((lse[b, h].double() - lse_ref).abs().max()) <= 1e-3, (b, h)
+            rows = torch.from_numpy(rng.choice(S, 8, replace=False)).cuda()
+            o_ref = torch.softmax(logits[rows], dim=1) @ v64
+            err = ((out[b, h][rows].double() - o_ref).abs() / (1 + o_ref.abs())).max()
+            assert float(err) <= HALF_TOL, (b, h)
 
 
 # --------------------------------------------------------------- head-dim-128 fast path (direct-to-LDS kernel)
