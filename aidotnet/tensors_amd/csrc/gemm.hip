@@ -835,15 +835,20 @@ template <> struct Mma16<bf16_t> {
     { acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0); }
 };
 
-template <typename T, typename OutT>
+// TJ = 16-column blocks per wave: the tile is 256 x (64 TJ) -- 256 x 256, 256 x 192 or 256 x 128 -- so that problems whose 256 x 256
+// tiles would leave CUs idle in the last round (4096 x 3072: 192 tiles on 256 CUs) get a tile count that fills them.  The B tile
+// keeps its 512-byte LDS rows for every TJ (the chunk swizzle needs a power-of-two row); lanes whose swizzled chunk lies past
+// the tile's columns fetch a valid chunk again and park it in a position that no fragment read touches.
+template <typename T, typename OutT, int TJ = 4>
 __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 {
     constexpr int E = 8, EB = 2;
     constexpr int WN = 4;
-    constexpr int BM = 256, BN = 256, BK = 64;
-    constexpr int WTM = 128, WTN = 64;
-    constexpr int TI = 8, TJ = 4;                 // 16 x 16 blocks of the wave tile
-    constexpr int BROW = BN * EB;
+    constexpr int BM = 256, BN = 64 * TJ, BK = 64;
+    constexpr int WTM = 128, WTN = 16 * TJ;
+    constexpr int TI = 8;                         // 16 x 16 blocks of the wave tile: TI x TJ
+    constexpr int BROW = 256 * EB;                // LDS pitch of a B k-row (32 chunk positions)
+    constexpr int BCH = BN / E;                   // 16-byte chunks of a k-row that hold tile columns
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
     constexpr int LA = 4, LB = 4, RPL = 2, LPR = 32;
     constexpr int OB = Elem<OutT>::BYTES;
@@ -875,7 +880,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 #pragma unroll
     for (int i = 0; i < LB; i++) {
         const int rb = lane / LPR, pos_b = lane % LPR;
-        const int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
+        int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
+        if (chunk >= BCH) chunk -= 32 - BCH >= BCH ? BCH : 32 - BCH;      // a valid chunk again (its LDS position is never read)
         b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
     }
     const unsigned char* a_base = A + (long long)(m0 + 8 * LA * wave_s) * g.lda * EB;
@@ -900,7 +906,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     // 32 s2 + 8 g4 + 4 q + l16 / 4 and the 8 bytes at column 16 j + 4 (l16 % 4), and receives k 8 g4 + 4 q .. + 3 of column 16 j + l16
     const int b_rowl = 8 * g4 + (l16 >> 2);
     const int b_half = (l16 & 1) * 8;
-    const int b_chunk0 = wn * 8 + ((l16 & 3) >> 1);      // + 2 j
+    const int b_chunk0 = wn * (2 * TJ) + ((l16 & 3) >> 1);      // + 2 j
 
     auto read_a = [&](const unsigned char* as, int s2, int i, u32x4& f) {
         f = *(const u32x4*)(as + a_row0 + i * 2048 + (((4 * s2 + g4) ^ a_sw) << 4));
@@ -929,11 +935,11 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     __syncthreads();
 
     // fa[p]: the four A fragments of half-step parity p; fb[p]: the four B fragments of k32-step parity p
-    u32x4 fa[2][4], fb[2][4];
+    u32x4 fa[2][4], fb[2][TJ];
 #pragma unroll
     for (int i = 0; i < 4; i++) read_a(smem, 0, i, fa[0][i]);
 #pragma unroll
-    for (int j = 0; j < 4; j++) read_b(smem + ABYTES, 0, j, fb[0][j]);
+    for (int j = 0; j < TJ; j++) read_b(smem + ABYTES, 0, j, fb[0][j]);
 
     for (int kt = 0; kt < KT; kt++) {
         const int stage = kt & 1;
@@ -952,7 +958,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
             } else if (u == 1) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) read_a(as, 1, i, fa[0][i]);
-                read_b(bs, 1, 2, fb[1][2]); read_b(bs, 1, 3, fb[1][3]);
+#pragma unroll
+                for (int j = 2; j < TJ; j++) read_b(bs, 1, j, fb[1][j]);
             } else if (u == 2) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) read_a(as, 1, 4 + i, fa[1][i]);
@@ -963,20 +970,23 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 #pragma unroll
                     for (int i = 0; i < 4; i++) read_a(an, 0, i, fa[0][i]);
 #pragma unroll
-                    for (int j = 0; j < 4; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
+                    for (int j = 0; j < TJ; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
                 }
             }
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int jj = 0; jj < 4; jj++) {
-                    const int j = (i & 1) ? 3 - jj : jj;
+                for (int jj = 0; jj < TJ; jj++) {
+                    const int j = (i & 1) ? TJ - 1 - jj : jj;
                     Mma16<T>::run(acc[4 * hs + i][j], fb[s2][j], fa[hs][i]);
                 }
             // one LDS read behind each of the first MFMAs, the remaining MFMAs after the reads have been issued
-            if (u < 2) { spread_schedule<8, 8, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 8, 0); }
-            else if (u == 2) { spread_schedule<4, 4, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 12, 0); }
-            else { spread_schedule<12, 12, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, 4, 0); }
+            constexpr int NM = 4 * TJ;                                   // MFMAs per half-step
+            constexpr int R0 = 8, R1 = 4 + 2 * (TJ - 2), R2 = 4, R3 = 4 + 2 * TJ;      // LDS reads of the four half-steps
+            if (u == 0) { spread_schedule<R0, R0, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R0, 0); }
+            else if (u == 1) { spread_schedule<R1, R1, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R1, 0); }
+            else if (u == 2) { spread_schedule<R2, R2, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R2, 0); }
+            else { spread_schedule<R3, R3, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R3, 0); }
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -985,11 +995,12 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     // the last stage (dead after the final barrier), 16-byte chunk c of a staged row at position c ^ ((row >> 1) & 7).
     {
         unsigned char* stg = smem + ((KT - 1) & 1) * STAGE + wave * 8192;
-        constexpr int ROWB = 64 * OB;
-        constexpr int RPR = 8192 / ROWB;              // rows per round: 64 (16-bit output) or 32 (fp32)
-        constexpr int IPR = RPR / 16;                 // 16-row blocks per round
-        constexpr int CPR = ROWB / 16;
-        const int sw = (l16 >> 1) & 7;
+        constexpr int ROWB = WTN * OB;                // bytes of one staged row
+        constexpr int CPR = ROWB / 16;                // 16-byte chunks per staged row
+        constexpr int FIT = 8192 / (16 * ROWB);       // 16-row blocks that fit the wave's 8 KiB
+        constexpr int IPR = FIT >= 8 ? 8 : FIT >= 4 ? 4 : FIT >= 2 ? 2 : 1;      // blocks per round (divides TI)
+        constexpr bool POW2 = (CPR & (CPR - 1)) == 0; // the XOR swizzle of the staged rows needs a power-of-two chunk count
+        const int sw = POW2 ? ((l16 >> 1) & (CPR - 1) & 7) : 0;
         const bool fused = g.bias != nullptr || g.act != 0;
         f32x4 bias4[TJ];
 #pragma unroll
@@ -1022,25 +1033,25 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 }
             }
 #pragma unroll
-            for (int q = 0; q < 8; q++) {
+            for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
                 const int u = q * 64 + lane;
                 const int row = u / CPR, c = u % CPR;
-                const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ ((row >> 1) & 7)) << 4));
+                const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
                 *(u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16) = v;
             }
         }
     }
 }
 
-template <typename T, typename OutT>
+template <typename T, typename OutT, int TJ = 4>
 static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_dl16_kernel<T, OutT>;
+    auto kern = gemm_dl16_kernel<T, OutT, TJ>;
     constexpr int smem = 2 * (256 * 128 + 128 * 256);
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     g.tiles_m = g.M / 256;
-    g.tiles_n = g.N / 256;
+    g.tiles_n = g.N / (64 * TJ);
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(512), smem, stream, g);
     return hipGetLastError();
 }
@@ -1384,6 +1395,38 @@ static int choose_tile(long long tiles128, long long tiles64, double rel64)
     return cu_fill(tiles128) >= rel64 * cu_fill(tiles64) ? 128 : 64;
 }
 
+// what the 16 x 16 x 32 kernel needs beyond whole tiles: 16-byte aligned operand rows, C rows and bias, and the plain product
+template <typename OutT>
+static bool dl16_applies(const GemmArgs& g)
+{
+    const int OB = Elem<OutT>::BYTES;
+    return aligned16(g.A) && aligned16(g.B) && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.sA % 8 == 0 && g.sB % 8 == 0 &&
+           g.lda < (1 << 21) && g.ldb < (1 << 21) &&
+           aligned16(g.C) && ((long long)g.ldc * OB) % 16 == 0 && (g.sC * OB) % 16 == 0 && (g.bias == nullptr || aligned16(g.bias)) &&
+           g.alpha == 1.0f && g.beta == 0.0f;
+}
+
+// Tile width (in 64-column units: 4, 3 or 2) of the 16 x 16 x 32 kernel for a 16-bit problem with M % 256 == 0 and K % 64 == 0, or 0
+// when none of the widths divides N or gives at least half a chip of tiles.  A narrower tile moves more A bytes per flop (and the
+// 256 x 128 one wastes half of its B loads), so it has to win on how evenly the tiles load the 256 CUs.
+static int dl16_width(int M, int N, int K, int batch)
+{
+    if (M % 256 != 0 || K % 64 != 0) return 0;
+    const int widths[3] = {4, 3, 2};
+    const double eff[3] = {1.0, 0.94, 0.8};
+    int best = 0;
+    double best_score = 0.0;
+    for (int i = 0; i < 3; i++) {
+        const int bn = 64 * widths[i];
+        if (N % bn != 0) continue;
+        const long long t = (long long)(M / 256) * (N / bn) * batch;
+        if (t < 128) continue;
+        const double score = cu_fill(t) * eff[i];
+        if (score > best_score) { best_score = score; best = widths[i]; }
+    }
+    return best;
+}
+
 // Kernel and tile choice: the 256 x 256 direct-to-LDS kernel for 16-bit B[K,N] problems with at least 128 such tiles,
 // otherwise the general kernel with the 128 x 128 or 64 x 64 tile (choose_tile), in its branch-free instance when the
 // operands are 16-byte aligned and the K-tile divides K.
@@ -1402,6 +1445,14 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if (vec && g.lda < (1 << 21) && g.ldb < (1 << 21) && (Elem<OutT>::BYTES == 4 || (g.alpha == 1.0f && g.beta == 0.0f))) {
                 // 16-bit: the 256 x 256 tile moves half the bytes per flop of the 128 x 128 one and wins from half a chip of
                 // tiles on; fp32 runs both at about the same rate per flop, so there the better CU load decides
+                if constexpr (E == 8 && !TRANSB) {
+                    if (dl16_applies<OutT>(g)) {
+                        const int w = dl16_width(g.M, g.N, g.K, batch);
+                        if (w == 4) return launch_gemm_dl16<T, OutT, 4>(g, batch, stream);
+                        if (w == 3) return launch_gemm_dl16<T, OutT, 3>(g, batch, stream);
+                        if (w == 2) return launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
+                    }
+                }
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
                 const bool big = E == 8 ? t256 >= 128 : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
                 // otherwise the same kernel with 128 x 128 or 64 x 64 tiles (codes 129, 65), whichever loads the CUs better; per
@@ -1412,6 +1463,14 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         }
         if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
     }
+    if constexpr (E == 8 && !TRANSB) {
+        if (tile == 192 || tile == 193) {                 // 256 x 192 / 256 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
+            const int bn = tile == 192 ? 192 : 128;
+            if (!(g.M % 256 == 0 && g.N % bn == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
+            return tile == 192 ? launch_gemm_dl16<T, OutT, 3>(g, batch, stream) : launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
+        }
+    }
+    if (tile == 192 || tile == 193) return hipErrorInvalidValue;
     if constexpr (E == 4 || !TRANSB) {
         if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
@@ -1433,9 +1492,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if constexpr (E == 8 && !TRANSB) {
                 // 16-bit, whole tiles: the 16 x 16 x 32 kernel (its stores and bias loads are 16-byte vectors: C rows and the bias
                 // must be 16-byte aligned; it computes act(A B + bias), so alpha = 1 and beta = 0)
-                const bool rows16 = aligned16(g.C) && (g.ldc * Elem<OutT>::BYTES) % 16 == 0 && (g.sC * Elem<OutT>::BYTES) % 16 == 0 &&
-                                    (g.bias == nullptr || aligned16(g.bias));
-                if (tile == 256 && exact_fit && rows16 && g.alpha == 1.0f && g.beta == 0.0f) return launch_gemm_dl16<T, OutT>(g, batch, stream);
+                if (tile == 256 && exact_fit && dl16_applies<OutT>(g)) return launch_gemm_dl16<T, OutT, 4>(g, batch, stream);
             }
             if (tile == 256 && exact_fit) return launch_gemm_dl<T, OutT, false, 256, TRANSB>(g, batch, stream);
             if constexpr (!kSpills256Edge) {

@@ -276,7 +276,9 @@ def test_config4_half_causal_b4_h32_s2048_d128(be, kind):
             logits = (q64 @ k64.T) * scale
             logits = logits.masked_fill(~causal_mask, float("-inf"))
             lse_ref = torch.logsumexp(logits, dim=1)
-            assert float((lse[b, h].double() - lse_ref).abs().max()) <= 1e-3, (b, h)
+            # the row sum adds the probabilities as rounded to the storage type (the numbers the P V product uses): relative
+            # error up to 2^-12 per term in fp16, 2^-9 in bf16, hence the wider bound for bf16
+            assert float((lse[b, h].double() - lse_ref).abs().max()) <= (1e-3 if kind == "f16" else 4e-3), (b, h)
             rows = torch.from_numpy(rng.choice(S, 8, replace=False)).cuda()
             o_ref = torch.softmax(logits[rows], dim=1) @ v64
             err = ((out[b, h][rows].double() - o_ref).abs() / (1 + o_ref.abs())).max()

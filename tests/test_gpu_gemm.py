@@ -462,3 +462,60 @@ def test_config2_square_8192_baseline_distribution_sampled_rows(be, kind):
     assert torch.equal(c16, c32.to(dt)), "16-bit output is not the RNE narrowing of the fp32 accumulator"
     # the reduced-precision result differs from the product of the unrounded inputs' fp32 GEMM: not a widened fp32 path
     assert bool(torch.isfinite(c32).all())
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("tile,M,N,K", [(192, 256, 192, 64), (192, 512, 576, 192), (192, 256, 768, 4096), (193, 256, 128, 64),
+                                        (193, 768, 384, 320), (193, 256, 640, 2048), (256, 512, 768, 128)])
+def test_half_gemm_16x16x32_kernel_tile_widths(be, kind, tile, M, N, K):
+    # the 256 x 192 and 256 x 128 tiles of the 16 x 16 x 32 kernel (codes 192 / 193) and its 256 x 256 tile, forced on small whole-tile
+    # shapes: bit-exact on dyadic inputs for both output types, bias + activation epilogue, guard band, refusal of ragged shapes
+    be.SetGemmTile(tile)
+    try:
+        rng = np.random.default_rng(tile + M + 2 * N + 3 * K)
+        a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+        ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+        fn = oracle.hgemm if kind == "f16" else oracle.bf16gemm
+        want16, want32 = fn(ab, bb, M, K, N)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, True), want32)
+        assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, False), want16)
+        a = rng.uniform(-1, 1, (M, K)).astype(np.float32); b = rng.uniform(-1, 1, (K, N)).astype(np.float32)
+        ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+        truth = oracle.gemm_f64(aw, bw, M, K, N)
+        assert mixed_err(_half_gemm(be, kind, ab, bb, M, N, K, True), truth) <= 1e-4
+        # fused bias + ReLU in the store path of this kernel
+        bias = rng.uniform(-1, 1, N).astype(np.float32)
+        A = be.WrapTensor(from_bits16(ab, TORCH16[kind])); B = be.WrapTensor(from_bits16(bb, TORCH16[kind]))
+        c = torch.full(((M + 1) * N,), -7.0, device="cuda")
+        be.GemmBiasActivationHalf(kind, A, B, be.WrapTensor(dev(bias)), be.WrapTensor(c), M, N, K, 1, 0.0, True)
+        got = c[:M * N].reshape(M, N).cpu().numpy()
+        assert mixed_err(got, np.maximum(truth + bias[None, :], 0.0)) <= 1e-4
+        assert bool((c[M * N:] == -7.0).all())                     # one row of guard band behind C stays untouched
+        if tile != 256:
+            from aidotnet.tensors_amd import HipException
+            with pytest.raises(HipException):                      # these tile codes take whole tiles only
+                _half_gemm(be, kind, ab[:(M - 1) * K], bb, M - 1, N, K, True)
+    finally:
+        be.SetGemmTile(0)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_projection_shape_takes_a_width_that_fills_the_chip_and_is_exact(be, kind):
+    # 4096 x 3072 x 768 (the projection configuration): the automatic choice (256 x 192 tiles: 256 of them) must agree bit for
+    # bit with the forced 256 x 256 tile and with the general 128 x 128 kernel on dyadic inputs
+    M, N, K = 4096, 3072, 768
+    rng = np.random.default_rng(3072)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+    ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+    auto = _half_gemm(be, kind, ab, bb, M, N, K, False)
+    try:
+        for tile in (256, 128, 192):
+            be.SetGemmTile(tile)
+            assert np.array_equal(_half_gemm(be, kind, ab, bb, M, N, K, False), auto), tile
+    finally:
+        be.SetGemmTile(0)
+    rows = np.sort(rng.choice(M, 16, replace=False))
+    back = oracle.f16_to_f32(auto[rows]) if kind == "f16" else oracle.bf16_to_f32(auto[rows])
+    want = a[rows].astype(np.float64) @ b.astype(np.float64)
+    rounded = oracle.f16_to_f32(oracle.f32_to_f16(want.astype(np.float32))) if kind == "f16" else oracle.bf16_to_f32(oracle.f32_to_bf16(want.astype(np.float32)))
+    assert np.array_equal(back, rounded)
