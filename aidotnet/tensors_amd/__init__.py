@@ -8,7 +8,13 @@ from ._lib import LIB_PATH, SIGNATURES, AttnDesc, load as load_library
 from .backend import (ArgumentException, ArgumentNullException, ArgumentOutOfRangeException, GpuBuffer,
                       HipException, InvalidOperationException, Mi355Backend, NotSupportedException)
 from .engine import Mi355Engine
+from .precision import (GpuAccuracyMode, GpuComputePlan, GpuComputePreference, GpuExecutionPolicy, GpuExecutionPolicyScope,
+                        GpuExecutionRoute, GpuPrecisionCapability, GpuPrecisionDiagnostics, GpuPrecisionFallbackBehavior,
+                        GpuPrecisionImplementation, GpuPrecisionOperation, GpuPrecisionPlanner, GpuScalarType)
 
 __all__ = ["Mi355Backend", "Mi355Engine", "GpuBuffer", "AttnDesc", "load_library", "LIB_PATH", "SIGNATURES",
            "ArgumentException", "ArgumentNullException", "ArgumentOutOfRangeException", "HipException",
-           "InvalidOperationException", "NotSupportedException"]
+           "InvalidOperationException", "NotSupportedException",
+           "GpuAccuracyMode", "GpuComputePlan", "GpuComputePreference", "GpuExecutionPolicy", "GpuExecutionPolicyScope", "GpuExecutionRoute",
+           "GpuPrecisionCapability", "GpuPrecisionDiagnostics", "GpuPrecisionFallbackBehavior", "GpuPrecisionImplementation",
+           "GpuPrecisionOperation", "GpuPrecisionPlanner", "GpuScalarType"]

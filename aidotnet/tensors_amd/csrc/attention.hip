@@ -498,9 +498,11 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 // for any reference point m.
 
 
-#ifndef AIDN_ATTN_RING
+// Heads whose query tiles are interleaved (heaviest first) in the causal workgroup order of one XCD: 4 heads x 1 MiB of K and V
+// (S = 2048, d = 128, 16-bit) is what one XCD's 4 MiB L2 holds, and four heads' tiles are enough to balance the CUs.
+#define ATTN_HEAD_GROUP 4
+// Depth of the register ring that prefetches MFMA operand fragments from LDS inside a tile; must divide 8.
 #define AIDN_ATTN_RING 4
-#endif
 template <typename T, typename OutT>
 __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 {
@@ -522,10 +524,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
         if (a.causal && rem == 0 && per % a.qtiles == 0) {
-            // every XCD owns whole heads: inside an XCD hand out the query tiles heaviest first across its heads
+            // every XCD owns whole heads: inside an XCD take the heads in groups of ATTN_HEAD_GROUP and hand out the query tiles of a
+            // group heaviest first across its heads (all heads at once runs as fast but re-fetches K and V 3.3 times from beyond the L2)
             const int hx = per / a.qtiles;                    // heads per XCD
-            qt = a.qtiles - 1 - idx / hx;
-            bh = xcd * hx + idx % hx;
+            const int gsz = hx < ATTN_HEAD_GROUP ? hx : ATTN_HEAD_GROUP;
+            const int per_group = gsz * a.qtiles;
+            const int grp = idx / per_group, in = idx - grp * per_group;
+            const int first = grp * gsz;
+            const int cur = hx - first < gsz ? hx - first : gsz;   // the last group may be short
+            qt = a.qtiles - 1 - in / cur;
+            bh = xcd * hx + first + in % cur;
         }
     }
     const int b = bh / a.H, hd = bh - b * a.H;
@@ -707,6 +715,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
             constexpr int R = AIDN_ATTN_RING;
+            static_assert(8 % R == 0, "the fragment ring is indexed s % R over 8 steps");
             u32x4 fr[R];
 #pragma unroll
             for (int s = 0; s < R; s++) fr[s] = k_frag(0, s);
@@ -792,14 +801,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             }
             __builtin_amdgcn_s_setprio(0);
         }
-#if defined(AIDN_ATTN_ABL) && (AIDN_ATTN_ABL & 2)
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-#else
         __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA of tile j+1 has landed ...
-#endif
-#if !(defined(AIDN_ATTN_ABL) && (AIDN_ATTN_ABL & 1))
         __syncthreads();                    // ... everyone's has, and everyone is done with tile j
-#endif
     };
     for (int j = 0; j < ntiles; j += 2) {
         tile_body(j, std::integral_constant<int, 0>{});

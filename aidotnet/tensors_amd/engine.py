@@ -17,6 +17,7 @@ import torch
 
 from .backend import (ArgumentException, ArgumentNullException, ArgumentOutOfRangeException, Mi355Backend,
                       NotSupportedException)
+from .precision import GpuPrecisionDiagnostics, GpuPrecisionOperation, GpuPrecisionPlanner, GpuScalarType, scalar_type_for
 
 _KIND = {torch.float32: "f32", torch.float16: "f16", torch.bfloat16: "bf16"}
 
@@ -26,10 +27,28 @@ class Mi355Engine:
         self.backend = backend or Mi355Backend()
 
     # ------------------------------------------------------------------ MatMul
+    def _storage_as(self, t: torch.Tensor, storage: GpuScalarType) -> torch.Tensor:
+        """``t`` in the storage type a plan asks for, converted on the device by the backend's converters when it differs
+        (AllocateReducedPrecisionInput, DirectGpuTensorEngine.cs:19520-19545; the reference's upload widens 16-bit tensors)."""
+        want = {GpuScalarType.Float32: torch.float32, GpuScalarType.Float16: torch.float16, GpuScalarType.BFloat16: torch.bfloat16}[storage]
+        if t.dtype == want:
+            return t
+        be = self.backend
+        if t.dtype != torch.float32 and want != torch.float32:                   # 16-bit -> the other 16-bit type: through fp32
+            t = self._storage_as(t, GpuScalarType.Float32)
+        out = torch.empty(t.shape, dtype=want, device=t.device)
+        convert = {(torch.float32, torch.float16): be.ConvertToFp16, (torch.float32, torch.bfloat16): be.ConvertToBf16,
+                   (torch.float16, torch.float32): be.ConvertToFp32, (torch.bfloat16, torch.float32): be.ConvertBf16ToFp32}[(t.dtype, want)]
+        convert(be.WrapTensor(t), be.WrapTensor(out), t.numel())
+        return out
+
     def TensorMatMul(self, a: torch.Tensor, b: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
         """rank-2 x rank-2, ND x 2D (leading dims collapse into M) and ND x ND of equal rank
-        (batched), as CpuEngine.TensorMatMul (CpuEngine.cs:12458-12575).  fp16 / bf16 inputs use
-        fp32 accumulation; out_dtype float32 selects the fp32-output route (GemmFp16In32fOut)."""
+        (batched), as CpuEngine.TensorMatMul (CpuEngine.cs:12458-12575).  The compute format comes from the precision
+        planner under the current ``GpuExecutionPolicyScope`` (DirectGpuTensorEngine.cs:19660-19857 with ExecutePlannedGemm
+        :19547-19590): by default 16-bit tensors multiply in their own type and fp32 tensors in fp32; an explicit Float16 /
+        BFloat16 preference converts fp32 operands on the device and runs the fp32-output half GEMM.  Accumulation is always
+        fp32.  The result has the operands' dtype (``out_dtype`` float32 keeps the fp32 accumulator of a 16-bit product)."""
         if a is None or b is None:
             raise ArgumentNullException("a" if a is None else "b")
         if a.dim() < 2 or b.dim() < 2:
@@ -43,19 +62,50 @@ class Mi355Engine:
         K, N = b.shape[-2], b.shape[-1]
         out_dtype = out_dtype or a.dtype
         if b.dim() == 2:
+            plan = GpuPrecisionPlanner.CreatePlan(a.dtype, GpuPrecisionOperation.MatMul, "TensorMatMul" if a.dim() == 2 else "TensorMatMul.NDx2D")
             M = a.numel() // K
-            out = torch.empty(*a.shape[:-1], N, dtype=out_dtype, device=a.device)
-            A, B, C = be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(out)
-            if a.dtype == torch.float32:
+            sa = self._storage_as(a, plan.InputStorage); sb = self._storage_as(b, plan.InputStorage)
+            # a 16-bit result of a 16-bit product is the fp32 accumulator rounded once: the 16-bit-output kernels do that in their epilogue
+            direct16 = sa.dtype != torch.float32 and out_dtype == sa.dtype
+            out = torch.empty(*a.shape[:-1], N, dtype=out_dtype if (direct16 or out_dtype == torch.float32) else torch.float32, device=a.device)
+            A, B, C = be.WrapTensor(sa), be.WrapTensor(sb), be.WrapTensor(out)
+            if sa.dtype == torch.float32:
                 be.Gemm(A, B, C, M, N, K)
-            elif a.dtype == torch.float16:
-                (be.GemmFp16In32fOut if out_dtype == torch.float32 else be.Hgemm)(A, B, C, M, N, K)
+            elif sa.dtype == torch.float16:
+                (be.Hgemm if direct16 else be.GemmFp16In32fOut)(A, B, C, M, N, K)
             else:
-                (be.GemmBf16In32fOut if out_dtype == torch.float32 else be.Bf16Gemm)(A, B, C, M, N, K)
-            return out
+                (be.Bf16Gemm if direct16 else be.GemmBf16In32fOut)(A, B, C, M, N, K)
+            GpuPrecisionDiagnostics.Publish(plan)
+            return out if out.dtype == out_dtype else self._storage_as(out, scalar_type_for(out_dtype))
         if a.dim() != b.dim() or a.shape[:-2] != b.shape[:-2]:
             raise ArgumentException("batched TensorMatMul needs equal leading dimensions")
         return self.BatchMatMul(a, b)
+
+    def TensorMatMulTransposed(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+        """a [..., M, K] times the transpose of b stored [..., N, K] -> [..., M, N] (CpuEngine.cs:12337-12452 for the argument rules;
+        DirectGpuTensorEngine.cs:19860-19905: rank 2 runs the backend's MatMulTransposed, which reads B in place with no transposed
+        copy; other ranks materialise the transpose and take TensorMatMul).  The backend route is fp32: 16-bit tensors are widened
+        on the device, as the reference's upload does, and the result returns in the operands' dtype."""
+        if a is None or b is None:
+            raise ArgumentNullException("a" if a is None else "b")
+        if a.dim() < 2 or b.dim() < 2:
+            raise ArgumentException("TensorMatMulTransposed requires rank >= 2 for both operands.")
+        if a.dtype != b.dtype or a.dtype not in _KIND:
+            raise NotSupportedException("TensorMatMulTransposed: unsupported dtype combination %s x %s" % (a.dtype, b.dtype))
+        M, K, N, Kb = a.shape[-2], a.shape[-1], b.shape[-2], b.shape[-1]
+        if K != Kb:
+            raise ArgumentException("TensorMatMulTransposed K mismatch: a's trailing dim %d != b's trailing dim %d." % (K, Kb))
+        if a.dim() != 2 or b.dim() != 2:
+            return self.TensorMatMul(a, b.transpose(-1, -2).contiguous())
+        plan = GpuPrecisionPlanner.CreatePlan(a.dtype, GpuPrecisionOperation.MatMulTransposed, "TensorMatMulTransposed")
+        if plan.InputStorage != GpuScalarType.Float32:
+            raise NotSupportedException("The selected %s transposed GEMM route has no backend dispatch implementation." % plan.InputStorage.name)
+        be = self.backend
+        sa = self._storage_as(a.contiguous(), GpuScalarType.Float32); sb = self._storage_as(b.contiguous(), GpuScalarType.Float32)
+        out = torch.empty(M, N, dtype=torch.float32, device=a.device)
+        be.MatMulTransposed(be.WrapTensor(sa), be.WrapTensor(sb), be.WrapTensor(out), M, N, K)
+        GpuPrecisionDiagnostics.Publish(plan)
+        return out if a.dtype == torch.float32 else self._storage_as(out, scalar_type_for(a.dtype))
 
     _ACTIVATIONS = {"None": 0, "ReLU": 1, "GELU": 2, "Sigmoid": 3, "Tanh": 4, "LeakyReLU": 5, "Swish": 6}
 
@@ -125,12 +175,18 @@ class Mi355Engine:
         """[..., M, K] x [..., K, N], fp32 (DirectGpuTensorEngine.cs:19987-20019 -> BatchedGemm)."""
         if a.dtype != torch.float32 or b.dtype != torch.float32:
             raise NotSupportedException("BatchMatMul is fp32 only (as the reference's batched route)")
+        # the batched backend contract is fp32: a reduced-precision preference resolves to Float32 here or is refused
+        # (ExecutePlannedBatchedGemm, DirectGpuTensorEngine.cs:19592-19624)
+        plan = GpuPrecisionPlanner.CreatePlan(a.dtype, GpuPrecisionOperation.BatchMatMul, "BatchMatMul")
+        if plan.InputStorage != GpuScalarType.Float32:
+            raise NotSupportedException("No batched GEMM dispatch exists for %s storage." % plan.InputStorage.name)
         a = a.contiguous(); b = b.contiguous()
         M, K, N = a.shape[-2], a.shape[-1], b.shape[-1]
         batch = a.numel() // (M * K)
         out = torch.empty(*a.shape[:-2], M, N, dtype=torch.float32, device=a.device)
         be = self.backend
         be.BatchedGemm(be.WrapTensor(a), be.WrapTensor(b), be.WrapTensor(out), M, N, K, batch)
+        GpuPrecisionDiagnostics.Publish(plan)
         return out
 
     # ------------------------------------------------------------------ attention

@@ -302,3 +302,64 @@ def decode_f32(q, k, v, heads, kv_heads, head_dim, seq_len, scale) -> np.ndarray
     lib().orc_decode_f32(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), _p(out, _f32p),
                          heads, kv_heads, head_dim, seq_len, ctypes.c_float(scale))
     return out
+
+
+# ------------------------------------------------- secondary reference paths
+def sgemm_direct_applies(m: int, k: int, n: int) -> bool:
+    """The gate of ``SgemmAddInternal`` that sends a product to the no-pack kernel (SimdGemm.cs:1575-1613)."""
+    return bool(lib().orc_sgemm_direct_applies(int(m), int(k), int(n)))
+
+
+def thin_m_direct_applies(m: int, n: int, k: int) -> bool:
+    """The thin-M carve-out of ``BlasManaged.Gemm`` to the same kernel (BlasManaged.cs:116-124, 139-154)."""
+    return bool(lib().orc_thin_m_direct_applies(int(m), int(n), int(k)))
+
+
+def sgemm_direct(a, b, m: int, k: int, n: int, c0=None, threads: int = 1) -> np.ndarray:
+    """``SimdGemm.SgemmDirect`` (src/AiDotNet.Tensors/Engines/Simd/SimdGemm.cs:1888-2075): one fused chain over k per element;
+    ``c0`` None = cleared output (store), else accumulate into a copy of it."""
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    assert a.size == m * k and b.size == k * n
+    c = np.zeros((m, n), np.float32) if c0 is None else np.array(c0, np.float32).reshape(m, n).copy()
+    lib().orc_sgemm_direct(_p(a, _f32p), k, _p(b, _f32p), n, _p(c, _f32p), m, k, n, 1 if c0 is None else 0, threads)
+    return c
+
+
+def goto_choose_blocks(m: int, n: int, cores: int):
+    """``GotoGemmFp32.ChooseParallelBlocks`` (src/AiDotNet.Tensors/Engines/BlasManaged/GotoGemmFp32.cs:91-121) -> (mc, nc, kc)."""
+    out = np.zeros(3, np.int32)
+    lib().orc_goto_choose_blocks(int(m), int(n), int(cores), _p(out, _i32p))
+    return int(out[0]), int(out[1]), int(out[2])
+
+
+def goto_gemm(a, b, m: int, k: int, n: int, blocks=None, cores: int = 16, threads: int = 0) -> np.ndarray:
+    """``GotoGemmFp32.RunParallel`` (GotoGemmFp32.cs:319-480): tile grid of (mc, nc), K-panels of kc, scalar tails.
+    ``blocks`` None = the reference's choice for a host with ``cores`` workers."""
+    a = _c(a, np.float32); b = _c(b, np.float32)
+    assert a.size == m * k and b.size == k * n
+    mc, nc, kc = blocks if blocks is not None else goto_choose_blocks(m, n, cores)
+    c = np.full((m, n), np.nan, np.float32)
+    lib().orc_goto_gemm(_p(a, _f32p), k, _p(b, _f32p), n, _p(c, _f32p), n, m, n, k, mc, nc, kc, threads or max_threads())
+    return c
+
+
+def fast_exp(x) -> np.ndarray:
+    """``SimdKernels.FastExp256`` per lane (src/AiDotNet.Tensors/Engines/Simd/SimdKernels.cs:3025-3077)."""
+    x = _c(x, np.float32)
+    L = lib()
+    L.orc_fast_exp.argtypes = [ctypes.c_float]
+    L.orc_fast_exp.restype = ctypes.c_float
+    return np.array([L.orc_fast_exp(float(t)) for t in x.ravel()], np.float32).reshape(x.shape)
+
+
+def fused_attention_fastexp(q, k, v, scale: float, causal: bool = False, threads: int = 0) -> np.ndarray:
+    """``FusedAttention.BatchedFlashAttention`` / ``FlashAttentionForward`` (src/AiDotNet.Tensors/Engines/Simd/FusedAttention.cs:
+    39-90, 292-325): q ``[..., seqQ, d]``, k and v ``[..., seqK, d]`` with equal leading dimensions -> out like q."""
+    q = _c(q, np.float32); k = _c(k, np.float32); v = _c(v, np.float32)
+    seq_q, d = q.shape[-2:]
+    seq_k = k.shape[-2]
+    bh = int(np.prod(q.shape[:-2], dtype=np.int64)) if q.ndim > 2 else 1
+    out = np.full(q.shape, np.nan, np.float32)
+    lib().orc_fused_attention_fastexp(_p(q, _f32p), _p(k, _f32p), _p(v, _f32p), _p(out, _f32p), bh, seq_q, seq_k, d,
+                                      ctypes.c_float(scale), int(causal), threads or max_threads())
+    return out
