@@ -119,6 +119,10 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 1 GiB device copies (a plain copy kernel of known size) so that FETCH_SIZE / "
                          "WRITE_SIZE counters collected over this command can be scaled")
+    ap.add_argument("--diagnostic-data", choices=["zeros", "ones"], default=None,
+                    help="NOT the metric: fill every operand with one value instead of seeded Gaussians.  The instruction stream is the "
+                         "same, the switching activity in the data paths is minimal; the difference to the default run is what the "
+                         "board's power management costs at this load")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards without "
@@ -139,6 +143,8 @@ def main() -> int:
     dts = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
 
     def randn(*shape, std=1.0, kind="f32"):
+        if args.diagnostic_data is not None:
+            return torch.full(shape, 0.0 if args.diagnostic_data == "zeros" else 1.0, device="cuda", dtype=dts[kind])
         return (std * torch.randn(*shape, device="cuda", generator=g)).to(dts[kind])
 
     # ------------------------------------------------------------------ headline: fp16 GEMM 8192^3
@@ -153,7 +159,7 @@ def main() -> int:
     out = {
         "metric": METRIC, "value": round(value, 3), "unit": "TFLOP/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": round(ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic" if args.diagnostic_data is None else "DIAGNOSTIC all-%s operands (not the metric)" % args.diagnostic_data,
         "config": {"workload": "fp16 GEMM C=A*B, M=N=K=8192, fp32 accumulate, fp16 out (A~N(0,1), B~N(0,0.02^2), seeded)",
                    "wall_ms_per_step": round(wall_ms, 5), "min_warmup_ms": MIN_WARM_MS},
         "step_stats": stats,
