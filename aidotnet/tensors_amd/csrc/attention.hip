@@ -177,12 +177,18 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
     const int* __restrict__ bt = a.bt ? a.bt + b * a.bt_bs : nullptr;
 
-    // ---- Q fragments (B operand of S^T): row qi, 16-byte chunk (2 s + h)
-    u32x4 qf[DSTEPS];
-#pragma unroll
-    for (int s = 0; s < DSTEPS; s++) {
+    // ---- Q fragments (B operand of S^T): row qi, 16-byte chunk (2 s + h).  Up to head dimension 128 they stay in registers for
+    // the whole kernel; at 256 (where O alone takes 128 registers and the kernel would spill) every tile fetches them again: the
+    // query tile is 128 KiB at most and stays in the CU's cache.
+    constexpr bool QREG = DP <= 128;
+    auto load_q = [&](int s) -> u32x4 {
         int d0 = (2 * s + h) * E;
-        qf[s] = (qi < a.Sq) ? ld16<T>(Q + (long long)qi * a.qs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+        return (qi < a.Sq) ? ld16<T>(Q + (long long)qi * a.qs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
+    };
+    u32x4 qf[QREG ? DSTEPS : 1];
+    if constexpr (QREG) {
+#pragma unroll
+        for (int s = 0; s < DSTEPS; s++) qf[s] = load_q(s);
     }
 
     // ---- number of K/V tiles this query tile needs
@@ -328,14 +334,26 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             // fp32: the two MFMA phases run at a raised wave priority, ahead of the other workgroup's softmax on the SIMD (1-3 %
             // measured; the 16-bit instances lose with it)
             if constexpr (EB == 4) __builtin_amdgcn_s_setprio(2);
+            constexpr int QA = 4;                 // Q fragments fetched ahead when they are not resident
+            u32x4 qring[QREG ? 1 : QA];
+            if constexpr (!QREG) {
+#pragma unroll
+                for (int s = 0; s < QA; s++) qring[s] = load_q(s);
+            }
 #pragma unroll
             for (int s = 0; s < DSTEPS; s++) {
+                u32x4 qs;
+                if constexpr (QREG) qs = qf[s];
+                else {
+                    qs = qring[s % QA];
+                    if (s + QA < DSTEPS) qring[s % QA] = load_q(s + QA);
+                }
 #pragma unroll
                 for (int kt = 0; kt < KT; kt++) {
                     u32x4 kf;
                     if constexpr (DMA) kf = *(const u32x4*)(Ks + stage * KBYTES + (kt * 32 + l32) * (DP * EB) + (((2 * s + h) ^ k_swz(l32)) << 4));
                     else kf = *(const u32x4*)(ks + kt * 32 * KPITCH + s * 32);
-                    Mma32<T>::run(st[kt], kf, qf[s]);
+                    Mma32<T>::run(st[kt], kf, qs);
                 }
             }
             if constexpr (EB == 4) __builtin_amdgcn_s_setprio(0);

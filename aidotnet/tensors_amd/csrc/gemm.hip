@@ -1058,20 +1058,22 @@ static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 
 // ---------------------------------------------------------------------------------------------
 // Skinny-M path (decode projections): M <= 32, 16-bit, B stored [K,N], N % 128 == 0, K % 64 == 0.
-// HBM-bound: B (K x N) is read exactly once.  grid = (N / 128, KS): each workgroup streams a 128-column
-// slab of B over its K range with the direct global->LDS load (two 20 KB stages, several workgroups per
-// CU so many loads are in flight), computes a 32 x 128 partial product on MFMA (A rows beyond M are
-// clamped duplicates that are never stored) and writes it either to C (KS == 1) or to an fp32 workspace
-// that skinny_reduce_kernel sums in split order (deterministic) and narrows.
+// HBM-bound: B (K x N) is read exactly once.  grid = (N / 128, KS), about one workgroup per CU: each workgroup streams a
+// 128-column slab of B over its K range with the direct global->LDS load through a ring of SKINNY_STAGES 20 KB stages, filled
+// SKINNY_STAGES - 1 K-tiles ahead (120 KB in flight per CU: one memory round trip covers a whole K range of up to six tiles,
+// where a two-stage ring paid one round trip per tile), computes a 32 x 128 partial product on MFMA (A rows beyond M are
+// clamped duplicates that are never stored) and writes it to an fp32 workspace that skinny_reduce_kernel sums in split order
+// (deterministic) and narrows.  Loads complete in issue order, so "tile kt has landed" is a count of younger loads.
 //   B tile [64 k][256 B]: chunk c of row k at position c ^ ((k & 3) << 2)   (transposing reads)
 //   A tile [32 m][128 B]: chunk c of row m at position c ^ ((m >> 1) & 7)   (b128 reads)
+#define SKINNY_STAGES 7
 template <typename T>
-__global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
+__global__ __launch_bounds__(256, 1) void gemm_skinny_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
 {
     typedef uint16_t raw_t;
-    constexpr int BK = 64;
+    constexpr int BK = 64, NS = SKINNY_STAGES, AHEAD = NS - 1;
     constexpr int ABYTES = 32 * 128, BBYTES = BK * 256, STAGE = ABYTES + BBYTES;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[2 * STAGE];
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];      // NS stages
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
@@ -1113,12 +1115,20 @@ __global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, f
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.0f;
 
-    issue_loads(0, 0);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    for (int kt = 0; kt < AHEAD && kt < KT; kt++) issue_loads(kt, kt);
+    int stage = 0;
     for (int kt = 0; kt < KT; kt++) {
-        const int stage = kt & 1;
-        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+        // tiles kt+1 .. kt+AHEAD-1 (those that exist) are younger than tile kt: five loads per wave each
+        switch (min(KT - 1 - kt, AHEAD - 1)) {
+            case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
+        }
+        __syncthreads();            // everyone's part of tile kt has landed, and everyone has left tile kt-1
+        if (kt + AHEAD < KT) issue_loads(kt + AHEAD, stage == 0 ? NS - 1 : stage - 1);      // into the stage tile kt-1 used
         const unsigned char* as = smem + stage * STAGE;
         const unsigned char* bs = as + ABYTES;
 #pragma unroll
@@ -1137,8 +1147,7 @@ __global__ __launch_bounds__(256, 3) void gemm_skinny_kernel(const GemmArgs g, f
             }
             Mma32<T>::run(acc, fa, fb);
         }
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
+        stage = stage + 1 == NS ? 0 : stage + 1;
     }
 
     const int col = n0 + wave * 32 + l32;
@@ -1184,7 +1193,7 @@ static bool skinny_applies(int M, int N, int K) { return M <= 32 && N % 128 == 0
 static int skinny_ksplit(int N, int K)
 {
     int slabs = N / 128, tiles = K / 64;
-    int ks = (768 + slabs - 1) / slabs;          // about three workgroups per CU
+    int ks = (256 + slabs - 1) / slabs;          // about one workgroup per CU
     if (ks > tiles) ks = tiles;
     if (ks < 1) ks = 1;
     while (tiles % ks != 0) ks--;                // equal K ranges, each a multiple of 64
@@ -1204,7 +1213,10 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
 {
     const int ks = skinny_ksplit(g.N, g.K);
     const int kper = g.K / ks;
-    hipLaunchKernelGGL((gemm_skinny_kernel<T>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), 0, stream, g, ws, ks, kper);
+    constexpr int smem = SKINNY_STAGES * (32 * 128 + 64 * 256);
+    static unsigned long long attr_done = 0;
+    if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny_kernel<T>, smem, &attr_done)) return e0;
+    hipLaunchKernelGGL((gemm_skinny_kernel<T>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), smem, stream, g, ws, ks, kper);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     long long total = (long long)g.M * g.N;

@@ -48,6 +48,8 @@ CASES = [
     (2, 2, 2, 256, 256, 128, True, 0),
     (1, 2, 2, 130, 200, 72, True, 70),      # DiT head dim 72
     (1, 1, 1, 64, 64, 256, True, 0),
+    (1, 2, 2, 300, 300, 256, True, 0),      # head dim 256 over several key tiles: Q fragments are re-fetched per tile
+    (1, 2, 1, 130, 200, 200, False, 0),     # head dim between 128 and 256, GQA
     (1, 3, 3, 200, 50, 16, True, 0),        # Sq > Sk top-left: late rows see every key
     (1, 2, 2, 5, 9, 7, False, 0),           # odd head dim: element-wise loads
 ]
@@ -202,6 +204,8 @@ HALF_CASES = [
     (1, 2, 2, 256, 256, 128, True, 0),
     (1, 2, 2, 130, 200, 72, True, 70),
     (1, 1, 1, 64, 96, 256, False, 0),
+    (1, 2, 2, 300, 300, 256, True, 0),
+    (1, 2, 1, 130, 200, 200, False, 0),
     (1, 2, 2, 5, 9, 7, False, 0),
 ]
 
