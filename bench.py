@@ -31,10 +31,17 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # measured yet.
 TRAFFIC_BYTES = {
     # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes)
-    "gemm_f16_8192": int((799260 * 2.0 + 139212) * 1024),
-    "decode_bf16": int((1048908 * 2.0 + 1088) * 1024),
-    "attn_f16_prefill": int((98519 * 2.0 + 132099) * 1024),
-    "attn_bf16_prefill": int((98466 * 2.0 + 132097) * 1024),
+    "gemm_f16_8192": int((809920 * 2.0 + 131072) * 1024),
+    "gemm_bf16_8192": int((825144 * 2.0 + 131072) * 1024),
+    "gemm_f16_proj": int((17105 * 2.0 + 24588) * 1024),
+    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49174) * 1024),
+    "gemm_f32_proj": int((43106 * 2.0 + 49152) * 1024),
+    "gemm_f32_1024": int((12324 * 2.0 + 4096) * 1024),
+    "decode_bf16": int((1048910 * 2.0 + 1088) * 1024),
+    "attn_f16_prefill": int((117711 * 2.0 + 132324) * 1024),
+    "attn_bf16_prefill": int((117516 * 2.0 + 132324) * 1024),
+    "attn_f32_prefill": int((22636 * 2.0 + 12480) * 1024),
+    "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
@@ -203,11 +210,11 @@ def main() -> int:
         if hbm:
             eb = a_.element_size()
             nbytes = (M * K + K * N) * eb + M * N * c_.element_size()
-            roof = _roof_bytes(nbytes, ms_)
+            roof = _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name))
             roof["tflops"] = round(fl / (ms_ * 1e-3) / 1e12, 3)
             roof["note"] = "%d weight matrices rotated to defeat the last-level cache" % rotate
         else:
-            roof = _roof_flops(kind, fl, ms_)
+            roof = _roof_flops(kind, fl, ms_, TRAFFIC_BYTES.get(name))
         add(name, kind, "GEMM M=%d N=%d K=%d%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else ""), ms_, roof, st_)
 
     def attn_case(name, kind, Bn, H, S, D):
