@@ -1419,8 +1419,10 @@ static bool dl16_applies(const GemmArgs& g)
 }
 
 // Tile width (in 64-column units: 4, 3 or 2) of the 16 x 16 x 32 kernel for a 16-bit problem with M % 256 == 0 and K % 64 == 0, or 0
-// when none of the widths divides N or gives at least half a chip of tiles.  A narrower tile moves more A bytes per flop (and the
-// 256 x 128 one wastes half of its B loads), so it has to win on how evenly the tiles load the 256 CUs.
+// when none of the widths divides N or the 128 x 128 / 64 x 64 tiles of the 32 x 32 x 16 kernel are expected to finish earlier.
+// Every candidate is scored as (how evenly its tiles load the 256 CUs) x (its rate per flop relative to the 256 x 256 tile): a
+// narrower tile moves more A bytes per flop (and the 256 x 128 one wastes half of its B loads); the 128 x 128 tile runs at about
+// 0.55 and the 64 x 64 tile at about 0.45 of the 256 x 256 rate (2048^3: 128 tiles of 256 x 128 take 36 us, 256 tiles of 128 x 128 29 us).
 static int dl16_width(int M, int N, int K, int batch)
 {
     if (M % 256 != 0 || K % 64 != 0) return 0;
@@ -1432,10 +1434,12 @@ static int dl16_width(int M, int N, int K, int batch)
         const int bn = 64 * widths[i];
         if (N % bn != 0) continue;
         const long long t = (long long)(M / 256) * (N / bn) * batch;
-        if (t < 128) continue;
         const double score = cu_fill(t) * eff[i];
         if (score > best_score) { best_score = score; best = widths[i]; }
     }
+    const long long t128 = (long long)((M + 127) / 128) * ((N + 127) / 128) * batch;
+    const long long t64 = (long long)((M + 63) / 64) * ((N + 63) / 64) * batch;
+    if (0.55 * cu_fill(t128) > best_score || 0.45 * cu_fill(t64) > best_score) return 0;
     return best;
 }
 
@@ -1466,7 +1470,8 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
                     }
                 }
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
-                const bool big = E == 8 ? t256 >= 128 : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
+                // (16-bit, ragged or unaligned for the 16 x 16 x 32 kernel: the 256 x 256 tile of this kernel when it scores best)
+                const bool big = E == 8 ? (t256 >= 128 && cu_fill(t256) >= 0.55 * cu_fill(t128)) : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
                 // otherwise the same kernel with 128 x 128 or 64 x 64 tiles (codes 129, 65), whichever loads the CUs better; per
                 // flop the 64 x 64 instance runs at about 0.85 (fp32) resp. 0.8 (16-bit) of the 128 x 128 one
                 if (big) tile = 256;
