@@ -839,18 +839,24 @@ template <> struct Mma16<bf16_t> {
 // tiles would leave CUs idle in the last round (4096 x 3072: 192 tiles on 256 CUs) get a tile count that fills them.  The B tile
 // keeps its 512-byte LDS rows for every TJ (the chunk swizzle needs a power-of-two row); lanes whose swizzled chunk lies past
 // the tile's columns fetch a valid chunk again and park it in a position that no fragment read touches.
-template <typename T, typename OutT, int TJ = 4>
+// HALF: the 128 x 128 tile (TJ = 2): wave tile 64 x 32, B k-rows of 256 bytes, for problems that give fewer than a chip of wider
+// tiles (2048^2, 1024 x 4096).  A K-tile is only 256 MFMA cycles per wave here, far less than a memory round trip, so the tile ring
+// has four 32 KB stages and is filled three K-tiles ahead (loads complete in issue order: "tile kt+1 has landed" is a count of
+// younger loads).
+#define DL16_HALF_STAGES 4
+template <typename T, typename OutT, int TJ = 4, bool HALF = false>
 __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 {
+    static_assert(!HALF || TJ == 2, "the 128-row tile is built for 128 columns");
     constexpr int E = 8, EB = 2;
     constexpr int WN = 4;
-    constexpr int BM = 256, BN = 64 * TJ, BK = 64;
-    constexpr int WTM = 128, WTN = 16 * TJ;
-    constexpr int TI = 8;                         // 16 x 16 blocks of the wave tile: TI x TJ
-    constexpr int BROW = 256 * EB;                // LDS pitch of a B k-row (32 chunk positions)
+    constexpr int BM = HALF ? 128 : 256, BN = 64 * TJ, BK = 64;
+    constexpr int WTM = BM / 2, WTN = 16 * TJ;
+    constexpr int TI = WTM / 16;                  // 16 x 16 blocks of the wave tile: TI x TJ
+    constexpr int BROW = (HALF ? 128 : 256) * EB; // LDS pitch of a B k-row (16 or 32 chunk positions)
     constexpr int BCH = BN / E;                   // 16-byte chunks of a k-row that hold tile columns
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
-    constexpr int LA = 4, LB = 4, RPL = 2, LPR = 32;
+    constexpr int LA = BM / 64, LB = BK * BROW / 8192, RPL = 1024 / BROW, LPR = BROW / 16;
     constexpr int OB = Elem<OutT>::BYTES;
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
@@ -881,7 +887,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     for (int i = 0; i < LB; i++) {
         const int rb = lane / LPR, pos_b = lane % LPR;
         int chunk = pos_b ^ b_swz(RPL * (LB * wave + i) + rb);
-        if (chunk >= BCH) chunk -= 32 - BCH >= BCH ? BCH : 32 - BCH;      // a valid chunk again (its LDS position is never read)
+        if (chunk >= BCH) chunk -= LPR - BCH >= BCH ? BCH : LPR - BCH;    // a valid chunk again (its LDS position is never read)
         b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
     }
     const unsigned char* a_base = A + (long long)(m0 + 8 * LA * wave_s) * g.lda * EB;
@@ -930,8 +936,21 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TJ; j++) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
 
-    issue_loads(0, 0);
-    __builtin_amdgcn_s_waitcnt(0);
+    constexpr int NS = HALF ? DL16_HALF_STAGES : 2;
+    // wait until at most `tiles` of this wave's tile loads (LA + LB instructions each) are outstanding, and for its LDS reads
+    auto wait_tiles = [&](int tiles) {
+        static_assert(!HALF || (LA + LB == 4 && NS == 4), "the wait counts below are for four loads per tile and a four-stage ring");
+        if (tiles <= 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        else if (tiles == 1) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
+    };
+    if constexpr (HALF) {
+        for (int kt = 0; kt < NS - 1 && kt < KT; kt++) issue_loads(kt, kt);
+        wait_tiles(min(KT - 1, NS - 2));
+    } else {
+        issue_loads(0, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+    }
     __syncthreads();
 
     // fa[p]: the four A fragments of half-step parity p; fb[p]: the four B fragments of k32-step parity p
@@ -941,64 +960,110 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 #pragma unroll
     for (int j = 0; j < TJ; j++) read_b(smem + ABYTES, 0, j, fb[0][j]);
 
-    for (int kt = 0; kt < KT; kt++) {
-        const int stage = kt & 1;
-        const unsigned char* as = smem + stage * STAGE;
-        const unsigned char* bs = as + ABYTES;
-        const unsigned char* an = smem + (stage ^ 1) * STAGE;
-        // the other stage was last read before the barrier inside the previous iteration
-        if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+    if constexpr (HALF) {
+        // two steps per K-tile (one k32-step each, the whole 64-row wave tile): 8 MFMAs and 8 LDS reads per step
+        int stage = 0;
+        for (int kt = 0; kt < KT; kt++) {
+            const int next = stage + 1 == NS ? 0 : stage + 1;
+            const unsigned char* as = smem + stage * STAGE;
+            const unsigned char* bs = as + ABYTES;
+            const unsigned char* an = smem + next * STAGE;
+            // the stage of tile kt-1 was last read before the barrier inside the previous iteration
+            if (kt + NS - 1 < KT) issue_loads(kt + NS - 1, stage == 0 ? NS - 1 : stage - 1);
 #pragma unroll
-        for (int u = 0; u < 4; u++) {              // half-step u = 2 s2 + hs
-            const int s2 = u >> 1, hs = u & 1;
-            if (u == 0) {
+            for (int s2 = 0; s2 < 2; s2++) {
+                if (s2 == 0) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) read_a(as, 0, 4 + i, fa[1][i]);
-                read_b(bs, 1, 0, fb[1][0]); read_b(bs, 1, 1, fb[1][1]);
-            } else if (u == 1) {
+                    for (int i = 0; i < 4; i++) read_a(as, 1, i, fa[1][i]);
 #pragma unroll
-                for (int i = 0; i < 4; i++) read_a(as, 1, i, fa[0][i]);
+                    for (int j = 0; j < TJ; j++) read_b(bs, 1, j, fb[1][j]);
+                } else {
+                    wait_tiles(min(KT - 2 - kt, NS - 2));   // this wave's part of tile kt+1 has landed (younger tiles may be in flight), its LDS reads of tile kt are done ...
+                    __syncthreads();                        // ... and so have everyone else's
+                    if (kt + 1 < KT) {
 #pragma unroll
-                for (int j = 2; j < TJ; j++) read_b(bs, 1, j, fb[1][j]);
-            } else if (u == 2) {
+                        for (int i = 0; i < 4; i++) read_a(an, 0, i, fa[0][i]);
 #pragma unroll
-                for (int i = 0; i < 4; i++) read_a(as, 1, 4 + i, fa[1][i]);
-            } else {
-                __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed and its LDS reads of this tile are done ...
-                __syncthreads();                    // ... and so have everyone else's
-                if (kt + 1 < KT) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++) read_a(an, 0, i, fa[0][i]);
-#pragma unroll
-                    for (int j = 0; j < TJ; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
+                        for (int j = 0; j < TJ; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
+                    }
                 }
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int jj = 0; jj < TJ; jj++) {
+                        const int j = (i & 1) ? TJ - 1 - jj : jj;
+                        Mma16<T>::run(acc[i][j], fb[s2][j], fa[s2][i]);
+                    }
+                constexpr int NM = 4 * TJ, RR = 4 + 2 * TJ;
+                spread_schedule<RR, RR, 0, 0>();
+                if (NM > RR) __builtin_amdgcn_sched_group_barrier(0x008, NM - RR, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int jj = 0; jj < TJ; jj++) {
-                    const int j = (i & 1) ? TJ - 1 - jj : jj;
-                    Mma16<T>::run(acc[4 * hs + i][j], fb[s2][j], fa[hs][i]);
-                }
-            // one LDS read behind each of the first MFMAs, the remaining MFMAs after the reads have been issued
-            constexpr int NM = 4 * TJ;                                   // MFMAs per half-step
-            constexpr int R0 = 8, R1 = 4 + 2 * (TJ - 2), R2 = 4, R3 = 4 + 2 * TJ;      // LDS reads of the four half-steps
-            if (u == 0) { spread_schedule<R0, R0, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R0, 0); }
-            else if (u == 1) { spread_schedule<R1, R1, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R1, 0); }
-            else if (u == 2) { spread_schedule<R2, R2, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R2, 0); }
-            else { spread_schedule<R3, R3, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R3, 0); }
-            __builtin_amdgcn_sched_barrier(0);
+            stage = next;
         }
-    }
+    } else {
+    for (int kt = 0; kt < KT; kt++) {
+            const int stage = kt & 1;
+            const unsigned char* as = smem + stage * STAGE;
+            const unsigned char* bs = as + ABYTES;
+            const unsigned char* an = smem + (stage ^ 1) * STAGE;
+            // the other stage was last read before the barrier inside the previous iteration
+            if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
+    #pragma unroll
+            for (int u = 0; u < 4; u++) {              // half-step u = 2 s2 + hs
+                const int s2 = u >> 1, hs = u & 1;
+                if (u == 0) {
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) read_a(as, 0, 4 + i, fa[1][i]);
+                    read_b(bs, 1, 0, fb[1][0]); read_b(bs, 1, 1, fb[1][1]);
+                } else if (u == 1) {
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) read_a(as, 1, i, fa[0][i]);
+    #pragma unroll
+                    for (int j = 2; j < TJ; j++) read_b(bs, 1, j, fb[1][j]);
+                } else if (u == 2) {
+    #pragma unroll
+                    for (int i = 0; i < 4; i++) read_a(as, 1, 4 + i, fa[1][i]);
+                } else {
+                    __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed and its LDS reads of this tile are done ...
+                    __syncthreads();                    // ... and so have everyone else's
+                    if (kt + 1 < KT) {
+    #pragma unroll
+                        for (int i = 0; i < 4; i++) read_a(an, 0, i, fa[0][i]);
+    #pragma unroll
+                        for (int j = 0; j < TJ; j++) read_b(an + ABYTES, 0, j, fb[0][j]);
+                    }
+                }
+    #pragma unroll
+                for (int i = 0; i < 4; i++)
+    #pragma unroll
+                    for (int jj = 0; jj < TJ; jj++) {
+                        const int j = (i & 1) ? TJ - 1 - jj : jj;
+                        Mma16<T>::run(acc[4 * hs + i][j], fb[s2][j], fa[hs][i]);
+                    }
+                // one LDS read behind each of the first MFMAs, the remaining MFMAs after the reads have been issued
+                constexpr int NM = 4 * TJ;                                   // MFMAs per half-step
+                constexpr int R0 = 8, R1 = 4 + 2 * (TJ - 2), R2 = 4, R3 = 4 + 2 * TJ;      // LDS reads of the four half-steps
+                if (u == 0) { spread_schedule<R0, R0, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R0, 0); }
+                else if (u == 1) { spread_schedule<R1, R1, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R1, 0); }
+                else if (u == 2) { spread_schedule<R2, R2, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R2, 0); }
+                else { spread_schedule<R3, R3, 0, 0>(); __builtin_amdgcn_sched_group_barrier(0x008, NM - R3, 0); }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    
+}
 
     // ---- epilogue.  acc[i][j]: the lane holds C[row 16 i + l16][columns 16 j + 4 g4 .. + 3].  Staged through the wave's 8 KiB of
     // the last stage (dead after the final barrier), 16-byte chunk c of a staged row at position c ^ ((row >> 1) & 7).
     {
-        unsigned char* stg = smem + ((KT - 1) & 1) * STAGE + wave * 8192;
+        // (HALF: every stage is dead after the final barrier; the eight waves' 8 KiB take the first two)
+        unsigned char* stg = smem + (HALF ? 0 : ((KT - 1) & 1) * STAGE) + wave * 8192;
         constexpr int ROWB = WTN * OB;                // bytes of one staged row
         constexpr int CPR = ROWB / 16;                // 16-byte chunks per staged row
         constexpr int FIT = 8192 / (16 * ROWB);       // 16-row blocks that fit the wave's 8 KiB
-        constexpr int IPR = FIT >= 8 ? 8 : FIT >= 4 ? 4 : FIT >= 2 ? 2 : 1;      // blocks per round (divides TI)
+        constexpr int IPR0 = FIT >= 8 ? 8 : FIT >= 4 ? 4 : FIT >= 2 ? 2 : 1;
+        constexpr int IPR = IPR0 < TI ? IPR0 : TI;    // blocks per round (divides TI)
         constexpr bool POW2 = (CPR & (CPR - 1)) == 0; // the XOR swizzle of the staged rows needs a power-of-two chunk count
         const int sw = POW2 ? ((l16 >> 1) & (CPR - 1) & 7) : 0;
         const bool fused = g.bias != nullptr || g.act != 0;
@@ -1043,14 +1108,14 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     }
 }
 
-template <typename T, typename OutT, int TJ = 4>
+template <typename T, typename OutT, int TJ = 4, bool HALF = false>
 static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_dl16_kernel<T, OutT, TJ>;
-    constexpr int smem = 2 * (256 * 128 + 128 * 256);
+    auto kern = gemm_dl16_kernel<T, OutT, TJ, HALF>;
+    constexpr int smem = HALF ? DL16_HALF_STAGES * (128 * 128 + 64 * 256) : 2 * (256 * 128 + 128 * 256);
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
-    g.tiles_m = g.M / 256;
+    g.tiles_m = g.M / (HALF ? 128 : 256);
     g.tiles_n = g.N / (64 * TJ);
     hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(512), smem, stream, g);
     return hipGetLastError();
@@ -1423,9 +1488,15 @@ static bool dl16_applies(const GemmArgs& g)
 // Every candidate is scored as (how evenly its tiles load the 256 CUs) x (its rate per flop relative to the 256 x 256 tile): a
 // narrower tile moves more A bytes per flop (and the 256 x 128 one wastes half of its B loads); the 128 x 128 tile runs at about
 // 0.55 and the 64 x 64 tile at about 0.45 of the 256 x 256 rate (2048^3: 128 tiles of 256 x 128 take 36 us, 256 tiles of 128 x 128 29 us).
+#define DL16_HALF_EFF 0.7
 static int dl16_width(int M, int N, int K, int batch)
 {
-    if (M % 256 != 0 || K % 64 != 0) return 0;
+    if (K % 64 != 0) return 0;
+    if (M % 256 != 0) {
+        if (M % 128 != 0 || N % 128 != 0) return 0;
+        const long long t128 = (long long)(M / 128) * (N / 128) * batch, t64 = (long long)(M / 64) * (N / 64) * batch;
+        return DL16_HALF_EFF * cu_fill(t128) >= 0.45 * cu_fill(t64) ? 1 : 0;
+    }
     const int widths[3] = {4, 3, 2};
     const double eff[3] = {1.0, 0.94, 0.8};
     int best = 0;
@@ -1439,6 +1510,8 @@ static int dl16_width(int M, int N, int K, int batch)
     }
     const long long t128 = (long long)((M + 127) / 128) * ((N + 127) / 128) * batch;
     const long long t64 = (long long)((M + 63) / 64) * ((N + 63) / 64) * batch;
+    // the 128 x 128 tile of this kernel (code 1): whole tiles only
+    if (M % 128 == 0 && N % 128 == 0 && DL16_HALF_EFF * cu_fill(t128) > best_score) { best_score = DL16_HALF_EFF * cu_fill(t128); best = 1; }
     if (0.55 * cu_fill(t128) > best_score || 0.45 * cu_fill(t64) > best_score) return 0;
     return best;
 }
@@ -1467,6 +1540,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
                         if (w == 4) return launch_gemm_dl16<T, OutT, 4>(g, batch, stream);
                         if (w == 3) return launch_gemm_dl16<T, OutT, 3>(g, batch, stream);
                         if (w == 2) return launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
+                        if (w == 1) return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
                     }
                 }
                 const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
@@ -1487,7 +1561,13 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             return tile == 192 ? launch_gemm_dl16<T, OutT, 3>(g, batch, stream) : launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
         }
     }
-    if (tile == 192 || tile == 193) return hipErrorInvalidValue;
+    if constexpr (E == 8 && !TRANSB) {
+        if (tile == 130) {                                // 128 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
+            if (!(g.M % 128 == 0 && g.N % 128 == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
+            return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
+        }
+    }
+    if (tile == 192 || tile == 193 || tile == 130) return hipErrorInvalidValue;
     if constexpr (E == 4 || !TRANSB) {
         if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;

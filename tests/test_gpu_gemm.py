@@ -466,9 +466,10 @@ def test_config2_square_8192_baseline_distribution_sampled_rows(be, kind):
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("tile,M,N,K", [(192, 256, 192, 64), (192, 512, 576, 192), (192, 256, 768, 4096), (193, 256, 128, 64),
-                                        (193, 768, 384, 320), (193, 256, 640, 2048), (256, 512, 768, 128)])
+                                        (193, 768, 384, 320), (193, 256, 640, 2048), (256, 512, 768, 128),
+                                        (130, 128, 128, 64), (130, 384, 640, 192), (130, 128, 256, 4096), (130, 1152, 384, 128)])
 def test_half_gemm_16x16x32_kernel_tile_widths(be, kind, tile, M, N, K):
-    # the 256 x 192 and 256 x 128 tiles of the 16 x 16 x 32 kernel (codes 192 / 193) and its 256 x 256 tile, forced on small whole-tile
+    # the 256 x 192, 256 x 128 and 128 x 128 tiles of the 16 x 16 x 32 kernel (codes 192 / 193 / 130) and its 256 x 256 tile, forced on small whole-tile
     # shapes: bit-exact on dyadic inputs for both output types, bias + activation epilogue, guard band, refusal of ragged shapes
     be.SetGemmTile(tile)
     try:
