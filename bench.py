@@ -86,6 +86,7 @@ def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
     for _ in range(steps):
         fn()
     end.record()
+    clk_load = _sclk_mhz()          # launches are asynchronous: for steps of a millisecond the device is still in the timed region here
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
     ms = start.elapsed_time(end) / steps
@@ -99,7 +100,7 @@ def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
     torch.cuda.synchronize()
     per = sorted(evs[i].elapsed_time(evs[i + 1]) for i in range(steps))
     stats = {"median_ms": round(per[len(per) // 2], 5), "p95_ms": round(per[min(len(per) - 1, int(math.ceil(0.95 * len(per))) - 1)], 5),
-             "min_ms": round(per[0], 5), "max_ms": round(per[-1], 5), "sclk_mhz_before_after": [clk0, clk1],
+             "min_ms": round(per[0], 5), "max_ms": round(per[-1], 5), "sclk_mhz_before_after": [clk0, clk1], "sclk_mhz_while_queued": clk_load,
              "note": "single steps timed in a second pass with one event pair each (includes the events' own cost)"}
     return ms, wall_ms, stats
 
@@ -130,6 +131,9 @@ def main() -> int:
                     help="NOT the metric: fill every operand with one value instead of seeded Gaussians.  The instruction stream is the "
                          "same, the switching activity in the data paths is minimal; the difference to the default run is what the "
                          "board's power management costs at this load")
+    ap.add_argument("--clock-probe", type=float, default=0.0, metavar="SECONDS",
+                    help="NOT the metric: keep the headline GEMM (then the bf16 causal prefill) queued for SECONDS each and sample the "
+                         "engine clock the driver reports meanwhile; prints one JSON line with the median clock and the rate")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards without "
@@ -153,6 +157,39 @@ def main() -> int:
         if args.diagnostic_data is not None:
             return torch.full(shape, 0.0 if args.diagnostic_data == "zeros" else 1.0, device="cuda", dtype=dts[kind])
         return (std * torch.randn(*shape, device="cuda", generator=g)).to(dts[kind])
+
+    if args.clock_probe > 0:
+        def sustained(fn, flops):
+            for _ in range(20):
+                fn()
+            torch.cuda.synchronize()
+            clocks, calls, t0 = [], 0, time.perf_counter()
+            while time.perf_counter() - t0 < args.clock_probe:
+                for _ in range(100):
+                    fn()
+                calls += 100
+                c = _sclk_mhz()                 # read while the hundred launches above are still queued
+                if c:
+                    clocks.append(c)
+                torch.cuda.synchronize()
+            el = time.perf_counter() - t0
+            clocks.sort()
+            return {"sclk_mhz_median": clocks[len(clocks) // 2] if clocks else None, "sclk_mhz_min": clocks[0] if clocks else None,
+                    "sclk_mhz_max": clocks[-1] if clocks else None, "us_per_call_wall": round(el / calls * 1e6, 2),
+                    "tflops_wall": round(flops * calls / el / 1e12, 1)}
+        n = 8192
+        a = randn(n, n, kind="f16"); b = randn(n, n, std=0.02, kind="f16"); c = torch.empty(n, n, device="cuda", dtype=torch.float16)
+        A, B, C = W(a), W(b), W(c)
+        probe = {"data": args.diagnostic_data or "gaussian", "seconds_each": args.clock_probe,
+                 "gemm_f16_8192": sustained(lambda: be.Hgemm(A, B, C, n, n, n), 2.0 * n * n * n)}
+        Bn, H, S, D = 4, 32, 2048, 128
+        q = randn(Bn, H, S, D, kind="bf16"); k = randn(Bn, H, S, D, kind="bf16"); v = randn(Bn, H, S, D, kind="bf16")
+        o = torch.empty(Bn, H, S, D, device="cuda"); lse = torch.empty(Bn, H, S, device="cuda")
+        probe["attn_bf16_prefill"] = sustained(
+            lambda: be.FlashAttentionHalf("bf16", W(q), W(k), W(v), W(o), W(lse), Bn, H, S, S, D, 1.0 / math.sqrt(D), True),
+            4.0 * Bn * H * D * (S * (S + 1) / 2))
+        print(json.dumps(probe))
+        return 0
 
     # ------------------------------------------------------------------ headline: fp16 GEMM 8192^3
     n = 8192
