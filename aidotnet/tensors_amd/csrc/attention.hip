@@ -32,6 +32,7 @@ struct AttnArgs {
     long long bias_bs;
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
+    int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
     const int* bt; int bsz; long long bt_bs;   // block table of a paged K/V cache (null = contiguous), block size, batch stride
@@ -541,7 +542,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
-        if (a.causal && rem == 0 && per % a.qtiles == 0) {
+        if (a.paired) {
+            // XCD-contiguous heads, qtiles / 2 workgroups per head: first the late (heavy) tile of the pair, then the early one
+            const int units = a.qtiles >> 1;
+            bh = logical / units;
+            qt = a.qtiles - 1 - (logical - bh * units);
+        } else if (a.causal && rem == 0 && per % a.qtiles == 0) {
             // every XCD owns whole heads: inside an XCD take the heads in groups of ATTN_HEAD_GROUP and hand out the query tiles of a
             // group heaviest first across its heads (all heads at once runs as fast but re-fetches K and V 3.3 times from beyond the L2)
             const int hx = per / a.qtiles;                    // heads per XCD
@@ -554,6 +560,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             bh = xcd * hx + first + in % cur;
         }
     }
+    const int npass = a.paired ? 2 : 1;
+    for (int pass = 0; pass < npass; pass++) {
+    if (pass == 1) qt = a.qtiles - 1 - qt;
     const int b = bh / a.H, hd = bh - b * a.H;
     const int kvh = hd / (a.H / a.Hkv);
     const int q0 = qt * BR;
@@ -853,6 +862,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         if (a.lse && h == 0)
             a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
     }
+    }   // pass
 }
 
 template <typename T, typename OutT>
@@ -863,7 +873,9 @@ static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
-    long long nblk = (long long)a.qtiles * a.B * a.H;
+    // causal self-attention with an even number of query tiles: pair tile i with tile qtiles-1-i, so every workgroup has the same work
+    a.paired = (a.causal && a.qoff == 0 && a.Sq == a.Sk && a.qtiles >= 2 && a.qtiles % 2 == 0) ? 1 : 0;
+    long long nblk = (long long)(a.paired ? a.qtiles / 2 : a.qtiles) * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
     return hipGetLastError();
@@ -941,6 +953,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
 {
     const bool g_attn_allow_dl = p.allow_fast_path != 0;      // 0 (test hook of the context): every shape takes the general kernel
     AttnArgs a;
+    a.paired = 0;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
     a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;

@@ -202,6 +202,9 @@ HALF_CASES = [
     (1, 4, 4, 70, 70, 64, True, 0),
     (2, 4, 2, 17, 40, 32, True, 23),
     (1, 2, 2, 256, 256, 128, True, 0),
+    (2, 3, 3, 512, 512, 128, True, 0),      # four query tiles: the fast kernel pairs tile 3 with 0 and 2 with 1 in one workgroup
+    (1, 2, 2, 384, 384, 128, True, 0),      # three query tiles: no pairing
+    (1, 3, 3, 700, 700, 128, True, 0),      # six tiles, the last one partial
     (1, 2, 2, 130, 200, 72, True, 70),
     (1, 1, 1, 64, 96, 256, False, 0),
     (1, 2, 2, 300, 300, 256, True, 0),
