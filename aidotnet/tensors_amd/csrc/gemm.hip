@@ -1265,11 +1265,27 @@ static int skinny_ksplit(int N, int K)
     return ks;
 }
 
+// Split-K for 16-bit problems whose 128 x 128 tiles fill less than half the chip over a long K (M <= 512 against a 4096-wide
+// weight): K ranges run as the batch dimension of the 128 x 128 kernel into fp32 partials, summed in range order by
+// skinny_reduce_kernel (deterministic; bias and activation there).  Returns the number of ranges, 0 = not worth it.
+static int splitk16_ranges(int M, int N, int K)
+{
+    if (M % 128 != 0 || N % 128 != 0 || K % 64 != 0) return 0;
+    const long long t = (long long)(M / 128) * (N / 128);
+    if (t > 128) return 0;                    // up to half a chip of tiles
+    int ks = (int)(256 / t);
+    if (ks > 16) ks = 16;
+    while (ks > 1 && (K % (ks * 64) != 0 || K / ks < 512)) ks--;
+    // the partials cost 8 bytes of traffic per output element and range; the product must be worth it
+    return ks >= 2 && (long long)K >= 1024 ? ks : 0;
+}
+
 #if AIDN_GEMM_PART == 0
 size_t gemm_16_workspace_bytes(int M, int N, int K)
 {
-    if (!skinny_applies(M, N, K)) return 0;
-    return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
+    if (skinny_applies(M, N, K)) return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
+    const int ks = splitk16_ranges(M, N, K);
+    return ks ? (size_t)ks * M * N * sizeof(float) : 0;
 }
 #endif
 
@@ -1661,6 +1677,23 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
     if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         float* ws = (float*)workspace;
         return out32 ? launch_skinny<T, float>(g, stream, ws) : launch_skinny<T, T>(g, stream, ws);
+    }
+    if (force_tile == 0 && workspace) {
+        const int ks = splitk16_ranges(M, N, K);
+        if (ks) {
+            GemmArgs gp = g;
+            gp.C = workspace; gp.K = K / ks; gp.ldc = N;
+            gp.sA = K / ks; gp.sB = (long long)(K / ks) * N; gp.sC = (long long)M * N;
+            gp.bias = nullptr; gp.act = 0;
+            if (dl16_applies<float>(gp)) {
+                if (hipError_t e = launch_gemm_dl16<T, float, 2, true>(gp, ks, stream)) return e;
+                const long long total = (long long)M * N;
+                const unsigned grid = (unsigned)((total + 255) / 256);
+                if (out32) hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)workspace, C, M, N, ks, bias, act, act_param, 1.0f, 0.0f);
+                else hipLaunchKernelGGL((skinny_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, (const float*)workspace, C, M, N, ks, bias, act, act_param, 1.0f, 0.0f);
+                return hipGetLastError();
+            }
+        }
     }
     if (out32) return dispatch_gemm<T, float, false>(g, 1, stream, force_tile);
     return dispatch_gemm<T, T, false>(g, 1, stream, force_tile);

@@ -148,7 +148,9 @@ def test_argument_errors_match_reference_behaviour(be):
 HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7, 13, 11), (96, 130, 80), (37, 53, 71),
                (128, 128, 64), (256, 256, 128), (512, 256, 192), (130, 260, 70), (32, 512, 4096),
                # skinny-M (decode projection) path: M <= 32, N % 128 == 0, K % 64 == 0
-               (1, 128, 64), (5, 256, 192), (17, 384, 1024), (32, 128, 64), (8, 4096, 512), (200, 304, 128), (129, 136, 256), (1000, 1000, 256)]
+               (1, 128, 64), (5, 256, 192), (17, 384, 1024), (32, 128, 64), (8, 4096, 512), (200, 304, 128), (129, 136, 256), (1000, 1000, 256),
+               # split-K through the batch dimension of the 128 x 128 kernel: few tiles over a long K (16, 8 and 2 K ranges)
+               (128, 512, 1024), (256, 1024, 4096), (384, 1152, 1536), (512, 2048, 1024)]
 
 
 def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
