@@ -515,28 +515,35 @@ __device__ __forceinline__ void dma16_addr(const void* gptr, uint32_t lds_dst)
 // TILE = 256: 8 waves (2 x 4), wave tile 128 x 64, one workgroup per CU.  TILE = 128: 4 waves (2 x 2), wave tile 64 x 64, two
 // workgroups per CU (for problems with too few 256 x 256 tiles to occupy the chip).
 // TRANSB: B is stored [N,K]; its tile is then loaded and read exactly like the A tile (rows of 128 bytes of K, b128 fragments).
-template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false>
-__global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
+// KSW = 2 (fp32, 64 x 64 tile, whole tiles): eight waves, two groups of four that take half of the k-steps of every K-tile each and are
+// summed through LDS at the end (group 0 + group 1, a fixed order).  With about one such tile per CU the four-wave form runs one wave
+// per SIMD, which has nothing to switch to while it issues loads or waits at the tile barrier (matrix pipe 69 % busy at 1024^3).
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false, int KSW = 1>
+__global__ __launch_bounds__((TILE == 256 ? 512 : 256) * KSW, TILE == 256 ? 1 : 2) void gemm_dl_kernel(const GemmArgs g)
 {
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     static_assert(TILE == 256 || TILE == 128 || TILE == 64, "tile edge");
+    static_assert(KSW == 1 || (KSW == 2 && TILE == 64 && EB == 4 && !EDGE && !TRANSB), "the split form exists for the fp32 64 x 64 tile");
     constexpr int WM = 2, WN = TILE == 256 ? 4 : 2;
     constexpr int BM = TILE, BN = TILE, BK = 128 / EB;          // 128 bytes of K per tile row: 64 halves / 32 floats
     constexpr int WTM = BM / WM, WTN = BN / WN;
     constexpr int TM = WTM / 32, TN = WTN / 32;
     constexpr int BROW = BN * EB;                 // bytes of one k-row of the B tile
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
-    constexpr int LA = BM / 8 / (WM * WN), LB = LA;   // 1 KiB wave-loads per wave per tile (4 + 4; 2 + 2 for the 64 x 64 tile)
+    constexpr int NWAVE = WM * WN * KSW;
+    constexpr int LA = BM / 8 / NWAVE, LB = LA;       // 1 KiB wave-loads per wave per tile (4 + 4; 2 + 2 for the 64 x 64 tile, 1 + 1 in its split form)
     constexpr int RPL = 1024 / BROW;              // k-rows of B per wave-load
     constexpr int LPR = 64 / RPL;                 // lanes (16-byte chunks) per B row
-    static_assert(BK * BROW / 1024 == LB * WM * WN && BN / 8 == LB * WM * WN && LA % 2 == 0, "B tile = as many wave-loads as the A tile");
+    static_assert(BK * BROW / 1024 == LB * NWAVE && BN / 8 == LB * NWAVE && (LA % 2 == 0 || KSW == 2), "B tile = as many wave-loads as the A tile");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int t = threadIdx.x;
-    const int lane = t & 63, wave = t >> 6;
+    const int lane = t & 63, wave = t >> 6;                 // wave: index among all waves (partition of the loads)
     const int l32 = lane & 31, h = lane >> 5;
-    const int wm = wave / WN, wn = wave % WN;
+    const int kgrp = KSW == 1 ? 0 : wave / (WM * WN);      // k-step group
+    const int wq = KSW == 1 ? wave : wave % (WM * WN);
+    const int wm = wq / WN, wn = wq % WN;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, gridDim.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -561,6 +568,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         const int ra = lane >> 3, pos_a = lane & 7;           // row inside the wave-load, 16-byte chunk
+        // (the swizzle of a row is ((row >> 1) & 7) with row = 8 (LA wave + i) + ra: only the parity of LA wave + i enters)
         if constexpr (!EDGE) a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
     }
 #pragma unroll
@@ -628,7 +636,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 #pragma unroll
         for (int i = 0; i < LA; i++) {
             if constexpr (EDGE) dma16_base(a_src, a_lane_off[i], as + i * 1024);
-            else dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
+            else dma16_base(a_src + i * a_step, a_lane_off[LA % 2 == 0 ? (i & 1) : ((wave + i) & 1)], as + i * 1024);
         }
 #pragma unroll
         for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i], bs + i * 1024);
@@ -640,7 +648,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
     for (int i = 0; i < TM; i++) {
         int row = wm * WTM + i * 32 + l32;
         a_off[i] = row * 128;
-        a_sw[i] = (row >> 1) & 7;
+        a_sw[i] = ((row >> 1) & 7) ^ (KSW == 2 ? 4 * kgrp : 0);      // group g reads k-steps 2 g and 2 g + 1: chunk (2 (2 g + u) + h) ^ sw
     }
     // 16-bit B fragments (transposing reads): lane j of a 16-lane group addresses k-row (base + j / 4), 8 bytes
     const int jl = lane & 15;
@@ -654,7 +662,7 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int col = wn * WTN + j * 32 + l32;
-        b_col32[j] = (((col >> 2) ^ (h << 3)) << 4) + (col & 3) * 4 + 4 * h * BROW;
+        b_col32[j] = (((col >> 2) ^ (h << 3)) << 4) + (col & 3) * 4 + 4 * h * BROW + (KSW == 2 ? 16 * kgrp * BROW : 0);
     }
 
     int bt_off[TN], bt_sw[TN];                               // B stored [N,K]: like the A fragments
@@ -715,8 +723,8 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         // the other stage was last read before the barrier inside the previous iteration
         if (kt + 1 < KT) issue_loads(kt + 1, stage ^ 1);
 #pragma unroll
-        for (int s = 0; s < 4; s++) {
-            if (s < 3) {
+        for (int s = 0; s < 4 / KSW; s++) {        // (split form: the group's two k-steps; the fragment bases carry the group's offset)
+            if (s < 4 / KSW - 1) {
                 read_frags(as, bs, s + 1, fa[(s + 1) & 1], fb[(s + 1) & 1]);
             } else {
                 __builtin_amdgcn_s_waitcnt(0);      // this wave's DMA has landed and its LDS reads of this tile are done ...
@@ -739,6 +747,26 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         }
     }
 
+    if constexpr (KSW == 2) {
+        // nobody reads the tile ring after the last barrier: group 1 parks its accumulators there, group 0 adds them to its own
+        float* red = (float*)smem;
+        if (kgrp == 1) {
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) red[(((wq * TM + i) * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+        }
+        __syncthreads();
+        if (kgrp == 1) return;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] += red[(((wq * TM + i) * TN + j) * 16 + r) * 64 + lane];
+    }
     typedef typename Raw<OutT>::type out_t;
     out_t* __restrict__ C = (out_t*)g.C + bz * g.sC;
     const bool fused = g.bias != nullptr || g.act != 0;
@@ -795,16 +823,16 @@ __global__ __launch_bounds__(TILE == 256 ? 512 : 256, TILE == 256 ? 1 : 2) void 
         }
 }
 
-template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false>
+template <typename T, typename OutT, bool EDGE = false, int TILE = 256, bool TRANSB = false, int KSW = 1>
 static hipError_t launch_gemm_dl(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE, TRANSB>;
+    auto kern = gemm_dl_kernel<T, OutT, EDGE, TILE, TRANSB, KSW>;
     constexpr int smem = 2 * (TILE * 128 + 128 * TILE);         // A tile + B tile (128 bytes of K each), two stages
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     g.tiles_m = (g.M + TILE - 1) / TILE;
     g.tiles_n = (g.N + TILE - 1) / TILE;
-    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(TILE == 256 ? 512 : 256), smem, stream, g);
+    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3((TILE == 256 ? 512 : 256) * KSW), smem, stream, g);
     return hipGetLastError();
 }
 
@@ -1589,6 +1617,10 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
             const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % (8 * E) == 0;
+            if constexpr (E == 4 && !TRANSB) {
+                // about one tile per CU: the eight-wave form (two k-step groups), so that every SIMD has a second wave to switch to
+                if (exact_fit && tiles(64, 64) <= 512) return launch_gemm_dl<T, OutT, false, 64, TRANSB, 2>(g, batch, stream);
+            }
             return exact_fit ? launch_gemm_dl<T, OutT, false, 64, TRANSB>(g, batch, stream) : launch_gemm_dl<T, OutT, true, 64, TRANSB>(g, batch, stream);
         }
     }
