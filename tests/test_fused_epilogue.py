@@ -140,7 +140,8 @@ def test_gpu_half_gemm_bias_act(be, kind, act, m, n, k):
 @pytest.mark.gpu
 def test_gpu_large_tile_and_skinny_paths_take_the_epilogue(be):
     rng = np.random.default_rng(77)
-    for (m, n, k) in ((2048, 2048, 256), (16, 4096, 512)):      # 256x256 direct-to-LDS tiles; split-K skinny path
+    # 256 x 256 direct-to-LDS tiles; split-K skinny path; 128 x 128 tiles of the 16x16x32 kernel; its split-K form (8 K ranges)
+    for (m, n, k) in ((2048, 2048, 256), (16, 4096, 512), (1024, 1024, 192), (256, 1024, 4096)):
         a = rng.standard_normal((m, k)).astype(np.float32); b = (rng.standard_normal((k, n)) / math.sqrt(k)).astype(np.float32)
         bias = rng.standard_normal(n).astype(np.float32)
         ab, ar = round_to(a, "bf16"); bb, br = round_to(b, "bf16")
