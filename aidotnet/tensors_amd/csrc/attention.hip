@@ -32,6 +32,7 @@ struct AttnArgs {
     long long bias_bs;
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
+    int hgroup;    // general kernel, causal, more workgroups than are resident at once: heads per group of the workgroup order (0 = off)
     int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
@@ -165,6 +166,21 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
             const int rank = (nblk > 256 && pid < 256) ? 255 - pid : pid;
             qt = a.qtiles - 1 - rank / nbh;
             bh = rank - (rank / nbh) * nbh;
+        } else if (a.causal && a.hgroup > 0) {
+            // A grid of several rounds: head by head (heavy tile first) leaves heavy tiles for the very end of the dispatch order
+            // and a long tail (measured: a causal launch as slow as the unmasked one).  Take the heads in groups of a.hgroup and
+            // hand out the query tiles of a group heaviest first across its heads, so that every group -- the last one included --
+            // ends on its light tiles.  When every XCD owns whole heads the groups are formed inside the XCD's own heads.
+            const bool whole = rem == 0 && per % a.qtiles == 0;
+            const int heads = whole ? per / a.qtiles : nblk / a.qtiles;      // heads the groups are cut from
+            const int at = whole ? idx : logical;                            // position among their workgroups
+            const int gsz = heads < a.hgroup ? heads : a.hgroup;
+            const int per_group = gsz * a.qtiles;
+            const int grp = at / per_group, in = at - grp * per_group;
+            const int first = grp * gsz;
+            const int cur = heads - first < gsz ? heads - first : gsz;       // the last group may be short
+            qt = a.qtiles - 1 - in / cur;
+            bh = (whole ? xcd * heads : 0) + first + in % cur;
         }
     }
     const int b = bh / a.H, hd = bh - b * a.H;
@@ -932,6 +948,8 @@ static hipError_t launch_attn(AttnArgs a, hipStream_t stream)
     a.qtiles = (a.Sq + 127) / 128;
     long long nblk = (long long)a.qtiles * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    // causal order of a grid of several rounds: groups of at least 16 heads and at least 128 workgroups
+    a.hgroup = (a.causal && nblk > 768) ? (a.qtiles >= 8 ? 16 : (128 + a.qtiles - 1) / a.qtiles) : 0;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
     return hipGetLastError();
 }
@@ -954,6 +972,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     const bool g_attn_allow_dl = p.allow_fast_path != 0;      // 0 (test hook of the context): every shape takes the general kernel
     AttnArgs a;
     a.paired = 0;
+    a.hgroup = 0;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
     a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;

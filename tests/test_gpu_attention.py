@@ -52,6 +52,8 @@ CASES = [
     (1, 2, 1, 130, 200, 200, False, 0),     # head dim between 128 and 256, GQA
     (1, 3, 3, 200, 50, 16, True, 0),        # Sq > Sk top-left: late rows see every key
     (1, 2, 2, 5, 9, 7, False, 0),           # odd head dim: element-wise loads
+    (8, 49, 49, 200, 200, 32, True, 0),     # 784 workgroups, whole heads per XCD: causal tiles handed out by head group
+    (7, 37, 37, 300, 300, 16, True, 0),     # 777 workgroups, heads straddle the XCDs: head groups over the whole grid
 ]
 
 
@@ -210,6 +212,8 @@ HALF_CASES = [
     (1, 2, 2, 300, 300, 256, True, 0),
     (1, 2, 1, 130, 200, 200, False, 0),
     (1, 2, 2, 5, 9, 7, False, 0),
+    (8, 49, 7, 200, 200, 64, True, 0),      # 784 workgroups (GQA): the head-group order of a causal grid of several rounds
+    (7, 37, 37, 300, 300, 48, True, 0),     # 777 workgroups, heads straddle the XCDs
 ]
 
 
@@ -356,7 +360,8 @@ def test_fast_path_all_masked_rows_and_large_logits(be):
 
 # --------------------------------------------------------------- fp32 head-dim-64 direct-to-LDS form of the general kernel
 @pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
-                                                                   (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
+                                                                   (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0),
+                                                                   (8, 49, 7, 200, 200, True, 0)])
 @pytest.mark.parametrize("D", [64, 128])
 def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, D, B, H, Hkv, Sq, Sk, causal, offset):
     rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + 64)
