@@ -32,7 +32,7 @@ struct AttnArgs {
     long long bias_bs;
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
-    int hgroup;    // general kernel, causal, more workgroups than are resident at once: heads per group of the workgroup order (0 = off)
+    int hgroup;    // general kernel, causal: > 0 heads per group of the workgroup order of a large grid; < 0 the placement of a small one
     int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
@@ -156,7 +156,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
-        if (a.causal && nblk <= 768) {
+        if (a.causal && a.hgroup < 0) {
             // A grid that is resident all at once (at most three workgroups per CU) is not balanced by the order of
             // dispatch: hand the query tiles out heaviest first across ALL heads, so the workgroups that end up sharing a
             // CU are a heavy one and, later in the id order, a light one.
@@ -563,17 +563,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             const int units = a.qtiles >> 1;
             bh = logical / units;
             qt = a.qtiles - 1 - (logical - bh * units);
-        } else if (a.causal && rem == 0 && per % a.qtiles == 0) {
-            // every XCD owns whole heads: inside an XCD take the heads in groups of ATTN_HEAD_GROUP and hand out the query tiles of a
-            // group heaviest first across its heads (all heads at once runs as fast but re-fetches K and V 3.3 times from beyond the L2)
-            const int hx = per / a.qtiles;                    // heads per XCD
-            const int gsz = hx < ATTN_HEAD_GROUP ? hx : ATTN_HEAD_GROUP;
+        } else if (a.causal) {
+            // take the heads in groups of ATTN_HEAD_GROUP and hand out the query tiles of a group heaviest first across its heads
+            // (all heads at once runs as fast but re-fetches K and V 3.3 times from beyond the L2; head by head leaves a heavy
+            // tile for the very end).  When every XCD owns whole heads the groups are formed inside the XCD's own heads.
+            const bool whole = rem == 0 && per % a.qtiles == 0;
+            const int heads = whole ? per / a.qtiles : nblk / a.qtiles;
+            const int at = whole ? idx : logical;
+            const int gsz = heads < ATTN_HEAD_GROUP ? heads : ATTN_HEAD_GROUP;
             const int per_group = gsz * a.qtiles;
-            const int grp = idx / per_group, in = idx - grp * per_group;
+            const int grp = at / per_group, in = at - grp * per_group;
             const int first = grp * gsz;
-            const int cur = hx - first < gsz ? hx - first : gsz;   // the last group may be short
+            const int cur = heads - first < gsz ? heads - first : gsz;   // the last group may be short
             qt = a.qtiles - 1 - in / cur;
-            bh = xcd * hx + first + in % cur;
+            bh = (whole ? xcd * heads : 0) + first + in % cur;
         }
     }
     const int npass = a.paired ? 2 : 1;
@@ -948,8 +951,9 @@ static hipError_t launch_attn(AttnArgs a, hipStream_t stream)
     a.qtiles = (a.Sq + 127) / 128;
     long long nblk = (long long)a.qtiles * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
-    // causal order of a grid of several rounds: groups of at least 16 heads and at least 128 workgroups
-    a.hgroup = (a.causal && nblk > 768) ? (a.qtiles >= 8 ? 16 : (128 + a.qtiles - 1) / a.qtiles) : 0;
+    // causal order: up to 768 workgroups the balanced placement of a grid that is (nearly) resident at once (measured equal or
+    // better than the grouped order up to that size); beyond, groups of at least 16 heads and at least 128 workgroups
+    a.hgroup = !a.causal ? 0 : nblk <= 768 ? -1 : (a.qtiles >= 8 ? 16 : (128 + a.qtiles - 1) / a.qtiles);
     hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
     return hipGetLastError();
 }
