@@ -965,7 +965,14 @@ static hipError_t dispatch_attn_d(const AttnArgs& a, bool full, hipStream_t stre
     if (D <= 32)  return full ? launch_attn<T, OutT, 32, BC, true, 2>(a, stream)  : launch_attn<T, OutT, 32, BC, false, 2>(a, stream);
     if (D <= 64)  return full ? launch_attn<T, OutT, 64, BC, true, 2>(a, stream)  : launch_attn<T, OutT, 64, BC, false, 2>(a, stream);
     if (D <= 128) return full ? launch_attn<T, OutT, 128, BC, true, 2>(a, stream) : launch_attn<T, OutT, 128, BC, false, 2>(a, stream);
-    if (D <= 256) return full ? launch_attn<T, OutT, 256, BC, true, 1>(a, stream) : launch_attn<T, OutT, 256, BC, false, 1>(a, stream);
+    if (D <= 256) {
+        // 16-bit, plain / causal, more than two workgroups per CU: 32-key tiles, so that two workgroups share a CU (10-30 % over
+        // one workgroup of 64-key tiles; smaller grids lose with it).  The other instances spill at two workgroups per CU.
+        if constexpr (Elem<T>::BYTES == 2) {
+            if (!full && (long long)((a.Sq + 127) / 128) * a.B * a.H > 512) return launch_attn<T, OutT, 256, 32, false, 2>(a, stream);
+        }
+        return full ? launch_attn<T, OutT, 256, BC, true, 1>(a, stream) : launch_attn<T, OutT, 256, BC, false, 1>(a, stream);
+    }
     return hipErrorInvalidValue;
 }
 

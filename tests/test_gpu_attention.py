@@ -213,6 +213,8 @@ HALF_CASES = [
     (1, 2, 1, 130, 200, 200, False, 0),
     (1, 2, 2, 5, 9, 7, False, 0),
     (8, 49, 7, 200, 200, 64, True, 0),      # 784 workgroups (GQA): the head-group order of a causal grid of several rounds
+    (33, 16, 16, 100, 150, 256, False, 0),  # head dim 256 on more than 512 workgroups: 32-key tiles, two workgroups per CU
+    (33, 16, 8, 130, 130, 200, True, 0),
     (7, 37, 37, 300, 300, 48, True, 0),     # 777 workgroups, heads straddle the XCDs
 ]
 
