@@ -409,12 +409,13 @@ AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
     return AIDN_OK;
 }
 
-// workspace of the small-M fp32 path (M <= 8, B [K,N]); *ws stays null when the path does not apply or a tile size is forced
+// workspace of the fp32 paths that need one: small M (M <= 8, B [K,N]) and split-K partials; mode 0 B [K,N], 1 B [N,K], 2 fp16
+// weights (small M only).  *ws stays null when no such path applies or a tile size is forced
 static int smallm_ws(Ctx* c, void* stream, int M, int N, int K, int transB, void** ws)
 {
     *ws = nullptr;
-    if (c->force_tile != 0 || transB) return 0;
-    size_t need = aidn::gemm_f32_workspace_bytes(M, N, K);
+    if (c->force_tile != 0) return 0;
+    size_t need = transB == 2 ? aidn::gemm_smallm_workspace_bytes(M, N, K) : aidn::gemm_f32_workspace_bytes(M, N, K, transB);
     if (!need) return 0;
     return acquire_ws(c, stream, need, ws);
 }
@@ -428,7 +429,7 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
     int tile = c->force_tile;
     void* ws = nullptr;
-    if (int st = smallm_ws(c, stream, M, N, K, transB, &ws)) return st;
+    if (int st = smallm_ws(c, stream, M, N, K, transB != 0, &ws)) return st;
     return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),
                       "gemm_f32");
 }
@@ -470,7 +471,7 @@ AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A,
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: unknown activation");
     void* ws = nullptr;
-    if (int st = smallm_ws(c, stream, M, N, K, 0, &ws)) return st;
+    if (int st = smallm_ws(c, stream, M, N, K, 2, &ws)) return st;
     return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param, ws),
                       "gemm_f32_f16weight");
 }

@@ -1173,7 +1173,7 @@ __global__ __launch_bounds__(256, 1) void gemm_skinny_kernel(const GemmArgs g, f
     const int n0 = blockIdx.x * 128;
     const int ks = blockIdx.y;
     const int kbeg = ks * kper;
-    const int KT = kper / BK;
+    const int KT = min(kper, g.K - kbeg) / BK;            // the last range may be shorter
     const raw_t* __restrict__ A = (const raw_t*)g.A;
     const raw_t* __restrict__ B = (const raw_t*)g.B;
 
@@ -1283,15 +1283,29 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
 
 static bool skinny_applies(int M, int N, int K) { return M <= 32 && N % 128 == 0 && K % 64 == 0 && N >= 128; }
 
-static int skinny_ksplit(int N, int K)
+// How evenly `tiles` workgroups load the 256 CUs: a CU works through its tiles at about the same rate whether it holds one or
+// several at a time, so what counts is the largest number of tiles any CU gets.
+static double cu_fill(long long tiles) { return (double)tiles / (double)(((tiles + 255) / 256) * 256); }
+
+// K ranges of the skinny paths: `tiles` K-tiles over `slabs` column slabs, one workgroup per CU at a time.  Returns the K-tiles per
+// range (the last range may be shorter); *ks = number of ranges.  Scored as (how evenly slabs x ranges load the 256 CUs) x (the
+// share of a workgroup's time that is not its first memory round trip, about three K-tiles' worth).
+static int skinny_plan(int slabs, int tiles, int* ks_out)
 {
-    int slabs = N / 128, tiles = K / 64;
-    int ks = (256 + slabs - 1) / slabs;          // about one workgroup per CU
-    if (ks > tiles) ks = tiles;
-    if (ks < 1) ks = 1;
-    while (tiles % ks != 0) ks--;                // equal K ranges, each a multiple of 64
-    return ks;
+    int best_kper = tiles, best_ks = 1;
+    double best = -1.0;
+    for (int ks = 1; ks <= 32 && ks <= tiles; ks++) {
+        const int kper = (tiles + ks - 1) / ks;
+        const int kse = (tiles + kper - 1) / kper;
+        if (kper < 4 && ks > 1) break;
+        const long long wg = (long long)slabs * kse;
+        const double score = cu_fill(wg) * (double)kper / (kper + 3.0);
+        if (score > best * 1.02) { best = score; best_kper = kper; best_ks = kse; }
+    }
+    *ks_out = best_ks;
+    return best_kper;
 }
+static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &ks); return ks; }
 
 // Split-K for 16-bit problems whose 128 x 128 tiles fill less than half the chip over a long K (M <= 512 against a 4096-wide
 // weight): K ranges run as the batch dimension of the 128 x 128 kernel into fp32 partials, summed in range order by
@@ -1320,8 +1334,8 @@ size_t gemm_16_workspace_bytes(int M, int N, int K)
 template <typename T, typename OutT>
 static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
 {
-    const int ks = skinny_ksplit(g.N, g.K);
-    const int kper = g.K / ks;
+    int ks;
+    const int kper = 64 * skinny_plan(g.N / 128, g.K / 64, &ks);
     constexpr int smem = SKINNY_STAGES * (32 * 128 + 64 * 256);
     static unsigned long long attr_done = 0;
     if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny_kernel<T>, smem, &attr_done)) return e0;
@@ -1439,6 +1453,148 @@ __global__ __launch_bounds__(256) void gemm_smallm_kernel(const GemmArgs g, floa
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Skinny-M fp32 path: 9 <= M <= 32, B stored [K,N], N % 128 == 0, K % 32 == 0 -- the fp32 form of gemm_skinny_kernel.
+// HBM-bound: B is read exactly once.  grid = (N / 128, KS); a workgroup streams a 128-column slab of B over its K range through
+// the same ring of SKINNY_STAGES 20 KB stages (32 k-rows of 512 bytes of B and 32 rows of 128 bytes of A per stage, five
+// direct-to-LDS loads per wave and K-tile), each wave multiplies the 32 x 32 block of its 32 columns on the fp32 MFMA (a 64-row
+// tile of the general kernel would spend three quarters of its matrix work on padding and run at a quarter of the memory rate)
+// and stores the partial product for skinny_reduce_kernel.
+//   B tile [32 k][512 B]: chunk c of row k at position c ^ (((k >> 2) & 1) << 3)   (32-bit reads; the lane halves read rows 4 apart)
+//   A tile [32 m][128 B]: chunk c of row m at position c ^ ((m >> 1) & 7)          (b128 reads)
+// The k index of MFMA step i of 8-k group j is 8 j + 4 h + i for both operands (h = lane half).
+#if AIDN_GEMM_PART == 0
+__global__ __launch_bounds__(256, 1) void gemm_skinny32_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
+{
+    constexpr int BK = 32, NS = SKINNY_STAGES, AHEAD = NS - 1;
+    constexpr int ABYTES = 32 * 128, BBYTES = BK * 512, STAGE = ABYTES + BBYTES;
+    extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];      // NS stages
+
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * 128;
+    const int ks = blockIdx.y;
+    const int kbeg = ks * kper;
+    const int KT = min(kper, g.K - kbeg) / BK;            // the last range may be shorter
+    const float* __restrict__ A = (const float*)g.A;
+    const float* __restrict__ B = (const float*)g.B;
+
+    // this wave's DMA per K-tile: 4 B wave-loads (k-rows 2w', 2w'+1 with w' = 4 wave + i) and A wave-load `wave` (rows 8 wave ..)
+    const float* pb[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int row = 2 * (wave * 4 + i) + (lane >> 5), pos = lane & 31;
+        pb[i] = B + (long long)(kbeg + row) * g.ldb + n0 + (pos ^ (((row >> 2) & 1) << 3)) * 4;
+    }
+    const float* pa;
+    {
+        const int row = 8 * wave + (lane >> 3), pos = lane & 7;
+        const int grow = min(row, g.M - 1);
+        pa = A + (long long)grow * g.lda + kbeg + (pos ^ ((row >> 1) & 7)) * 4;
+    }
+    auto issue_loads = [&](int kt, int stage) {
+        unsigned char* as = smem + stage * STAGE;
+        unsigned char* bs = as + ABYTES;
+        dma16_to_lds(pa + kt * BK, as + wave * 1024);
+#pragma unroll
+        for (int i = 0; i < 4; i++) dma16_to_lds(pb[i] + (long long)kt * BK * g.ldb, bs + (wave * 4 + i) * 1024);
+    };
+
+    const int a_off = l32 * 128, a_sw = (l32 >> 1) & 7;
+    const int b_col = wave * 32 + l32;                  // column inside the slab
+
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    for (int kt = 0; kt < AHEAD && kt < KT; kt++) issue_loads(kt, kt);
+    int stage = 0;
+    for (int kt = 0; kt < KT; kt++) {
+        // tiles kt+1 .. kt+AHEAD-1 (those that exist) are younger than tile kt: five loads per wave each
+        switch (min(KT - 1 - kt, AHEAD - 1)) {
+            case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(5)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(15)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(25)" ::: "memory"); break;
+        }
+        __syncthreads();            // everyone's part of tile kt has landed, and everyone has left tile kt-1
+        if (kt + AHEAD < KT) issue_loads(kt + AHEAD, stage == 0 ? NS - 1 : stage - 1);      // into the stage tile kt-1 used
+        const unsigned char* as = smem + stage * STAGE;
+        const unsigned char* bs = as + ABYTES;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const u32x4 fa = *(const u32x4*)(as + a_off + (((2 * j + h) ^ a_sw) << 4));
+            u32x4 fb;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int row = 8 * j + 4 * h + i;          // (row >> 2) & 1 == h
+                fb[i] = *(const uint32_t*)(bs + row * 512 + ((((b_col >> 2) ^ (h << 3)) << 4) + (b_col & 3) * 4));
+            }
+            Mma32<float>::run(acc, fa, fb);
+        }
+        stage = stage + 1 == NS ? 0 : stage + 1;
+    }
+
+    const int col = n0 + b_col;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = acc_row(r, h);
+        if (row < g.M) ws[((long long)ks * g.M + row) * g.N + col] = acc[r];
+    }
+}
+#endif
+
+[[maybe_unused]] static bool skinny32_applies(int M, int N, int K) { return M > 8 && M <= 32 && N % 128 == 0 && K % 32 == 0 && N >= 128; }
+
+[[maybe_unused]] static int skinny32_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 32, &ks); return ks; }
+
+// fp32: estimated run time (microseconds) of the direct-to-LDS kernel with `tile` x `tile` tiles when K is cut into `ks` ranges
+// that run as batches.  A CU works through its tiles at the same total rate whether it holds one or two at a time, so the time
+// is (tiles of the busiest CU) x (MFMA time of one padded tile); per flop the 256 and 128 tiles run at about 0.88 and the 64
+// tile at about 0.75 of the fp32 peak (614 GFLOP/s per CU).  K ranges add the pass that sums the fp32 partials.  The estimate
+// reproduces what was measured where the choice matters (128 x 50304 x 768: 186 / 93 / 96 us estimated for the three tiles,
+// 179 / 93 / 84 measured; 16 x 4096 x 4096 on 64 x 64 tiles: 73 estimated, 77 measured).
+[[maybe_unused]] static double f32_time_us(int M, int N, int K, long long batch, int tile, int ks)
+{
+    const long long wg = (long long)((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch * ks;
+    const double rounds = wg <= 2048 ? (double)((wg + 255) / 256) : (double)wg / 256.0 + 0.5;
+    const double eff = tile == 64 ? 0.75 : 0.88;
+    const double tile_us = 2.0 * tile * tile * (double)(K / ks) / (0.614e6 * eff) + 1.5;
+    double t = rounds * tile_us;
+    if (ks > 1) t += 3.0 + (double)(ks + 2) * M * N * 4.0 / 3.0e6;
+    return t;
+}
+
+// fp32 tile edge for a problem that is not split (256 only where the direct-to-LDS kernel may run it)
+[[maybe_unused]] static int f32_tile(int M, int N, int K, long long batch, bool allow256)
+{
+    int best = 128;
+    double bt = f32_time_us(M, N, K, batch, 128, 1);
+    const double t64 = f32_time_us(M, N, K, batch, 64, 1);
+    if (t64 < bt) { bt = t64; best = 64; }
+    if (allow256 && f32_time_us(M, N, K, batch, 256, 1) <= bt) best = 256;
+    return best;
+}
+
+// fp32 split-K: number of K ranges (1 = none) that the estimate prefers for a single product.  Ranges are equal multiples of 32
+// of at least 256; a split must beat the unsplit estimate by 15 % to be taken (it costs a second launch and workspace).
+[[maybe_unused]] static int splitk32_ranges(int M, int N, int K)
+{
+    if (K < 1024 || K % 32 != 0) return 1;
+    double best = f32_time_us(M, N, K, 1, f32_tile(M, N, K, 1, true), 1) * 0.85;
+    int best_ks = 1;
+    const int cand[7] = {2, 3, 4, 6, 8, 12, 16};
+    for (int i = 0; i < 7; i++) {
+        const int ks = cand[i];
+        if (K % (ks * 32) != 0 || K / ks < 256) continue;
+        const double t = std::min(f32_time_us(M, N, K, 1, 128, ks), f32_time_us(M, N, K, 1, 64, ks));
+        if (t < best) { best = t; best_ks = ks; }
+    }
+    return best_ks;
+}
+
 static bool smallm_applies(int M, int N, int K) { return M >= 1 && M <= 8 && (long long)N * K >= 4096; }
 
 // K range of one workgroup: about 1024 workgroups, at least 128 k-rows each (32 per wave), a multiple of 32
@@ -1453,11 +1609,18 @@ static int smallm_kper(int N, int K)
 }
 
 #if AIDN_GEMM_PART == 0
-size_t gemm_f32_workspace_bytes(int M, int N, int K)
+size_t gemm_smallm_workspace_bytes(int M, int N, int K)
 {
     if (!smallm_applies(M, N, K)) return 0;
     const int kper = smallm_kper(N, K);
     return (size_t)((K + kper - 1) / kper) * M * N * sizeof(float);
+}
+size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB)
+{
+    if (!transB && smallm_applies(M, N, K)) return gemm_smallm_workspace_bytes(M, N, K);
+    if (!transB && skinny32_applies(M, N, K)) return (size_t)skinny32_ksplit(N, K) * M * N * sizeof(float);
+    const int ks = splitk32_ranges(M, N, K);
+    return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
 }
 #endif
 
@@ -1505,9 +1668,6 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
 
 static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
-// How evenly `tiles` workgroups load the 256 CUs: a CU works through its tiles at about the same rate whether it holds one or
-// several at a time, so what counts is the largest number of tiles any CU gets.
-static double cu_fill(long long tiles) { return (double)tiles / (double)(((tiles + 255) / 256) * 256); }
 
 // 128 x 128 or 64 x 64 tile; rel64 = efficiency per flop of the smaller tile relative to the larger one when both load the
 // CUs equally well (measured: about 0.85 for fp32, 0.55 for the 16-bit types).
@@ -1587,16 +1747,22 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
                         if (w == 1) return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
                     }
                 }
-                const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
-                // (16-bit, ragged or unaligned for the 16 x 16 x 32 kernel: the 256 x 256 tile of this kernel when it scores best)
-                const bool big = E == 8 ? (t256 >= 128 && cu_fill(t256) >= 0.55 * cu_fill(t128)) : (t256 >= 128 && cu_fill(t256) >= cu_fill(t128));
-                // otherwise the same kernel with 128 x 128 or 64 x 64 tiles (codes 129, 65), whichever loads the CUs better; per
-                // flop the 64 x 64 instance runs at about 0.85 (fp32) resp. 0.8 (16-bit) of the 128 x 128 one
-                if (big) tile = 256;
-                else tile = choose_tile(t128, tiles(64, 64), E == 4 ? 0.85 : 0.8) == 128 ? 129 : 65;
+                if constexpr (E == 4) {
+                    // fp32 runs every tile at about the same rate per flop: the estimated time, padding included, decides
+                    const int t = f32_tile(g.M, g.N, g.K, batch, true);
+                    tile = t == 256 ? 256 : t == 128 ? 129 : 65;
+                } else {
+                    const long long t256 = tiles(256, 256), t128 = tiles(128, 128);
+                    // (16-bit, ragged or unaligned for the 16 x 16 x 32 kernel: the 256 x 256 tile of this kernel when it scores best)
+                    const bool big = t256 >= 128 && cu_fill(t256) >= 0.55 * cu_fill(t128);
+                    // otherwise the same kernel with 128 x 128 or 64 x 64 tiles (codes 129, 65), whichever loads the CUs better; per
+                    // flop the 64 x 64 instance runs at about 0.8 of the 128 x 128 one
+                    if (big) tile = 256;
+                    else tile = choose_tile(t128, tiles(64, 64), 0.8) == 128 ? 129 : 65;
+                }
             }
         }
-        if (tile == 0) tile = choose_tile(tiles(128, 128), tiles(64, 64), E == 4 ? 0.85 : 0.55);
+        if (tile == 0) tile = E == 4 ? f32_tile(g.M, g.N, g.K, batch, false) : choose_tile(tiles(128, 128), tiles(64, 64), 0.55);
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 192 || tile == 193) {                 // 256 x 192 / 256 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
@@ -1676,6 +1842,36 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
     if (force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
         return launch_smallm<false>(g, stream, (float*)workspace);
+    if (force_tile == 0 && workspace && !transB && batch == 1 && skinny32_applies(M, N, K) && aligned16(A) && aligned16(B)) {
+        int ks;
+        const int kper = 32 * skinny_plan(N / 128, K / 32, &ks);
+        constexpr int smem = SKINNY_STAGES * (32 * 128 + 32 * 512);
+        static unsigned long long attr_done = 0;
+        if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny32_kernel, smem, &attr_done)) return e0;
+        hipLaunchKernelGGL(gemm_skinny32_kernel, dim3((unsigned)(N / 128), (unsigned)ks), dim3(256), smem, stream, g, (float*)workspace, ks, kper);
+        if (hipError_t e = hipGetLastError()) return e;
+        const long long total = (long long)M * N;
+        hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const float*)workspace,
+                           C, M, N, ks, bias, act, act_param, alpha, beta);
+        return hipGetLastError();
+    }
+    if (force_tile == 0 && workspace && batch == 1) {
+        // few tiles over a long K: the K ranges run as batches into fp32 partials, summed in range order (deterministic)
+        // by the pass that also applies alpha, beta, bias and activation
+        const int ks = splitk32_ranges(M, N, K);
+        if (ks > 1) {
+            GemmArgs gp = g;
+            gp.C = workspace; gp.K = K / ks; gp.ldc = N; gp.alpha = 1.0f; gp.beta = 0.0f;
+            gp.sA = K / ks; gp.sB = transB ? (long long)(K / ks) : (long long)(K / ks) * N; gp.sC = (long long)M * N;
+            gp.bias = nullptr; gp.act = 0;
+            hipError_t e = transB ? dispatch_gemm<float, float, true>(gp, ks, stream, 0) : dispatch_gemm<float, float, false>(gp, ks, stream, 0);
+            if (e != hipSuccess) return e;
+            const long long total = (long long)M * N;
+            hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const float*)workspace,
+                               C, M, N, ks, bias, act, act_param, alpha, beta);
+            return hipGetLastError();
+        }
+    }
     if (transB) return dispatch_gemm<float, float, true>(g, batch, stream, force_tile);
     return dispatch_gemm<float, float, false>(g, batch, stream, force_tile);
 }

@@ -10,8 +10,10 @@ namespace aidn {
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
                     int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f, void* workspace = nullptr);
-// bytes of workspace that let gemm_f32 / gemm_f32_f16weight take the small-M (M <= 8, B [K,N], one batch) path; 0 = not applicable
-size_t gemm_f32_workspace_bytes(int M, int N, int K);
+// bytes of workspace that let gemm_f32 take its small-M (M <= 8, B [K,N], one batch) or split-K path, and gemm_f32_f16weight its
+// small-M path; 0 = not applicable
+size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB);
+size_t gemm_smallm_workspace_bytes(int M, int N, int K);
 // weight-only fp16 GEMM: fp32 A [M,K] x fp16 B [K,N] -> fp32 C (the weights are widened exactly, everything else is fp32)
 hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K,
                               int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f,

@@ -188,3 +188,49 @@ def test_gpu_small_m_fp16_weights_and_epilogue(be, m, k, n):
     c2 = torch.full((m * n,), float("nan"), device="cuda")
     be.GemmBiasActivationInto(W(dev(a)), W(dev(br)), W(dev(bias)), W(c2), m, n, k, 1)
     assert mixed_err(c2.cpu().numpy().reshape(m, n), t) <= 1e-4
+
+
+# ------------------------------------------------------------------------------- fp32: 9 <= M <= 32 and split-K (few tiles, long K)
+# M, K, N: the skinny path needs N % 128 == 0 and K % 32 == 0 (unequal K ranges included: 5 slabs x 37 K-tiles); the others go through
+# K ranges run as batches of the tiled kernel (K >= 1024, K % 32 == 0, tiles that do not fill the chip) or stay unsplit
+SKINNY32_SHAPES = [(9, 1024, 128), (16, 4096, 4096), (32, 1184, 640), (20, 2048, 1536), (32, 96, 256), (17, 32, 128),
+                   (16, 1024, 1000), (33, 2048, 512), (128, 4096, 1024), (200, 3072, 768), (64, 11008, 320), (100, 1056, 300)]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,k,n", SKINNY32_SHAPES)
+def test_gpu_fp32_skinny_and_split_k_match_oracle(be, m, k, n):
+    rng = np.random.default_rng(m * 7 + k + 3 * n)
+    a = (rng.standard_normal((m, k)) * 0.1).astype(np.float32); b = (rng.standard_normal((k, n)) * 0.05).astype(np.float32)
+    got = gpu_gemm(be, a, b, m, n, k)
+    t = truth64(a, b)
+    assert rel_frobenius(got, t) < 1e-4 and mixed_err(got, t) <= 1e-4
+    assert mixed_err(got, oracle.sgemm(a, b, m, k, n, threads=oracle.max_threads())) <= 1e-4
+    assert np.array_equal(got, gpu_gemm(be, a, b, m, n, k))          # fixed summation order: repeatable
+    # alpha, beta and a NaN-filled C under beta == 0
+    c0 = rng.standard_normal((m, n)).astype(np.float32)
+    got = gpu_gemm(be, a, b, m, n, k, 0.5, -2.0, c0)
+    assert mixed_err(got, 0.5 * t - 2.0 * c0.astype(np.float64)) <= 1e-4
+    got = gpu_gemm(be, a, b, m, n, k, 1.0, 0.0, np.full((m, n), np.nan, np.float32))
+    assert mixed_err(got, t) <= 1e-4
+    # B stored [N, K]
+    c = torch.full((m, n), float("nan"), device="cuda")
+    be.MatMulTransposed(be.WrapTensor(dev(a)), be.WrapTensor(dev(np.ascontiguousarray(b.T))), be.WrapTensor(c), m, n, k)
+    assert mixed_err(c.cpu().numpy(), t) <= 1e-4
+    # fused bias + activation
+    bias = rng.standard_normal(n).astype(np.float32)
+    c = torch.full((m, n), float("nan"), device="cuda")
+    be.GemmBiasActivationInto(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(dev(bias)), be.WrapTensor(c), m, n, k, be.ACT_RELU)
+    assert mixed_err(c.cpu().numpy(), np.maximum(t + bias.astype(np.float64), 0.0)) <= 1e-4
+
+
+@pytest.mark.gpu
+def test_gpu_fp32_skinny_exact_on_dyadic_inputs(be):
+    m, k, n = 24, 2048, 1536
+    a = np.random.default_rng(0).integers(-8, 9, (m, k)).astype(np.float32) / 8
+    b = np.random.default_rng(1).integers(-8, 9, (k, n)).astype(np.float32) / 8
+    assert np.array_equal(gpu_gemm(be, a, b, m, n, k).astype(np.float64), a.astype(np.float64) @ b.astype(np.float64))
+    m, k, n = 128, 4096, 512                                          # split-K through the tiled kernel
+    a = np.random.default_rng(2).integers(-8, 9, (m, k)).astype(np.float32) / 8
+    b = np.random.default_rng(3).integers(-8, 9, (k, n)).astype(np.float32) / 8
+    assert np.array_equal(gpu_gemm(be, a, b, m, n, k).astype(np.float64), a.astype(np.float64) @ b.astype(np.float64))
