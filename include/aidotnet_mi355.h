@@ -73,7 +73,10 @@ AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream);
  * accumulation (no TF32-style truncation).  M <= 8 with B [K,N] takes the bandwidth-bound small-M path (B streamed once,
  * split-K partials in the context workspace, summed in a fixed order): the GPU form of SimdGemm.SgemmNParallelSmallM /
  * SgemmConcatenatedProjections (Engines/Simd/SimdGemm.NParallelSmallM.cs:31-109); the same holds for the bias/activation
- * and fp16-weight entry points below. */
+ * and fp16-weight entry points below.  With 9 <= M <= 32 (B [K,N], N a multiple of 128, K a multiple of 32) the weight matrix is
+ * likewise streamed once, through a 32-row MFMA kernel, and larger products whose tiles would not fill the chip over a long K
+ * (K >= 1024, K a multiple of 32, either layout of B) run their K ranges side by side; both keep fp32 partials in the context
+ * workspace and sum them in range order, so results are repeatable run to run (this entry point and the bias/activation one). */
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
                      int M, int N, int K, float alpha, float beta, int transB);
 
