@@ -158,7 +158,8 @@ int decode_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, co
     if (p.softcap > 0.0f || p.mask_mode != 0)
         return fail(c, AIDN_ERR_UNSUPPORTED, "decode: soft-cap and masks are not available here; use aidn_mi355_attn_fwd_* with Sq = 1");
     p.q = q; p.k = k; p.v = v; p.o = o; p.lse = lse; p.bias = nullptr; p.mask = nullptr; p.weights = nullptr;
-    int eff = aidn::attn_decode_splits(p, splits);
+    p.allow_fast_path = c->attn_fast_path;
+    int eff = aidn::attn_decode_splits(kind, p, splits);
     size_t need = aidn::attn_decode_workspace_bytes(p, eff);
     void* ws = nullptr;
     if (scratch_override) {
@@ -293,7 +294,7 @@ int paged_common(void* ctx, void* stream, int kind, const void* q, const void* k
     p.vs[0] = 0; p.vs[1] = head_dim; p.vs[2] = (long long)kv_heads * head_dim;
     p.block_table = block_table; p.block_size = block_size; p.block_table_stride = 0;
     if (decode) {
-        int eff = aidn::attn_decode_splits(p, splits);
+        int eff = aidn::attn_decode_splits(kind, p, splits);
         size_t need = aidn::attn_decode_workspace_bytes(p, eff);
         void* ws = nullptr;
         if (need) { int st = acquire_ws(c, stream, need, &ws); if (st) return st; }

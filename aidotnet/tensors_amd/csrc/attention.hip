@@ -33,6 +33,9 @@ struct AttnArgs {
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
     int hgroup;    // general kernel, causal: > 0 heads per group of the workgroup order of a large grid; < 0 the placement of a small one
+    // fast kernel, grouped decode: the workgroup's key range is split `split` of nsplit (chunk keys each) and, when part is not
+    // null, it stores its unnormalised partial (m, l, O[128]) at part + ((b H_q + head) nsplit + split) * 130 for the merge pass
+    int nsplit, chunk; float* part;
     int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
@@ -550,7 +553,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    int bh, qt;
+    int bh, qt, split = 0;
     {
         int nblk = gridDim.x, pid = blockIdx.x;
         int per = nblk >> 3, rem = nblk & 7;
@@ -558,7 +561,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
-        if (a.paired) {
+        if (a.nsplit > 1) {
+            split = logical % a.nsplit;          // one query tile per head; the splits of a head are neighbours
+            bh = logical / a.nsplit;
+            qt = 0;
+        } else if (a.paired) {
             // XCD-contiguous heads, qtiles / 2 workgroups per head: first the late (heavy) tile of the pair, then the early one
             const int units = a.qtiles >> 1;
             bh = logical / units;
@@ -590,6 +597,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
     const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+    // keys this workgroup sees: all of them, or its split's range (which may be empty)
+    int Sk = a.Sk;
+    if (a.nsplit > 1) {
+        const int kbeg = split * a.chunk;
+        K += (long long)kbeg * a.ks[2];
+        V += (long long)kbeg * a.vs[2];
+        Sk = max(0, min(a.chunk, a.Sk - kbeg));
+    }
 
     u32x4 qf[DSTEPS];
 #pragma unroll
@@ -598,7 +613,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         qf[s] = (qi < a.Sq) ? *(const u32x4*)(Q + (long long)qi * a.qs[2] + (2 * s + h) * 8) : z;
     }
 
-    int ntiles = (a.Sk + BC - 1) / BC;
+    int ntiles = (Sk + BC - 1) / BC;
     if (a.causal) {
         long long lastkey = (long long)q0 + BR - 1 + a.qoff;
         if (lastkey < 0) ntiles = 0;
@@ -619,7 +634,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     const uint32_t v_lane_off = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (ld_key << 2)) << 4);
     auto issue_k = [&](int tile) {
         const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * 4096;
-        if (tile * BC + BC <= a.Sk) {
+        if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)K + (long long)(tile * BC + 16 * wave_s) * k_row_bytes;
 #pragma unroll
             for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
@@ -627,14 +642,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 int key = 4 * (wave * 4 + i) + ld_key;               // key inside the tile
-                int gkey = min(tile * BC + key, a.Sk - 1);           // clamp: rows past the end are masked later
+                int gkey = min(tile * BC + key, Sk - 1);           // clamp: rows past the end are masked later
                 attn_dma16(K + (long long)gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 8, dst + i * 1024);
             }
         }
     };
     auto issue_v = [&](int tile) {
         const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * 4096;
-        if (tile * BC + BC <= a.Sk) {
+        if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
 #pragma unroll
             for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
@@ -642,7 +657,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 int key = 4 * (wave * 4 + i) + ld_key;
-                int gkey = min(tile * BC + key, a.Sk - 1);
+                int gkey = min(tile * BC + key, Sk - 1);
                 attn_dma16(V + (long long)gkey * a.vs[2] + (ld_pos ^ ((key & 3) << 2)) * 8, dst + i * 1024);
             }
         }
@@ -659,7 +674,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     const int wq_min = q0 + wave * 32, wq_max = wq_min + 31;
     const float sl2 = a.scale * LOG2E;
     // tiles this wave computes: under a causal mask a prefix of the workgroup's tiles
-    int nact = ntiles;
+    int nact = wq_min < a.Sq ? ntiles : 0;      // a wave without query rows only takes part in the loads
     if (a.causal) {
         long long lk = (long long)wq_max + a.qoff;
         if (lk < 0) nact = 0;
@@ -677,7 +692,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     // last key a query may see (sequence end and causal diagonal folded into one 32-bit bound); klim carries the
     // lane's accumulator row offset 4 h so that the per-element test is against a constant
     auto key_limit = [&](int q) -> int {
-        long long lim = a.Sk - 1;
+        long long lim = Sk - 1;
         if (a.causal) { long long c = (long long)q + a.qoff; if (c < lim) lim = c; }
         return (int)(lim < -1 ? -1 : lim);
     };
@@ -724,7 +739,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         // Loads of the next tile: when this wave computes and the next tile lies fully inside the sequence they are
         // issued one per MFMA inside the first phase below (a vector-memory instruction holds the wave's issue slot for
         // some tens of cycles; there it is covered by the running MFMA).  Otherwise all at once here.
-        const bool spread = j < nact && j + 1 < ntiles && (j + 1) * BC + BC <= a.Sk;
+        const bool spread = j < nact && j + 1 < ntiles && (j + 1) * BC + BC <= Sk;
         if (j + 1 < ntiles && !spread) { issue_k(j + 1); issue_v(j + 1); }
         if (j < nact) {
             const int kv0 = j * BC;
@@ -857,6 +872,21 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
     const float l_tot = sum_with_partner32(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if (a.part) {
+        // grouped decode over several splits: query row qi is head hd * Sq + qi of the caller; unnormalised partial for the merge
+        if (qi < a.Sq) {
+            float* __restrict__ P = a.part + (((long long)bh * a.Sq + qi) * a.nsplit + split) * 130;
+            if (h == 0) { P[0] = m_ref; P[1] = l_tot; }
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int d0 = i * 32 + 8 * g + 4 * h;
+                    *(u32x2*)(P + 2 + d0) = u32x2{as_u32(oacc[i][4 * g + 0]), as_u32(oacc[i][4 * g + 1])};      // 8-byte aligned
+                    *(u32x2*)(P + 4 + d0) = u32x2{as_u32(oacc[i][4 * g + 2]), as_u32(oacc[i][4 * g + 3])};
+                }
+        }
+    } else
     if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
         out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
@@ -898,6 +928,53 @@ static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
     if (nblk > 0x7FFFFFFFLL) return hipErrorInvalidValue;
     hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
     return hipGetLastError();
+}
+
+// Grouped decode (one query row per head, H / Hkv >= 2 query heads per K/V head, 16-bit, head dimension 128, contiguous aligned
+// cache): the query heads of a K/V head are the rows of one query tile of the fast kernel, so a K/V row is fetched once for the
+// whole group instead of once per query head.  One workgroup per (batch, K/V head, split); with several splits the partials go
+// to `part` ([B*H][nsplit][130] floats: m, l, O) for the decode merge pass, with one split the kernel writes O and LSE itself.
+bool attn_group_decode_applies(int kind, const AttnParams& p)
+{
+    if (kind == 0 || p.D != 128 || p.Sq != 1 || p.Hkv <= 0 || p.H % p.Hkv != 0 || p.block_table || !p.allow_fast_path) return false;
+    const int G = p.H / p.Hkv;
+    if (G < 2 || G > 128 || !(p.scale > 0.0f)) return false;
+    auto al = [](const void* ptr, long long s0, long long s1, long long s2) {
+        return ((uintptr_t)ptr & 15u) == 0 && (s0 * 2) % 16 == 0 && (s1 * 2) % 16 == 0 && (s2 * 2) % 16 == 0;
+    };
+    if (!al(p.q, p.qs[0], p.qs[1], 0) || !al(p.k, p.ks[0], p.ks[1], p.ks[2]) || !al(p.v, p.vs[0], p.vs[1], p.vs[2])) return false;
+    const int oeb = p.out16 ? 2 : 4;
+    if (((uintptr_t)p.o & 15u) != 0 || (p.os[0] * oeb) % 16 != 0 || (p.os[1] * oeb) % 16 != 0) return false;
+    return p.ks[2] > 0 && p.ks[2] < (1LL << 28) && p.vs[2] > 0 && p.vs[2] < (1LL << 28);
+}
+
+// sk: keys every query sees (the causal offset already applied); nsplit ranges of `chunk` keys (a multiple of 64)
+hipError_t attn_group_decode(hipStream_t stream, int kind, const AttnParams& p, int sk, int nsplit, int chunk, float* part)
+{
+    const int G = p.H / p.Hkv;
+    AttnArgs a;
+    a.paired = 0; a.hgroup = 0;
+    a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = nullptr; a.mask = nullptr;
+    a.B = p.B; a.H = p.Hkv; a.Hkv = p.Hkv; a.Sq = G; a.Sk = sk; a.D = p.D;
+    a.scale = p.scale; a.causal = 0; a.qoff = 0; a.softcap = 0.0f; a.mask_mode = 0; a.bias_bs = 0;
+    a.qs[0] = p.qs[0]; a.qs[1] = p.qs[1] * G; a.qs[2] = p.qs[1];        // a query row is a query head
+    a.os[0] = p.os[0]; a.os[1] = p.os[1] * G; a.os[2] = p.os[1];
+    for (int i = 0; i < 3; i++) { a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; }
+    a.vec_in = 1; a.vec_out = 1;
+    a.bt = nullptr; a.bsz = 0; a.bt_bs = 0;
+    a.nsplit = nsplit; a.chunk = chunk; a.part = nsplit > 1 ? part : nullptr;
+    a.qtiles = 1;
+    const long long nblk = (long long)p.B * p.Hkv * nsplit;
+    if (nblk > 0x7FFFFFFFLL || sk <= 0) return hipErrorInvalidValue;
+    constexpr int smem = 2 * (64 * 256 + 64 * 256);
+    auto go = [&](auto kern) -> hipError_t {
+        static unsigned long long attr_done = 0;
+        if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
+        return hipGetLastError();
+    };
+    if (kind == 1) return p.out16 ? go(attn_fwd_dl_kernel<f16_t, f16_t>) : go(attn_fwd_dl_kernel<f16_t, float>);
+    return p.out16 ? go(attn_fwd_dl_kernel<bf16_t, bf16_t>) : go(attn_fwd_dl_kernel<bf16_t, float>);
 }
 
 // Normalised probabilities P[b,h,i,j] = exp(logit - LSE[b,h,i]) for callers that ask for the
@@ -984,6 +1061,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     AttnArgs a;
     a.paired = 0;
     a.hgroup = 0;
+    a.nsplit = 1; a.chunk = 0; a.part = nullptr;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
     a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;

@@ -233,13 +233,14 @@ static int effective_sk(const AttnParams& p)
     return (int)(lim < p.Sk ? lim : p.Sk);
 }
 
-int attn_decode_splits(const AttnParams& p, int splits)
+int attn_decode_splits(int kind, const AttnParams& p, int splits)
 {
     const int sk = effective_sk(p);
     int maxs = (sk + 255) / 256;            // at least 256 keys per split
     if (maxs < 1) maxs = 1;
     if (splits <= 0) {
-        long long bh = (long long)p.B * p.H;
+        // workgroups per split: one per query head, or one per K/V head when the grouped form runs
+        long long bh = (long long)p.B * (attn_group_decode_applies(kind, p) ? p.Hkv : p.H);
         splits = (int)((2048 + bh - 1) / bh);   // ~8 workgroups per CU
     }
     if (splits > maxs) splits = maxs;
@@ -291,6 +292,26 @@ static hipError_t dispatch_decode(const DecodeArgs& a, hipStream_t stream)
 
 hipError_t attn_decode(hipStream_t stream, int kind, const AttnParams& p, int eff_splits, void* workspace)
 {
+    if (attn_group_decode_applies(kind, p) && effective_sk(p) > 0) {
+        const int sk = effective_sk(p);
+        int chunk = (sk + eff_splits - 1) / eff_splits;
+        chunk = (chunk + 63) / 64 * 64;
+        if (hipError_t e = attn_group_decode(stream, kind, p, sk, eff_splits, chunk, (float*)workspace)) return e;
+        if (eff_splits > 1) {
+            DecodeArgs r;
+            r.q = nullptr; r.k = nullptr; r.v = nullptr; r.o = p.o; r.lse = p.lse; r.ws = (float*)workspace;
+            r.B = p.B; r.H = p.H; r.Hkv = p.Hkv; r.Sk = sk; r.D = p.D; r.scale = p.scale; r.splits = eff_splits; r.chunk = chunk;
+            r.qs[0] = p.qs[0]; r.qs[1] = p.qs[1]; r.os[0] = p.os[0]; r.os[1] = p.os[1];
+            for (int i = 0; i < 3; i++) { r.ks[i] = p.ks[i]; r.vs[i] = p.vs[i]; }
+            r.vec_in = 1; r.bt = nullptr; r.bsz = 0; r.bt_bs = 0;
+            const dim3 grid((unsigned)(p.B * p.H));
+            if (!p.out16) hipLaunchKernelGGL((decode_reduce_kernel<float>), grid, dim3(128), 0, stream, r, 128);
+            else if (kind == 1) hipLaunchKernelGGL((decode_reduce_kernel<f16_t>), grid, dim3(128), 0, stream, r, 128);
+            else hipLaunchKernelGGL((decode_reduce_kernel<bf16_t>), grid, dim3(128), 0, stream, r, 128);
+            return hipGetLastError();
+        }
+        return hipSuccess;
+    }
     DecodeArgs a;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.ws = (float*)workspace;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sk = effective_sk(p); a.D = p.D;

@@ -56,7 +56,10 @@ hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p);
 
 // Decode (Sq == 1).  eff_splits: the split count actually used for `splits` requested (<= 0 = auto).
-int attn_decode_splits(const AttnParams& p, int splits);
+int attn_decode_splits(int kind, const AttnParams& p, int splits);
+// grouped-query decode through the fast prefill kernel (the query heads of a K/V head as the rows of one query tile)
+bool attn_group_decode_applies(int kind, const AttnParams& p);
+hipError_t attn_group_decode(hipStream_t stream, int kind, const AttnParams& p, int sk, int nsplit, int chunk, float* part);
 size_t attn_decode_workspace_bytes(const AttnParams& p, int eff_splits);
 hipError_t attn_decode(hipStream_t stream, int kind, const AttnParams& p, int eff_splits, void* workspace);
 

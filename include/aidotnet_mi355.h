@@ -206,7 +206,9 @@ AIDN_API int aidn_mi355_attn_fwd_bf16(void* ctx, void* stream, const aidn_attn_d
  * (HipFlashDecodeKernels.cs:9-10; host FlashDecode HipBackend.cs:919-965) or its dense KVCache
  * [B,Sk,Hkv,D] (Engines/Autodiff/KVCache.cs:5-8).  splits <= 0 picks the split count
  * (the reference default is min(Sk, 8), HipBackend.cs:936); results do not depend on it beyond
- * rounding.  o is fp32 or the input type per desc->out_is_16bit. */
+ * rounding.  o is fp32 or the input type per desc->out_is_16bit.  Grouped-query caches (Hkv < H) in fp16 / bf16 at head
+ * dimension 128 with 16-byte aligned rows fetch each K/V row once for all query heads of its group (the group runs as the rows
+ * of one query tile on the matrix cores; the probabilities are rounded to the input type there, as in the prefill kernel). */
 AIDN_API int aidn_mi355_attn_decode_f32(void* ctx, void* stream, const aidn_attn_desc* desc,
                                const float* q, const float* k, const float* v, float* o, float* lse, int splits);
 AIDN_API int aidn_mi355_attn_decode_f16(void* ctx, void* stream, const aidn_attn_desc* desc,

@@ -127,3 +127,41 @@ def test_config5_decode_bf16_b32_h32_s4096_d128(be):
         o64, lse64 = oracle.attention_f64(qs, ks, vs, scale)
         assert mixed_err(out[b, h].cpu().numpy(), o64[0, 0]) <= 2e-2
         assert mixed_err(lse[b, h].cpu().numpy(), lse64[0, 0]) <= 1e-3
+
+
+# Grouped-query decode at head dimension 128 in the 16-bit types: the query heads of a K/V head run as the rows of one query tile of
+# the fast prefill kernel (one fetch of a K/V row for the whole group).  Checked against the fp64 oracle, against the per-head decode
+# kernel (fast path switched off) and across split counts; G = H / Hkv from 2 to 48 (more than 32 rows: a second wave computes).
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("B,H,Hkv,S,splits", [(2, 8, 4, 300, 0), (1, 32, 8, 4096, 0), (3, 12, 2, 1000, 3), (2, 32, 1, 777, 1), (5, 16, 8, 63, 0),
+                                              (1, 48, 1, 500, 2), (2, 16, 2, 64, 1), (1, 8, 2, 129, 64), (4, 32, 8, 2048, 5)])
+def test_grouped_decode_d128_matches_oracle_and_per_head_kernel(be, kind, B, H, Hkv, S, splits):
+    D = 128
+    rng = np.random.default_rng(B + 3 * H + 5 * Hkv + S)
+    q = rng.standard_normal((B, H, 1, D)).astype(np.float32)
+    k = rng.standard_normal((B, Hkv, S, D)).astype(np.float32)
+    v = rng.standard_normal((B, Hkv, S, D)).astype(np.float32)
+    scale = 1.0 / math.sqrt(D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+    dt = TORCH16[kind]
+    tq, tk, tv = from_bits16(qb, dt), from_bits16(kb, dt), from_bits16(vb, dt)
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale)
+
+    def run(out16):
+        out = torch.full((B, H, 1, D), float("nan"), device="cuda", dtype=dt if out16 else torch.float32)
+        lse = torch.full((B, H, 1), float("nan"), device="cuda")
+        be.DecodeAttention(kind, be.WrapTensor(tq), be.WrapTensor(tk), be.WrapTensor(tv), be.WrapTensor(out), B, H, S, D, scale,
+                           Hkv, splits, out16, be.WrapTensor(lse))
+        return out.float().cpu().numpy(), lse.cpu().numpy()
+
+    got, lse = run(False)
+    assert mixed_err(got, o64) <= 2e-2 and mixed_err(lse, lse64) <= 1e-3
+    got16, _ = run(True)
+    assert mixed_err(got16, o64) <= 2e-2
+    be.SetAttentionFastPath(False)
+    try:
+        per_head, per_head_lse = run(False)
+    finally:
+        be.SetAttentionFastPath(True)
+    assert mixed_err(got, per_head) <= 2e-2 and mixed_err(lse, per_head_lse) <= 1e-3
+    assert mixed_err(per_head, o64) <= 2e-2
