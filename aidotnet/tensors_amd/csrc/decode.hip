@@ -65,10 +65,31 @@ __device__ __forceinline__ void widen16(const u32x4& x, float (&f)[Elem<T>::PER1
     }
 }
 
+// Sum over the LPK consecutive lanes that share a key row (LPK a power of two >= 4, aligned): quad permutes and row mirrors are
+// VALU data-parallel-primitive operands (no LDS round trip); beyond a 16-lane row one permute and the half-wave swap.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v)
+{
+    return as_f32((uint32_t)__builtin_amdgcn_update_dpp(0, (int)as_u32(v), CTRL, 0xF, 0xF, false));
+}
+template <int LPK>
+__device__ __forceinline__ float group_sum(float p)
+{
+    p += dpp_f<0xB1>(p);                       // quad_perm [1,0,3,2]
+    p += dpp_f<0x4E>(p);                       // quad_perm [2,3,0,1]
+    if constexpr (LPK >= 8) p += dpp_f<0x141>(p);      // row_half_mirror
+    if constexpr (LPK >= 16) p += dpp_f<0x140>(p);     // row_mirror
+    if constexpr (LPK >= 32) p += shfl_xor_f(p, 16);
+    if constexpr (LPK >= 64) p = sum_with_partner32(p);
+    return p;
+}
+
 constexpr float D_LOG2E = 1.4426950408889634f;
 constexpr float D_LN2 = 0.6931471805599453f;
 
-template <typename T, typename OutT, int LPK, int U>
+// GH: query heads of one K/V head that a workgroup serves from the same loads (1 = one head per workgroup).  The K/V rows of a
+// grouped-query cache are then fetched once per GH query heads instead of once per head.
+template <typename T, typename OutT, int LPK, int U, int GH>
 __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
 {
     typedef typename Raw3<T>::type raw_t;
@@ -83,33 +104,43 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int dl = lane % LPK, sk = lane / LPK;
-    const int split = blockIdx.x, bh = blockIdx.y;
-    const int b = bh / a.H, hd = bh - b * a.H;
-    const int kvh = hd / (a.H / a.Hkv);
+    const int split = blockIdx.x;
+    // blockIdx.y = (batch, K/V head, chunk of GH query heads of that K/V head)
+    const int gq = a.H / a.Hkv;                    // query heads per K/V head (a multiple of GH)
+    const int chunks = gq / GH;
+    const int by = blockIdx.y;
+    const int b = by / (a.Hkv * chunks);
+    const int kvh = (by - b * a.Hkv * chunks) / chunks;
+    const int hd0 = kvh * gq + (by % chunks) * GH;  // first query head
     const bool vec = a.vec_in != 0;
     const int d0 = dl * E;
 
     const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
-    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
     const int* __restrict__ bt = a.bt ? a.bt + b * a.bt_bs : nullptr;
 
-    float qf[E];
-    {
+    float qf[GH][E];
+#pragma unroll
+    for (int g = 0; g < GH; g++) {
+        const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + (hd0 + g) * a.qs[1];
         u32x4 qx = ld16d<T>(Q + d0, a.D - d0, vec);
-        widen16<T>(qx, qf);
+        widen16<T>(qx, qf[g]);
         const float sl2 = a.scale * D_LOG2E;
 #pragma unroll
-        for (int e = 0; e < E; e++) qf[e] *= sl2;      // scores come out in the log2 domain
+        for (int e = 0; e < E; e++) qf[g][e] *= sl2;      // scores come out in the log2 domain
     }
 
     const int kbeg = split * a.chunk;
     const int kend = min(a.Sk, kbeg + a.chunk);
 
-    float m_run = -INFINITY, l_run = 0.0f;
-    float acc[E];
+    float m_run[GH], l_run[GH];
+    float acc[GH][E];
 #pragma unroll
-    for (int e = 0; e < E; e++) acc[e] = 0.0f;
+    for (int g = 0; g < GH; g++) {
+        m_run[g] = -INFINITY; l_run[g] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < E; e++) acc[g][e] = 0.0f;
+    }
 
     for (int base = kbeg + wave * (U * KPW); base < kend; base += NWV * U * KPW) {
         u32x4 kx[U], vx[U];
@@ -121,69 +152,88 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
             kx[u] = ok ? ld16d<T>(K + row * a.ks[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
             vx[u] = ok ? ld16d<T>(V + row * a.vs[2] + d0, a.D - d0, vec) : u32x4{0u, 0u, 0u, 0u};
         }
-        float s[U];
-        float mloc = -INFINITY;
+        float s[GH][U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             float kf[E];
             widen16<T>(kx[u], kf);
-            float p = 0.0f;
+            const bool live = base + u * KPW + sk < kend;
 #pragma unroll
-            for (int e = 0; e < E; e++) p = fmaf(qf[e], kf[e], p);
+            for (int g = 0; g < GH; g++) {
+                float p = 0.0f;
 #pragma unroll
-            for (int off = 1; off < LPK; off <<= 1) p += shfl_xor_f(p, off);
-            int key = base + u * KPW + sk;
-            s[u] = key < kend ? p : -INFINITY;
-            mloc = fmaxf(mloc, s[u]);
+                for (int e = 0; e < E; e++) p = fmaf(qf[g][e], kf[e], p);
+                p = group_sum<LPK>(p);
+                s[g][u] = live ? p : -INFINITY;
+            }
         }
-        const float m_new = fmaxf(m_run, mloc);
-        const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        m_run = m_new;
-        l_run *= alpha;
+        float pr[GH][U];
 #pragma unroll
-        for (int e = 0; e < E; e++) acc[e] *= alpha;
+        for (int g = 0; g < GH; g++) {
+            float mloc = s[g][0];
+#pragma unroll
+            for (int u = 1; u < U; u++) mloc = fmaxf(mloc, s[g][u]);
+            const float m_new = fmaxf(m_run[g], mloc);
+            const float m_use = (m_new == -INFINITY) ? 0.0f : m_new;
+            const float alpha = __builtin_amdgcn_exp2f(m_run[g] - m_use);
+            m_run[g] = m_new;
+            float l = l_run[g] * alpha;
+#pragma unroll
+            for (int e = 0; e < E; e++) acc[g][e] *= alpha;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                pr[g][u] = __builtin_amdgcn_exp2f(s[g][u] - m_use);
+                l += pr[g][u];
+            }
+            l_run[g] = l;
+        }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            float p = __builtin_amdgcn_exp2f(s[u] - m_use);
-            l_run += p;
             float vf[E];
             widen16<T>(vx[u], vf);
 #pragma unroll
-            for (int e = 0; e < E; e++) acc[e] = fmaf(p, vf[e], acc[e]);
+            for (int g = 0; g < GH; g++)
+#pragma unroll
+                for (int e = 0; e < E; e++) acc[g][e] = fmaf(pr[g][u], vf[e], acc[g][e]);
         }
     }
 
-    // ---- merge the key slots of all waves
+    // ---- merge the key slots of all waves, one query head at a time through the same LDS
     const int slot = wave * KPW + sk;
-    if (dl == 0) { s_m[slot] = m_run; s_l[slot] = l_run; }
 #pragma unroll
-    for (int e = 0; e < E; e++) s_acc[slot][d0 + e] = acc[e];
-    __syncthreads();
+    for (int g = 0; g < GH; g++) {
+        if (g > 0) __syncthreads();
+        if (dl == 0) { s_m[slot] = m_run[g]; s_l[slot] = l_run[g]; }
+#pragma unroll
+        for (int e = 0; e < E; e++) s_acc[slot][d0 + e] = acc[g][e];
+        __syncthreads();
 
-    float M = -INFINITY;
+        const int hd = hd0 + g;
+        const int bh = b * a.H + hd;
+        float M = -INFINITY;
 #pragma unroll
-    for (int i = 0; i < SLOTS; i++) M = fmaxf(M, s_m[i]);
-    const float Muse = (M == -INFINITY) ? 0.0f : M;
-    for (int d = t; d < DPAD; d += 256) {
-        float L = 0.0f, A = 0.0f;
+        for (int i = 0; i < SLOTS; i++) M = fmaxf(M, s_m[i]);
+        const float Muse = (M == -INFINITY) ? 0.0f : M;
+        for (int d = t; d < DPAD; d += 256) {
+            float L = 0.0f, A = 0.0f;
 #pragma unroll
-        for (int i = 0; i < SLOTS; i++) {
-            float w = __builtin_amdgcn_exp2f(s_m[i] - Muse);
-            L += s_l[i] * w;
-            A += s_acc[i][d] * w;
-        }
-        if (a.splits > 1) {
-            float* ws = a.ws + ((long long)bh * a.splits + split) * (2 + DPAD);
-            if (d == 0) { ws[0] = M; ws[1] = L; }
-            ws[2 + d] = A;
-        } else if (d < a.D) {
-            typedef typename Raw3<OutT>::type out_t;
-            out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
-            float r = L > 0.0f ? A / L : 0.0f;
-            if constexpr (Elem<OutT>::BYTES == 4) O[d] = as_u32(r);
-            else O[d] = (out_t)Elem<OutT>::narrow(r);
-            if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
+            for (int i = 0; i < SLOTS; i++) {
+                float w = __builtin_amdgcn_exp2f(s_m[i] - Muse);
+                L += s_l[i] * w;
+                A += s_acc[i][d] * w;
+            }
+            if (a.splits > 1) {
+                float* ws = a.ws + ((long long)bh * a.splits + split) * (2 + DPAD);
+                if (d == 0) { ws[0] = M; ws[1] = L; }
+                ws[2 + d] = A;
+            } else if (d < a.D) {
+                typedef typename Raw3<OutT>::type out_t;
+                out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
+                float r = L > 0.0f ? A / L : 0.0f;
+                if constexpr (Elem<OutT>::BYTES == 4) O[d] = as_u32(r);
+                else O[d] = (out_t)Elem<OutT>::narrow(r);
+                if (d == 0 && a.lse) a.lse[bh] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * D_LN2 : -INFINITY;
+            }
         }
     }
 }
@@ -240,7 +290,8 @@ int attn_decode_splits(int kind, const AttnParams& p, int splits)
     if (maxs < 1) maxs = 1;
     if (splits <= 0) {
         // workgroups per split: one per query head, or one per K/V head when the grouped form runs
-        long long bh = (long long)p.B * (attn_group_decode_applies(kind, p) ? p.Hkv : p.H);
+        const int gq = p.Hkv > 0 ? p.H / p.Hkv : 1;
+        long long bh = (long long)p.B * (attn_group_decode_applies(kind, p) ? p.Hkv : p.H / (gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1));
         splits = (int)((2048 + bh - 1) / bh);   // ~8 workgroups per CU
     }
     if (splits > maxs) splits = maxs;
@@ -264,8 +315,13 @@ template <typename T, typename OutT, int LPK, int U>
 static hipError_t launch_decode(DecodeArgs a, hipStream_t stream)
 {
     constexpr int DPAD = LPK * Elem<T>::PER16;
-    dim3 grid((unsigned)a.splits, (unsigned)(a.B * a.H));
-    hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U>), grid, dim3(256), 0, stream, a);
+    // query heads of a K/V head that share a workgroup (and its loads): 4, 2 or 1, whichever divides the group
+    const int gq = a.H / a.Hkv;
+    const int gh = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;
+    dim3 grid((unsigned)a.splits, (unsigned)(a.B * a.H / gh));
+    if (gh == 4) hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 4>), grid, dim3(256), 0, stream, a);
+    else if (gh == 2) hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 2>), grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 1>), grid, dim3(256), 0, stream, a);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     if (a.splits > 1) {

@@ -44,7 +44,10 @@ def test_mha_decode_matches_oracle(be, heads, d, seq, splits):
     assert mixed_err(got, want) <= 1e-4                                     # the task's
 
 
-@pytest.mark.parametrize("heads,kv,d,seq,splits", [(8, 2, 64, 50, 8), (8, 1, 32, 300, 4), (12, 4, 128, 1025, 0)])
+# query heads per K/V head 4, 8 (two workgroups of four), 3 (one head per workgroup), 6 and 2 (pairs): the heads that share a workgroup
+# share its K/V loads
+@pytest.mark.parametrize("heads,kv,d,seq,splits", [(8, 2, 64, 50, 8), (8, 1, 32, 300, 4), (12, 4, 128, 1025, 0), (12, 2, 64, 333, 0),
+                                                   (4, 2, 128, 200, 3), (16, 4, 256, 130, 2)])
 def test_gqa_decode_matches_oracle(be, heads, kv, d, seq, splits):
     got, want = _run_flash_decode(be, heads, kv, d, seq, splits, 0xABC + heads + kv + seq)
     assert mixed_err(got, want) <= 1e-4
