@@ -215,8 +215,9 @@ def main() -> int:
     others = []
     only = set(x for x in args.only.split(",") if x)
 
-    def want(name):
-        return not only or name in only
+    def want(name, extra=False):
+        # extra workloads (shapes beside the listed configurations) run only when --only names them
+        return name in only if (only or extra) else True
 
     def add(name, kind, workload, ms, roof, stats):
         others.append({"name": name, "dtype": kind, "workload": workload, "ms_per_step": round(ms, 5), "roofline": roof,
@@ -227,8 +228,8 @@ def main() -> int:
             return randn(*shape, kind=kind)
         return (2.0 * torch.rand(*shape, device="cuda", generator=g) - 1.0).to(dts[kind])
 
-    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False):
-        if not want(name):
+    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False, extra=False):
+        if not want(name, extra):
             return
         # rotate > 1: cycle through that many distinct weight matrices so the timed loop reads HBM, not the
         # 256 MB last-level cache
@@ -260,8 +261,8 @@ def main() -> int:
             roof = _roof_flops(kind, fl, ms_, TRAFFIC_BYTES.get(name))
         add(name, kind, "GEMM M=%d N=%d K=%d%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else ""), ms_, roof, st_)
 
-    def attn_case(name, kind, Bn, H, S, D):
-        if not want(name):
+    def attn_case(name, kind, Bn, H, S, D, extra=False):
+        if not want(name, extra):
             return
         q = randn(Bn, H, S, D, kind=kind); k = randn(Bn, H, S, D, kind=kind); v = randn(Bn, H, S, D, kind=kind)
         o = torch.empty(Bn, H, S, D, device="cuda"); lse = torch.empty(Bn, H, S, device="cuda")
@@ -276,16 +277,26 @@ def main() -> int:
         roof["tflops_full_matrix_convention"] = round(4.0 * Bn * H * S * S * D / (ms_ * 1e-3) / 1e12, 3)
         add(name, kind, "causal attention B=%d H=%d S=%d d=%d (fp32 softmax/accumulate, fp32 O + LSE)" % (Bn, H, S, D), ms_, roof, st_)
 
-    def decode_case(name, kind, Bn, H, S, D):
-        if not want(name):
+    def decode_case(name, kind, Bn, H, S, D, Hkv=0, rotate=1, extra=False):
+        if not want(name, extra):
             return
-        q = randn(Bn, H, 1, D, kind=kind); k = randn(Bn, H, S, D, kind=kind); v = randn(Bn, H, S, D, kind=kind)
+        # Hkv: K/V heads of a grouped-query cache (0 = one per query head); rotate: distinct caches cycled through so that a cache
+        # smaller than the 256 MB last-level cache is still read from HBM
+        kvh = Hkv or H
+        q = randn(Bn, H, 1, D, kind=kind)
+        ks_ = [randn(Bn, kvh, S, D, kind=kind) for _ in range(rotate)]
+        vs_ = [randn(Bn, kvh, S, D, kind=kind) for _ in range(rotate)]
         o = torch.empty(Bn, H, 1, D, device="cuda")
         sc = 1.0 / math.sqrt(D)
-        fn = lambda: be.DecodeAttention(kind, W(q), W(k), W(v), W(o), Bn, H, S, D, sc)
+        it = [0]
+
+        def fn():
+            j = it[0] % rotate; it[0] += 1
+            be.DecodeAttention(kind, W(q), W(ks_[j]), W(vs_[j]), W(o), Bn, H, S, D, sc, numKVHeads=kvh)
         ms_, _, st_ = _events_time(torch, fn, steps, warmup)
-        nbytes = 2.0 * Bn * H * S * D * q.element_size()
-        add(name, kind, "decode attention B=%d H=%d q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, S, D), ms_, _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)), st_)
+        nbytes = 2.0 * Bn * kvh * S * D * q.element_size()
+        add(name, kind, "decode attention B=%d H=%d%s q_len=1 KV=%d d=%d, contiguous KV cache" % (Bn, H, " Hkv=%d" % kvh if Hkv else "", S, D), ms_,
+            _roof_bytes(nbytes, ms_, TRAFFIC_BYTES.get(name)), st_)
 
     gemm_case("gemm_f32_1024", "f32", 1024, 1024, 1024, uniform_inputs=True)
     gemm_case("gemm_f32_proj", "f32", 4096, 3072, 768)
@@ -297,6 +308,13 @@ def main() -> int:
     attn_case("attn_bf16_prefill", "bf16", 4, 32, 2048, 128)
     decode_case("decode_bf16", "bf16", 32, 32, 4096, 128)
     gemm_case("gemm_bf16_decode_proj", "bf16", 32, 4096, 4096, hbm=True, rotate=12)
+    # shapes beside the listed configurations (run with --only NAME[,NAME...]): grouped-query decode, fp32 products with few rows,
+    # a causal fp32 attention grid of several rounds
+    decode_case("decode_bf16_gqa", "bf16", 32, 32, 4096, 128, Hkv=8, rotate=2, extra=True)
+    decode_case("decode_f32_gqa", "f32", 32, 32, 4096, 128, Hkv=8, extra=True)
+    gemm_case("gemm_f32_m16", "f32", 16, 4096, 4096, hbm=True, rotate=6, extra=True)
+    gemm_case("gemm_f32_m128", "f32", 128, 4096, 4096, extra=True)
+    attn_case("attn_f32_prefill_b32", "f32", 32, 12, 512, 64, extra=True)
     out["others"] = others
 
     if args.copy_calibration:
