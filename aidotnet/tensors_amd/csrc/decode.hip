@@ -238,24 +238,45 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
     }
 }
 
-// Merge the per-split (m, l, acc) triples: grid = B*H, one thread per head-dim element.
+// Merge the per-split (m, l, acc) triples: grid = B*H, one thread per head-dim element.  The split weights are formed once per
+// head (through LDS); the partial rows are then read eight splits at a time so that the loads of a thread overlap.
 template <typename OutT>
 __global__ __launch_bounds__(256) void decode_reduce_kernel(const DecodeArgs a, int dpad)
 {
+    __shared__ float s_w[64], s_ml[2];
     const int bh = blockIdx.x;
     const int b = bh / a.H, hd = bh - b * a.H;
-    const float* ws = a.ws + (long long)bh * a.splits * (2 + dpad);
-    float M = -INFINITY;
-    for (int s = 0; s < a.splits; s++) M = fmaxf(M, ws[(long long)s * (2 + dpad)]);
-    const float Muse = (M == -INFINITY) ? 0.0f : M;
-    for (int d = threadIdx.x; d < a.D; d += blockDim.x) {
-        float L = 0.0f, A = 0.0f;
-        for (int s = 0; s < a.splits; s++) {
-            const float* p = ws + (long long)s * (2 + dpad);
-            float w = __builtin_amdgcn_exp2f(p[0] - Muse);
-            L += p[1] * w;
-            A += p[2 + d] * w;
+    const long long stride = 2 + dpad;
+    const float* ws = a.ws + (long long)bh * a.splits * stride;
+    const int t = threadIdx.x;
+    // splits <= 64: lane s of the first wave holds split s
+    if (t < 64) {
+        const float m = t < a.splits ? ws[t * stride] : -INFINITY;
+        const float l = t < a.splits ? ws[t * stride + 1] : 0.0f;
+        float M = m;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, shfl_xor_f(M, off));
+        const float Muse = (M == -INFINITY) ? 0.0f : M;
+        const float w = __builtin_amdgcn_exp2f(m - Muse);
+        float L = l * w;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) L += shfl_xor_f(L, off);
+        s_w[t] = w;
+        if (t == 0) { s_ml[0] = M; s_ml[1] = L; }
+    }
+    __syncthreads();
+    const float M = s_ml[0], L = s_ml[1];
+    for (int d = t; d < a.D; d += blockDim.x) {
+        float A = 0.0f;
+        int s0 = 0;
+        for (; s0 + 8 <= a.splits; s0 += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = ws[(s0 + u) * stride + 2 + d];
+#pragma unroll
+            for (int u = 0; u < 8; u++) A += v[u] * s_w[s0 + u];
         }
+        for (; s0 < a.splits; s0++) A += ws[s0 * stride + 2 + d] * s_w[s0];
         typedef typename Raw3<OutT>::type out_t;
         out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1];
         float r = L > 0.0f ? A / L : 0.0f;
