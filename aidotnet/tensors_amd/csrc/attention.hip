@@ -36,6 +36,7 @@ struct AttnArgs {
     // fast kernel, grouped decode: the workgroup's key range is split `split` of nsplit (chunk keys each) and, when part is not
     // null, it stores its unnormalised partial (m, l, O[128]) at part + ((b H_q + head) nsplit + split) * 130 for the merge pass
     int nsplit, chunk; float* part;
+    int stream;    // fast kernel: K and V are read once per launch (grouped decode): non-temporal loads
     int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
@@ -78,6 +79,16 @@ __device__ __forceinline__ void attn_dma16(const void* gptr, uint32_t lds_dst)
 __device__ __forceinline__ void attn_dma16_base(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
+}
+
+// non-temporal forms for a cache that is read once per launch (decode)
+__device__ __forceinline__ void attn_dma16_stream(const void* gptr, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds_dst), "v"(gptr) : "memory");
+}
+__device__ __forceinline__ void attn_dma16_base_stream(const void* base_uniform, uint32_t lane_off, uint32_t lds_dst)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt" ::"s"(lds_dst), "v"(lane_off), "s"(base_uniform) : "memory");
 }
 
 typedef short s16x4a __attribute__((ext_vector_type(4)));
@@ -636,8 +647,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * 4096;
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)K + (long long)(tile * BC + 16 * wave_s) * k_row_bytes;
+            if (a.stream) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+                for (int i = 0; i < 4; i++) attn_dma16_base_stream(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -651,8 +667,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * 4096;
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
+            if (a.stream) {
 #pragma unroll
-            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+                for (int i = 0; i < 4; i++) attn_dma16_base_stream(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+            }
         } else {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -739,7 +760,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         // Loads of the next tile: when this wave computes and the next tile lies fully inside the sequence they are
         // issued one per MFMA inside the first phase below (a vector-memory instruction holds the wave's issue slot for
         // some tens of cycles; there it is covered by the running MFMA).  Otherwise all at once here.
-        const bool spread = j < nact && j + 1 < ntiles && (j + 1) * BC + BC <= Sk;
+        const bool spread = !a.stream && j < nact && j + 1 < ntiles && (j + 1) * BC + BC <= Sk;
         if (j + 1 < ntiles && !spread) { issue_k(j + 1); issue_v(j + 1); }
         if (j < nact) {
             const int kv0 = j * BC;
@@ -962,7 +983,7 @@ hipError_t attn_group_decode(hipStream_t stream, int kind, const AttnParams& p, 
     for (int i = 0; i < 3; i++) { a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; }
     a.vec_in = 1; a.vec_out = 1;
     a.bt = nullptr; a.bsz = 0; a.bt_bs = 0;
-    a.nsplit = nsplit; a.chunk = chunk; a.part = nsplit > 1 ? part : nullptr;
+    a.nsplit = nsplit; a.chunk = chunk; a.part = nsplit > 1 ? part : nullptr; a.stream = 1;
     a.qtiles = 1;
     const long long nblk = (long long)p.B * p.Hkv * nsplit;
     if (nblk > 0x7FFFFFFFLL || sk <= 0) return hipErrorInvalidValue;
@@ -1061,7 +1082,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     AttnArgs a;
     a.paired = 0;
     a.hgroup = 0;
-    a.nsplit = 1; a.chunk = 0; a.part = nullptr;
+    a.nsplit = 1; a.chunk = 0; a.part = nullptr; a.stream = 0;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
     a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;
