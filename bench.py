@@ -37,7 +37,7 @@ TRAFFIC_BYTES = {
     "gemm_f16_proj_f32out": int((17048 * 2.0 + 49174) * 1024),
     "gemm_f32_proj": int((43106 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12324 * 2.0 + 4096) * 1024),
-    "decode_bf16": int((1048910 * 2.0 + 1088) * 1024),
+    "decode_bf16": int((1048890 * 2.0 + 1088) * 1024),
     "attn_f16_prefill": int((117711 * 2.0 + 132324) * 1024),
     "attn_bf16_prefill": int((117516 * 2.0 + 132324) * 1024),
     "attn_f32_prefill": int((22636 * 2.0 + 12480) * 1024),
