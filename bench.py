@@ -42,6 +42,10 @@ TRAFFIC_BYTES = {
     "attn_bf16_prefill": int((117516 * 2.0 + 132324) * 1024),
     "attn_f32_prefill": int((22636 * 2.0 + 12480) * 1024),
     "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
+    # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass)
+    "decode_bf16_gqa": int(((262406 + 2641) * 2.0 + 4166 + 512) * 1024),
+    "decode_f32_gqa": int(((526428 + 2641) * 2.0 + 4352 + 512) * 1024),
+    "gemm_f32_m16": int(((33827 + 1026) * 2.0 + 2048 + 256) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
