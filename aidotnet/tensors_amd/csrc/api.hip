@@ -140,6 +140,13 @@ int attn_common(void* ctx, void* stream, int kind, const aidn_attn_desc* d, cons
         p.lse = (float*)ws;
     }
     p.allow_fast_path = c->attn_fast_path;
+    if (!(weights && !lse)) {
+        // key-range partials of a call whose query tiles alone would leave most of the chip idle; a stream under capture whose
+        // workspace would have to grow simply runs unsplit
+        const size_t need = aidn::attn_fwd_workspace_bytes(kind, p);
+        void* ws = nullptr;
+        if (need && acquire_ws(c, stream, need, &ws) == AIDN_OK) { p.workspace = ws; p.workspace_bytes = need; }
+    }
     return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "attn_fwd");
 }
 

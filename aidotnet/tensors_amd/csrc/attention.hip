@@ -573,9 +573,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         bh = logical / a.qtiles;
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
         if (a.nsplit > 1) {
-            split = logical % a.nsplit;          // one query tile per head; the splits of a head are neighbours
-            bh = logical / a.nsplit;
-            qt = 0;
+            // the key ranges of a query tile are neighbours; late (heavy, under a causal mask) query tiles first
+            const int per_head = a.qtiles * a.nsplit;
+            bh = logical / per_head;
+            const int r = logical - bh * per_head;
+            qt = a.qtiles - 1 - r / a.nsplit;
+            split = r % a.nsplit;
         } else if (a.paired) {
             // XCD-contiguous heads, qtiles / 2 workgroups per head: first the late (heavy) tile of the pair, then the early one
             const int units = a.qtiles >> 1;
@@ -610,11 +613,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
     // keys this workgroup sees: all of them, or its split's range (which may be empty)
     int Sk = a.Sk;
+    long long qoff = a.qoff;                 // causal: query i sees keys j <= i + qoff (j counted from the first key of the range)
     if (a.nsplit > 1) {
         const int kbeg = split * a.chunk;
         K += (long long)kbeg * a.ks[2];
         V += (long long)kbeg * a.vs[2];
         Sk = max(0, min(a.chunk, a.Sk - kbeg));
+        qoff -= kbeg;
     }
 
     u32x4 qf[DSTEPS];
@@ -626,7 +631,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 
     int ntiles = (Sk + BC - 1) / BC;
     if (a.causal) {
-        long long lastkey = (long long)q0 + BR - 1 + a.qoff;
+        long long lastkey = (long long)q0 + BR - 1 + qoff;
         if (lastkey < 0) ntiles = 0;
         else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
     }
@@ -697,7 +702,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     // tiles this wave computes: under a causal mask a prefix of the workgroup's tiles
     int nact = wq_min < a.Sq ? ntiles : 0;      // a wave without query rows only takes part in the loads
     if (a.causal) {
-        long long lk = (long long)wq_max + a.qoff;
+        long long lk = (long long)wq_max + qoff;
         if (lk < 0) nact = 0;
         else { long long nt = lk / BC + 1; if (nt < nact) nact = (int)nt; }
     }
@@ -714,7 +719,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     // lane's accumulator row offset 4 h so that the per-element test is against a constant
     auto key_limit = [&](int q) -> int {
         long long lim = Sk - 1;
-        if (a.causal) { long long c = (long long)q + a.qoff; if (c < lim) lim = c; }
+        if (a.causal) { long long c = (long long)q + qoff; if (c < lim) lim = c; }
         return (int)(lim < -1 ? -1 : lim);
     };
     const int klim = key_limit(qi) - 4 * h;
@@ -935,6 +940,50 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     }   // pass
 }
 
+// Merge of the key-range partials of the fast kernel (head dimension 128): one workgroup per query row; the weights of the
+// ranges are formed once (first wave), the partial rows are read with their loads overlapped.  part: [row][nsplit][130].
+template <typename OutT>
+__global__ __launch_bounds__(128) void attn_split_merge_kernel(const AttnArgs a)
+{
+    __shared__ float s_w[64], s_ml[2];
+    const long long row = blockIdx.x;                  // (b * H + hd) * Sq + qi
+    const int bh = (int)(row / a.Sq), qi = (int)(row - (long long)bh * a.Sq);
+    const int b = bh / a.H, hd = bh - b * a.H;
+    const float* __restrict__ P = a.part + row * a.nsplit * 130;
+    const int t = threadIdx.x;
+    if (t < 64) {
+        const float m = t < a.nsplit ? P[t * 130] : -INFINITY;
+        const float l = t < a.nsplit ? P[t * 130 + 1] : 0.0f;
+        float M = m;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) M = fmaxf(M, shfl_xor_f(M, off));
+        const float w = __builtin_amdgcn_exp2f(m - ((M == -INFINITY) ? 0.0f : M));
+        float L = l * w;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) L += shfl_xor_f(L, off);
+        s_w[t] = w;
+        if (t == 0) { s_ml[0] = M; s_ml[1] = L; }
+    }
+    __syncthreads();
+    const float M = s_ml[0], L = s_ml[1];
+    float A = 0.0f;
+    int s0 = 0;
+    for (; s0 + 8 <= a.nsplit; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) v[u] = P[(s0 + u) * 130 + 2 + t];
+#pragma unroll
+        for (int u = 0; u < 8; u++) A += v[u] * s_w[s0 + u];
+    }
+    for (; s0 < a.nsplit; s0++) A += P[s0 * 130 + 2 + t] * s_w[s0];
+    typedef typename Raw2<OutT>::type out_t;
+    out_t* O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
+    const float r = L > 0.0f ? A / L : 0.0f;
+    if constexpr (Elem<OutT>::BYTES == 4) O[t] = as_u32(r);
+    else O[t] = (out_t)Elem<OutT>::narrow(r);
+    if (t == 0 && a.lse) a.lse[row] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * LN2 : -INFINITY;
+}
+
 template <typename T, typename OutT>
 static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
 {
@@ -943,6 +992,17 @@ static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
+    if (a.nsplit > 1) {
+        // few query tiles over a long key sequence: every tile's keys are cut into ranges that run side by side; a merge pass follows
+        a.paired = 0;
+        const long long nblk = (long long)a.qtiles * a.B * a.H * a.nsplit;
+        const long long rows = (long long)a.B * a.H * a.Sq;
+        if (nblk > 0x7FFFFFFFLL || rows > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+        hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
+        if (hipError_t e = hipGetLastError()) return e;
+        hipLaunchKernelGGL((attn_split_merge_kernel<OutT>), dim3((unsigned)rows), dim3(128), 0, stream, a);
+        return hipGetLastError();
+    }
     // causal self-attention with an even number of query tiles: pair tile i with tile qtiles-1-i, so every workgroup has the same work
     a.paired = (a.causal && a.qoff == 0 && a.Sq == a.Sk && a.qtiles >= 2 && a.qtiles % 2 == 0) ? 1 : 0;
     long long nblk = (long long)(a.paired ? a.qtiles / 2 : a.qtiles) * a.B * a.H;
@@ -1075,6 +1135,53 @@ static hipError_t dispatch_attn_d(const AttnArgs& a, bool full, hipStream_t stre
 }
 
 
+static bool attn_aligned16(const void* ptr, const long long* s, int bytes)
+{
+    return ((uintptr_t)ptr & 15u) == 0 && (s[0] * bytes) % 16 == 0 && (s[1] * bytes) % 16 == 0 && (s[2] * bytes) % 16 == 0;
+}
+
+// the fast kernel: 16-bit, head dimension 128, aligned contiguous rows, plain (optionally causal) attention
+static bool attn_dl_applies(int kind, const AttnParams& p)
+{
+    if (kind == 0 || p.D != 128 || !(p.scale > 0.0f) || p.block_table || !p.allow_fast_path) return false;
+    if (p.bias != nullptr || (p.mask && p.mask_mode != 0) || p.softcap > 0.0f) return false;
+    if (!(attn_aligned16(p.q, p.qs, 2) && attn_aligned16(p.k, p.ks, 2) && attn_aligned16(p.v, p.vs, 2))) return false;
+    // the kernel addresses the K/V rows of a 4-key load group with unsigned 32-bit byte offsets
+    return p.ks[2] > 0 && p.ks[2] < (1LL << 28) && p.vs[2] > 0 && p.vs[2] < (1LL << 28);
+}
+
+// Key ranges per query tile for the fast kernel (1 = none): when the query tiles alone leave most CUs idle and the key
+// sequence is long (chunked prefill against a long cache, a few speculative tokens), ranges of at least 512 keys up to about two
+// workgroups per CU.  *chunk = keys per range (a multiple of 64).
+static int attn_dl_splits(const AttnParams& p, int* chunk)
+{
+    const long long base = (long long)((p.Sq + 127) / 128) * p.B * p.H;
+    int sk = p.Sk;
+    if (p.causal) {                              // keys nobody sees do not count
+        const long long lim = (long long)p.Sq + p.qoff;
+        if (lim < sk) sk = (int)(lim < 0 ? 0 : lim);
+    }
+    *chunk = 0;
+    if (base >= 256 || sk < 1024 || p.weights) return 1;
+    int ns = (int)((512 + base - 1) / base);
+    if (ns > sk / 512) ns = sk / 512;
+    if (ns > 32) ns = 32;
+    if (ns < 2) return 1;
+    int c = (sk + ns - 1) / ns;
+    c = (c + 63) / 64 * 64;
+    ns = (sk + c - 1) / c;
+    *chunk = c;
+    return ns >= 2 ? ns : 1;
+}
+
+size_t attn_fwd_workspace_bytes(int kind, const AttnParams& p)
+{
+    if (!attn_dl_applies(kind, p)) return 0;
+    int chunk;
+    const int ns = attn_dl_splits(p, &chunk);
+    return ns > 1 ? (size_t)p.B * p.H * p.Sq * ns * 130 * sizeof(float) : 0;
+}
+
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
 {
@@ -1104,6 +1211,13 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     // the fast kernel addresses K/V rows of a 4-key load group with unsigned 32-bit byte offsets
     const bool rows32 = p.ks[2] > 0 && p.ks[2] < (1LL << 28) && p.vs[2] > 0 && p.vs[2] < (1LL << 28);
     const bool dl = kind != 0 && !full && a.vec_in && p.D == 128 && p.scale > 0.0f && rows32 && !p.block_table && g_attn_allow_dl;
+    if (dl && p.workspace && attn_dl_applies(kind, p)) {
+        int chunk;
+        const int ns = attn_dl_splits(p, &chunk);
+        if (ns > 1 && p.workspace_bytes >= (size_t)p.B * p.H * p.Sq * ns * 130 * sizeof(float)) {
+            a.nsplit = ns; a.chunk = chunk; a.part = (float*)p.workspace;
+        }
+    }
     if (dl) {
         if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
         else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);

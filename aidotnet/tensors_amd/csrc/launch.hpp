@@ -46,6 +46,10 @@ struct AttnParams {
     long long block_table_stride = 0;
     // 0: every shape takes the general kernel (the direct-to-LDS instances are not used); set per call from the context
     int allow_fast_path = 1;
+    // optional scratch of attn_fwd_workspace_bytes() bytes: lets attn_fwd cut the key sequence into ranges when the query tiles
+    // alone would leave most of the chip idle
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
 };
 
 // Raises a kernel's dynamic shared-memory limit once per device (the attribute belongs to the device's copy of the function).
@@ -54,6 +58,7 @@ hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long
 
 // kind: 0 fp32, 1 fp16, 2 bf16
 hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p);
+size_t attn_fwd_workspace_bytes(int kind, const AttnParams& p);
 
 // Decode (Sq == 1).  eff_splits: the split count actually used for `splits` requested (<= 0 = auto).
 int attn_decode_splits(int kind, const AttnParams& p, int splits);

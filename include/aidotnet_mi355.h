@@ -168,7 +168,9 @@ AIDN_API int aidn_mi355_convert_bf16_to_f32(void* ctx, void* stream, const uint1
  * (out_is_16bit != 0).  Any 1 <= D <= 256 is accepted (GpuKernelGuards.MaxHeadDim,
  * Engines/DirectGpu/GpuKernelGuards.cs:12; larger: AIDN_ERR_UNSUPPORTED); rows whose start and strides
  * are multiples of 16 bytes take the vector loads, head dimensions 64 and 128 with such rows the
- * direct-to-LDS kernels.
+ * direct-to-LDS kernels.  A 16-bit call at head dimension 128 with few query rows against many keys (chunked prefill, a few
+ * speculative tokens) runs the key ranges of a query tile side by side and merges them; the partials live in the stream's
+ * workspace (a stream under capture whose workspace would have to grow runs the call unsplit).
  */
 typedef struct aidn_attn_desc {
     int32_t B, H, Hkv, Sq, Sk, D;

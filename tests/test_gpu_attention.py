@@ -308,6 +308,12 @@ FAST_CASES = [
     (2, 2, 2, 64, 1000, False, 0),
     (1, 2, 2, 1, 4097, True, 4096),       # decode shape through the prefill kernel
     (1, 1, 1, 300, 300, True, 0),
+    # few query tiles over a long key sequence: the keys of every tile are cut into ranges that run side by side (merge pass)
+    (1, 4, 2, 16, 2100, True, 2084),      # a few new tokens against a long cache, GQA
+    (1, 2, 2, 300, 1100, True, 800),      # chunked prefill, three query tiles, ragged ranges
+    (2, 2, 2, 200, 3000, False, 0),
+    (1, 2, 2, 1024, 1024, True, 0),       # causal self-attention: late ranges are empty for early query tiles
+    (1, 3, 3, 130, 1500, True, 100),      # small offset: most ranges are empty for every row
 ]
 
 
@@ -345,19 +351,21 @@ def test_fast_path_d128_matches_oracle_and_general_kernel(be, kind, B, H, Hkv, S
 def test_fast_path_all_masked_rows_and_large_logits(be):
     # rows above the diagonal with a negative offset see no key: O = 0, LSE = -inf (CpuEngine.cs:29243-29249);
     # logits of magnitude ~60 exercise the lazily raised exponent reference
-    B, H, S, D = 1, 2, 200, 128
-    rng = np.random.default_rng(77)
-    q, k, v = 3 * _rand(rng, B, H, S, D), 3 * _rand(rng, B, H, S, D), _rand(rng, B, H, S, D)
-    (qb, qw), (kb, kw), (vb, vw) = round_to(q, "bf16"), round_to(k, "bf16"), round_to(v, "bf16")
-    o64, lse64 = oracle.attention_f64(qw, kw, vw, 0.5, True, -3)
-    dt = torch.bfloat16
-    out = torch.full((B, H, S, D), float("nan"), device="cuda"); lse = torch.full((B, H, S), float("nan"), device="cuda")
-    be.FlashAttentionHalf("bf16", be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)),
-                          be.WrapTensor(out), be.WrapTensor(lse), B, H, S, S, D, 0.5, True, -3)
-    o = out.cpu().numpy(); l = lse.cpu().numpy()
-    assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
-    assert mixed_err(o, o64) <= HALF_TOL
-    assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
+    # (the second size runs with its keys cut into ranges: rows without keys must stay O = 0, LSE = -inf through the merge)
+    for S in (200, 1100):
+        B, H, D = 1, 2, 128
+        rng = np.random.default_rng(77)
+        q, k, v = 3 * _rand(rng, B, H, S, D), 3 * _rand(rng, B, H, S, D), _rand(rng, B, H, S, D)
+        (qb, qw), (kb, kw), (vb, vw) = round_to(q, "bf16"), round_to(k, "bf16"), round_to(v, "bf16")
+        o64, lse64 = oracle.attention_f64(qw, kw, vw, 0.5, True, -3)
+        dt = torch.bfloat16
+        out = torch.full((B, H, S, D), float("nan"), device="cuda"); lse = torch.full((B, H, S), float("nan"), device="cuda")
+        be.FlashAttentionHalf("bf16", be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)),
+                              be.WrapTensor(out), be.WrapTensor(lse), B, H, S, S, D, 0.5, True, -3)
+        o = out.cpu().numpy(); l = lse.cpu().numpy()
+        assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
+        assert mixed_err(o, o64) <= HALF_TOL
+        assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
 
 
 # --------------------------------------------------------------- fp32 head-dim-64 direct-to-LDS form of the general kernel
