@@ -193,7 +193,8 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
     size_t need = c->force_tile == 0 ? aidn::gemm_16_workspace_bytes(M, N, K) : 0;
     if (need) {
         int st = acquire_ws(c, stream, need, &ws);
-        if (st) return st;
+        if (st == AIDN_ERR_WORKSPACE) ws = nullptr;      // under capture and not reserved: the tiled kernel needs no workspace
+        else if (st) return st;
     }
     if (!valid_activation(act)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: unknown activation");
     return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, bias, act, act_param), "gemm_16");
@@ -425,7 +426,10 @@ static int smallm_ws(Ctx* c, void* stream, int M, int N, int K, int transB, void
     if (c->force_tile != 0) return 0;
     size_t need = transB == 2 ? aidn::gemm_smallm_workspace_bytes(M, N, K) : aidn::gemm_f32_workspace_bytes(M, N, K, transB);
     if (!need) return 0;
-    return acquire_ws(c, stream, need, ws);
+    const int st = acquire_ws(c, stream, need, ws);
+    // a stream under capture whose workspace would have to grow: the tiled kernel needs none
+    if (st == AIDN_ERR_WORKSPACE) { *ws = nullptr; return 0; }
+    return st;
 }
 
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,

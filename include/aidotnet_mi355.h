@@ -58,7 +58,8 @@ AIDN_API const char* aidn_mi355_version(void);
 /* hipStreamSynchronize(stream): replaces HipBackend.Synchronize (HipBackend.cs:1444-1446). */
 AIDN_API int aidn_mi355_sync(void* ctx, void* stream);
 /* Makes the workspace of `stream` at least `bytes` large now, so that later calls on it allocate nothing -- required before
- * the calls are captured into a HIP graph (no allocation can happen during capture: such a call returns AIDN_ERR_WORKSPACE);
+ * the calls are captured into a HIP graph (no allocation can happen during capture: a decode or fused-MHA call, which cannot
+ * run without its workspace, then returns AIDN_ERR_WORKSPACE; a GEMM or prefill-attention call takes its kernel that needs none);
  * one eager run of the same call sequence has the same effect.  aidn_mi355_workspace_bytes reads the current size (after a
  * warm-up run: the amount to reserve on another stream or context).  No counterpart in the reference, whose backend allocates
  * per call from its buffer pool (HipBackend.cs:12214-12270). */

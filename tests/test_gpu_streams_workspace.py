@@ -110,6 +110,35 @@ def test_graph_replay_survives_workspace_growth_and_capture_refuses_growth(be):
                 step()
 
 
+def test_gemm_under_capture_without_reserved_workspace_takes_the_tiled_kernel(be):
+    # a few-row fp32 product and a skinny bf16 product would use split-K partials; on a stream that is being captured and has no
+    # workspace yet they run their workspace-free kernels instead of failing, and the replay matches an eager run within tolerance
+    W = be.WrapTensor
+    torch.manual_seed(9)
+    M, N, K = 128, 1024, 4096
+    a = torch.randn(M, K, device="cuda"); b = 0.02 * torch.randn(K, N, device="cuda"); c = torch.zeros(M, N, device="cuda")
+    a16 = torch.randn(16, K, device="cuda").bfloat16(); b16 = (0.02 * torch.randn(K, N, device="cuda")).bfloat16()
+    c16 = torch.zeros(16, N, device="cuda", dtype=torch.bfloat16)
+    ref = (a.double() @ b.double()); ref16 = a16.double() @ b16.double()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        assert be.WorkspaceBytes() == 0
+        with torch.cuda.graph(graph, stream=side):
+            be.Gemm(W(a), W(b), W(c), M, N, K)
+            be.Bf16Gemm(W(a16), W(b16), W(c16), 16, N, K)
+        assert be.WorkspaceBytes() == 0
+    for _ in range(2):
+        c.zero_(); c16.zero_(); torch.cuda.synchronize()
+        graph.replay(); torch.cuda.synchronize()
+        assert float((c.double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+        assert float((c16.double() - ref16).abs().max()) <= 2e-2 * float(ref16.abs().max())
+    # eager, the same calls take the split paths (the workspace appears) and agree
+    be.Gemm(W(a), W(b), W(c), M, N, K); torch.cuda.synchronize()
+    assert be.WorkspaceBytes() > 0
+    assert float((c.double() - ref).abs().max()) <= 1e-4 * float(ref.abs().max())
+
+
 def test_decode_refuses_softcap_and_masks(be):
     from aidotnet.tensors_amd._lib import AttnDesc
     t = torch.zeros(4 * 64, device="cuda")
