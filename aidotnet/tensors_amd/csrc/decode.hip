@@ -8,7 +8,7 @@
 // reference decode test's oracle (tests/AiDotNet.Tensors.Tests/Engines/DirectGpu/
 // FlashDecodeHipTests.cs:43-69), i.e. softmax(scale * q.K^T) V over all cached keys.
 //
-// grid = (splits, B*H), 256 threads.  Wave w of the workgroup walks its split in blocks of
+// grid = (B*H / heads per workgroup) * splits, 256 threads.  Wave w of the workgroup walks its split in blocks of
 // U * KPW keys (KPW = 64 / LPK keys per load, U loads in flight for K and U for V).  Every lane
 // keeps an online-softmax state (m, l, acc[E]) for its key slot and its 16-byte slice of the head
 // dim; slots and waves are merged through LDS, splits through a workspace and a second kernel.
@@ -106,11 +106,11 @@ __global__ __launch_bounds__(256) void decode_partial_kernel(const DecodeArgs a)
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int dl = lane % LPK, sk = lane / LPK;
-    const int split = blockIdx.x;
-    // blockIdx.y = (batch, K/V head, chunk of GH query heads of that K/V head)
+    // one grid dimension (y and z are limited to 65535): the splits of a (batch, K/V head, chunk of GH query heads) are neighbours
+    const int split = blockIdx.x % a.splits;
     const int gq = a.H / a.Hkv;                    // query heads per K/V head (a multiple of GH)
     const int chunks = gq / GH;
-    const int by = blockIdx.y;
+    const int by = blockIdx.x / a.splits;
     const int b = by / (a.Hkv * chunks);
     const int kvh = (by - b * a.Hkv * chunks) / chunks;
     const int hd0 = kvh * gq + (by % chunks) * GH;  // first query head
@@ -341,7 +341,9 @@ static hipError_t launch_decode(DecodeArgs a, hipStream_t stream)
     // query heads of a K/V head that share a workgroup (and its loads): 4, 2 or 1, whichever divides the group
     const int gq = a.H / a.Hkv;
     const int gh = gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1;
-    dim3 grid((unsigned)a.splits, (unsigned)(a.B * a.H / gh));
+    const long long nwg = (long long)a.B * a.H / gh * a.splits;
+    if (nwg > 0x7FFFFFFFLL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)nwg);
     if (gh == 4) hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 4>), grid, dim3(256), 0, stream, a);
     else if (gh == 2) hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 2>), grid, dim3(256), 0, stream, a);
     else hipLaunchKernelGGL((decode_partial_kernel<T, OutT, LPK, U, 1>), grid, dim3(256), 0, stream, a);
