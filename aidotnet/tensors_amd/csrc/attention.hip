@@ -37,6 +37,7 @@ struct AttnArgs {
     // null, it stores its unnormalised partial (m, l, O[128]) at part + ((b H_q + head) nsplit + split) * 130 for the merge pass
     int nsplit, chunk; float* part;
     int stream;    // fast kernel: K and V are read once per launch (grouped decode): non-temporal loads
+    int stage_out; // fast kernel: fp32 O goes through LDS and is written as whole rows
     int paired;    // fast kernel, causal: a workgroup runs query tile qtiles-1-i and then tile i of a head (equal work for every workgroup)
     int vec_in;    // q/k/v rows are 16-byte aligned and D is a multiple of the 16-byte element count
     int vec_out;
@@ -913,6 +914,32 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
                 }
         }
     } else
+    if (Elem<OutT>::BYTES == 4 && a.vec_out && a.stage_out) {
+        // fp32 O through LDS: the lane holds 16-byte pieces of ONE row (64 rows per store instruction, each a partial line);
+        // staged per wave as [32 rows][512 B] (chunk c of row r at position c ^ r, conflict-free both ways) and written back
+        // as whole 512-byte rows, two per instruction.  The tile memory is idle here: every wave left the last tile at the
+        // barrier that ends the loop; the barrier below keeps the next pass's loads off the staged rows.
+        unsigned char* stg = smem + wave * 16384;
+#pragma unroll
+        for (int i = 0; i < DT; i++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int c = 8 * i + 2 * g + h;
+                *(f32x4*)(stg + l32 * 512 + ((c ^ l32) << 4)) =
+                    f32x4{oacc[i][4 * g + 0] * inv, oacc[i][4 * g + 1] * inv, oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv};
+            }
+        if (a.lse && h == 0 && qi < a.Sq)
+            a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+        const int c = lane & 31;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const int r = 2 * q + (lane >> 5);
+            const int row = q0 + wave * 32 + r;
+            const f32x4 v = *(const f32x4*)(stg + r * 512 + ((c ^ r) << 4));
+            if (row < a.Sq) *(f32x4*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)row * a.os[2] + c * 4) = v;
+        }
+        if (npass > 1) __syncthreads();
+    } else
     if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
         out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
@@ -992,6 +1019,7 @@ static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
+    a.stage_out = 1;
     if (a.nsplit > 1) {
         // few query tiles over a long key sequence: every tile's keys are cut into ranges that run side by side; a merge pass follows
         a.paired = 0;
@@ -1043,7 +1071,7 @@ hipError_t attn_group_decode(hipStream_t stream, int kind, const AttnParams& p, 
     for (int i = 0; i < 3; i++) { a.ks[i] = p.ks[i]; a.vs[i] = p.vs[i]; }
     a.vec_in = 1; a.vec_out = 1;
     a.bt = nullptr; a.bsz = 0; a.bt_bs = 0;
-    a.nsplit = nsplit; a.chunk = chunk; a.part = nsplit > 1 ? part : nullptr; a.stream = 1;
+    a.nsplit = nsplit; a.chunk = chunk; a.part = nsplit > 1 ? part : nullptr; a.stream = 1; a.stage_out = 0;
     a.qtiles = 1;
     const long long nblk = (long long)p.B * p.Hkv * nsplit;
     if (nblk > 0x7FFFFFFFLL || sk <= 0) return hipErrorInvalidValue;
@@ -1189,7 +1217,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     AttnArgs a;
     a.paired = 0;
     a.hgroup = 0;
-    a.nsplit = 1; a.chunk = 0; a.part = nullptr; a.stream = 0;
+    a.nsplit = 1; a.chunk = 0; a.part = nullptr; a.stream = 0; a.stage_out = 0;
     a.q = p.q; a.k = p.k; a.v = p.v; a.o = p.o; a.lse = p.lse; a.bias = p.bias; a.mask = p.mask;
     a.B = p.B; a.H = p.H; a.Hkv = p.Hkv; a.Sq = p.Sq; a.Sk = p.Sk; a.D = p.D;
     a.scale = p.scale; a.causal = p.causal; a.qoff = p.qoff; a.softcap = p.softcap; a.mask_mode = p.mask ? p.mask_mode : 0;

@@ -881,7 +881,9 @@ template <> struct Mma16<bf16_t> {
 // has four 32 KB stages and is filled three K-tiles ahead (loads complete in issue order: "tile kt+1 has landed" is a count of
 // younger loads).
 #define DL16_HALF_STAGES 4
-template <typename T, typename OutT, int TJ = 4, bool HALF = false>
+// NTS: C is written with non-temporal stores (a compile-time switch: as a run-time branch the two stores are merged by the compiler
+// and the hint is lost).
+template <typename T, typename OutT, int TJ = 4, bool HALF = false, bool NTS = false>
 __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 {
     static_assert(!HALF || TJ == 2, "the 128-row tile is built for 128 columns");
@@ -1139,7 +1141,9 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 const int u = q * 64 + lane;
                 const int row = u / CPR, c = u % CPR;
                 const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
-                *(u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16) = v;
+                u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
+                if constexpr (NTS) __builtin_nontemporal_store(v, dst);
+                else *dst = v;
             }
         }
     }
@@ -1148,13 +1152,29 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 template <typename T, typename OutT, int TJ = 4, bool HALF = false>
 static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 {
-    auto kern = gemm_dl16_kernel<T, OutT, TJ, HALF>;
     constexpr int smem = HALF ? DL16_HALF_STAGES * (128 * 128 + 64 * 256) : 2 * (256 * 128 + 128 * 256);
-    static unsigned long long attr_done = 0;
-    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     g.tiles_m = g.M / (HALF ? 128 : 256);
     g.tiles_n = g.N / (64 * TJ);
-    hipLaunchKernelGGL(kern, dim3((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch), dim3(512), smem, stream, g);
+    const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch);
+    // Non-temporal stores of C when A, B and C together exceed the 256 MB last-level cache: C then no longer displaces the operand
+    // tiles that later workgroups re-read (alternated in one process: fp16 8192^3 1336 -> 1408 TFLOP/s, bf16 1397 -> 1464,
+    // 16384 x 8192 x 1024 989 -> 1166, 8192 x 50304 x 768 764 -> 873); a problem that fits the cache is better left to its
+    // write-back path (4096 x 3072 x 768 881 -> 770, 8192 x 8192 x 2048 1283 -> 1248 with such stores).
+    const long long footprint = ((long long)g.M * g.K + (long long)g.K * g.N) * 2 * batch + (long long)g.M * g.N * batch * Elem<OutT>::BYTES;
+    const bool nts = footprint > (240LL << 20);
+    if constexpr (!HALF) {
+        if (nts) {
+            auto kern = gemm_dl16_kernel<T, OutT, TJ, false, true>;
+            static unsigned long long attr_done_nt = 0;
+            if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done_nt)) return e;
+            hipLaunchKernelGGL(kern, grid, dim3(512), smem, stream, g);
+            return hipGetLastError();
+        }
+    }
+    auto kern = gemm_dl16_kernel<T, OutT, TJ, HALF, false>;
+    static unsigned long long attr_done = 0;
+    if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
+    hipLaunchKernelGGL(kern, grid, dim3(512), smem, stream, g);
     return hipGetLastError();
 }
 
