@@ -31,16 +31,16 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # measured yet.
 TRAFFIC_BYTES = {
     # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes)
-    "gemm_f16_8192": int((809920 * 2.0 + 131072) * 1024),
-    "gemm_bf16_8192": int((825144 * 2.0 + 131072) * 1024),
-    "gemm_f16_proj": int((17105 * 2.0 + 24588) * 1024),
-    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49174) * 1024),
-    "gemm_f32_proj": int((43106 * 2.0 + 49152) * 1024),
-    "gemm_f32_1024": int((12324 * 2.0 + 4096) * 1024),
+    "gemm_f16_8192": int((787044 * 2.0 + 131352) * 1024),
+    "gemm_bf16_8192": int((786877 * 2.0 + 131584) * 1024),
+    "gemm_f16_proj": int((17124 * 2.0 + 24579) * 1024),
+    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49178) * 1024),
+    "gemm_f32_proj": int((43100 * 2.0 + 49152) * 1024),
+    "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
     "decode_bf16": int((1048890 * 2.0 + 1088) * 1024),
-    "attn_f16_prefill": int((117711 * 2.0 + 132324) * 1024),
-    "attn_bf16_prefill": int((117516 * 2.0 + 132324) * 1024),
-    "attn_f32_prefill": int((22636 * 2.0 + 12480) * 1024),
+    "attn_f16_prefill": int((148105 * 2.0 + 132096) * 1024),
+    "attn_bf16_prefill": int((148963 * 2.0 + 132096) * 1024),
+    "attn_f32_prefill": int((22648 * 2.0 + 12480) * 1024),
     "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
     # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass)
     "decode_bf16_gqa": int(((262406 + 2641) * 2.0 + 4166 + 512) * 1024),
