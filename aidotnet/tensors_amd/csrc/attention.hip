@@ -497,6 +497,34 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     // ---- normalise and store: lane holds query qi, head-dim elements i*32 + 8 g + 4 h + (0..3)
     const float l_tot = l_run + shfl_xor_f(l_run, 32);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    if constexpr (DMA && Elem<OutT>::BYTES == 4 && DP <= 128) {
+        if (a.vec_out && a.D == DP) {
+            // fp32 O through the (idle) tile memory, as in the fast kernel: staged per wave as [32 rows][DP * 4 bytes] (chunk c of row
+            // r at position c ^ r) and written back as whole rows with non-temporal stores; a lane otherwise writes 16-byte pieces
+            // of one row, 64 partial lines per instruction.  Every wave left the last tile at the barrier that ends the loop.
+            constexpr int CH = DP / 4;                   // 16-byte chunks of a row
+            constexpr int RPI = 64 / CH;                 // rows per store instruction
+            unsigned char* stg = smem + wave * (32 * DP * 4);
+#pragma unroll
+            for (int i = 0; i < DT; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    *(f32x4*)(stg + l32 * (DP * 4) + (((8 * i + 2 * g + h) ^ (l32 & (CH - 1))) << 4)) =
+                        f32x4{oacc[i][4 * g + 0] * inv, oacc[i][4 * g + 1] * inv, oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv};
+            if (a.lse && h == 0 && qi < a.Sq)
+                a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_run + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
+            const int c = lane % CH;
+#pragma unroll
+            for (int q = 0; q < 32 / RPI; q++) {
+                const int r = RPI * q + lane / CH;
+                const int row = q0 + wave * 32 + r;
+                const f32x4 v = *(const f32x4*)(stg + r * (DP * 4) + ((c ^ (r & (CH - 1))) << 4));
+                f32x4* dst = (f32x4*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)row * a.os[2] + c * 4);
+                if (row < a.Sq) __builtin_nontemporal_store(v, dst);
+            }
+            return;
+        }
+    }
     if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
         out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
