@@ -38,9 +38,9 @@ TRAFFIC_BYTES = {
     "gemm_f32_proj": int((43100 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
     "decode_bf16": int((1048890 * 2.0 + 1088) * 1024),
-    "attn_f16_prefill": int((148105 * 2.0 + 132096) * 1024),
-    "attn_bf16_prefill": int((148963 * 2.0 + 132096) * 1024),
-    "attn_f32_prefill": int((22648 * 2.0 + 12480) * 1024),
+    "attn_f16_prefill": int((139311 * 2.0 + 132113) * 1024),
+    "attn_bf16_prefill": int((139768 * 2.0 + 132113) * 1024),
+    "attn_f32_prefill": int((22644 * 2.0 + 12480) * 1024),
     "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
     # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass)
     "decode_bf16_gqa": int(((262406 + 2641) * 2.0 + 4166 + 512) * 1024),
