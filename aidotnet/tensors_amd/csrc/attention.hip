@@ -135,8 +135,9 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
 template <typename T, typename OutT, int DP, int BC, bool FULL, int MINB, bool DMA = false>
 __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 {
-    static_assert(!DMA || (!FULL && ((DP == 64 && BC == 64) || (Elem<T>::BYTES == 4 && DP == 128 && BC == 32))),
-                  "DMA form: head dimension 64 with 64-key tiles (or fp32 128 with 32-key tiles), plain / causal");
+    static_assert(!DMA || (!FULL && ((DP == 64 && BC == 64) || (Elem<T>::BYTES == 4 && DP == 128 && BC == 32) ||
+                                     (Elem<T>::BYTES == 2 && DP == 256 && BC == 32))),
+                  "DMA form: head dimension 64 with 64-key tiles (or fp32 128 / 16-bit 256 with 32-key tiles), plain / causal");
     typedef typename Raw2<T>::type raw_t;
     constexpr int E = Elem<T>::PER16, EB = Elem<T>::BYTES;
     constexpr int NT = 256, BR = 128;
@@ -316,10 +317,12 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     // swizzles of the DMA form (chunk position of 16-byte chunk c of key row `key`):
-    //   fp32 (256-byte rows):   K  c ^ (key & 15);         V  c ^ (((key >> 2) & 1) << 3)   (32-bit reads, lane halves 4 keys apart)
-    //   16-bit (128-byte rows): K  c ^ ((key >> 1) & 7);   V  c ^ (((key >> 1) & 1) << 2)   (transposing reads of 4 consecutive keys)
-    auto k_swz = [](int key) -> int { return EB == 4 ? (key & 15) : ((key >> 1) & 7); };
-    auto v_swz = [](int key) -> int { return EB == 4 ? (((key >> 2) & 1) << 3) : (((key >> 1) & 1) << 2); };
+    //   fp32 (256- / 512-byte rows): K  c ^ (key & 15);         V  c ^ (((key >> 2) & 1) << 3)   (32-bit reads, lane halves 4 keys apart)
+    //   16-bit, 128-byte rows:       K  c ^ ((key >> 1) & 7);   V  c ^ (((key >> 1) & 1) << 2)   (transposing reads of 4 consecutive keys)
+    //   16-bit, 512-byte rows:       K  c ^ (key & 15);         V  c ^ ((key & 3) << 2)
+    constexpr bool WIDE16 = EB == 2 && DP * EB > 128;
+    auto k_swz = [](int key) -> int { return (EB == 4 || WIDE16) ? (key & 15) : ((key >> 1) & 7); };
+    auto v_swz = [](int key) -> int { return EB == 4 ? (((key >> 2) & 1) << 3) : WIDE16 ? ((key & 3) << 2) : (((key >> 1) & 1) << 2); };
     auto issue_tile = [&](int tile, int stage) {
         constexpr int ROWB = DP * EB;                      // 256 / 128 bytes per key row
         constexpr int KPL = 1024 / ROWB;                   // keys per 1 KiB wave-load
@@ -476,7 +479,7 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
                             for (int q = 0; q < 2; q++) {
                                 const int row = kt * 32 + 16 * ps + 8 * q + 4 * h + (jl >> 2);
                                 u32x2 w = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                                    (__attribute__((address_space(3))) s16x4a*)(Vs + stage * VBYTES + row * 128 + ((chunk ^ v_swz(row)) << 4) + (jl & 1) * 8)));
+                                    (__attribute__((address_space(3))) s16x4a*)(Vs + stage * VBYTES + row * (DP * 2) + ((chunk ^ v_swz(row)) << 4) + (jl & 1) * 8)));
                                 vf[2 * q] = w[0];
                                 vf[2 * q + 1] = w[1];
                             }
@@ -1288,6 +1291,11 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
         else if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
                                   : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
         else err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    }
+    else if (p.D == 256 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) {
+        // head dimension 256, plain / causal, aligned contiguous K/V: the direct-to-LDS form on 32-key tiles (Q streamed)
+        if (kind == 1) err = p.out16 ? launch_attn<f16_t, f16_t, 256, 32, false, 2, true>(a, stream) : launch_attn<f16_t, float, 256, 32, false, 2, true>(a, stream);
+        else err = p.out16 ? launch_attn<bf16_t, bf16_t, 256, 32, false, 2, true>(a, stream) : launch_attn<bf16_t, float, 256, 32, false, 2, true>(a, stream);
     }
     else if (p.D == 64 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) {
         // head dimension 64, plain / causal, aligned contiguous K/V: the direct-to-LDS form of the general kernel
