@@ -177,6 +177,39 @@ def test_strided_qkv_from_packed_projection(be):
     assert mixed_err(lse.cpu().numpy(), lse_w) <= FP32_TOL
 
 
+@pytest.mark.parametrize("kind,D", [("bf16", 128), ("f16", 128), ("f32", 64), ("bf16", 64)])
+def test_output_layouts_of_the_direct_to_lds_kernels(be, kind, D):
+    # The kernels that stage O through LDS write whole rows; the same call with O laid out [B,S,H,D] (row stride H*D), with a
+    # dense O, and with an O that starts 4 bytes off a 16-byte boundary (element-wise stores) must give the same numbers.
+    from aidotnet.tensors_amd import AttnDesc
+    B, H, S = 2, 3, 333
+    g = torch.Generator(device="cuda"); g.manual_seed(D + len(kind))
+    dt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[kind]
+    q, k, v = (torch.randn(B, H, S, D, device="cuda", generator=g).to(dt) for _ in range(3))
+    sc = 1 / math.sqrt(D)
+
+    def run(o_view, o_strides):
+        d = AttnDesc(B=B, H=H, Hkv=H, Sq=S, Sk=S, D=D, scale=sc, causal=1)
+        d.o_strides[:] = o_strides
+        lse = torch.full((B, H, S), float("nan"), device="cuda")
+        be._attn(kind, be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), o_view, be.WrapTensor(lse), None, None, None, d)
+        return lse
+
+    dense = torch.full((B, H, S, D), float("nan"), device="cuda")
+    lse0 = run(be.WrapTensor(dense), [H * S * D, S * D, D])
+    bshd = torch.full((B, S, H, D), float("nan"), device="cuda")
+    lse1 = run(be.WrapTensor(bshd), [S * H * D, D, H * D])
+    raw = torch.full((B * H * S * D + 1,), float("nan"), device="cuda")
+    lse2 = run(_Off(raw, 1), [H * S * D, S * D, D])
+    torch.cuda.synchronize()
+    assert torch.isfinite(dense).all()
+    assert torch.equal(bshd.permute(0, 2, 1, 3), dense) and torch.equal(lse1, lse0)
+    assert torch.equal(raw[1:].view(B, H, S, D), dense) and torch.equal(lse2, lse0)
+    assert torch.isnan(raw[0])
+    ref = torch.nn.functional.scaled_dot_product_attention(q.double(), k.double(), v.double(), is_causal=True)
+    assert float((dense.double() - ref).abs().max()) <= (1e-4 if kind == "f32" else 2e-2)
+
+
 class _Off:
     """A buffer view starting `off` elements into a tensor (raw device pointer arithmetic)."""
 
