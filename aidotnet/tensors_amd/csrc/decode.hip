@@ -316,9 +316,10 @@ int attn_decode_splits(int kind, const AttnParams& p, int splits)
         const int gq = p.Hkv > 0 ? p.H / p.Hkv : 1;
         const bool grouped = attn_group_decode_applies(kind, p);
         long long bh = (long long)p.B * (grouped ? p.Hkv : p.H / (gq % 4 == 0 ? 4 : gq % 2 == 0 ? 2 : 1));
-        // ~8 workgroups per CU for the per-head kernel; the grouped form (one computing wave per workgroup, a key tile per barrier)
-        // is fastest at about two workgroups per CU (B32 H32 Hkv8 KV4096: 85 us with 2 ranges, 92 with 8; B8 KV8192: 46 with 8, 54 with 32)
-        splits = (int)(((grouped ? 512 : 2048) + bh - 1) / bh);
+        // about four workgroups per CU for the per-head kernel, rounded to the nearest count (a grid that is already that large is not
+        // split: the merge pass costs more than it balances); the grouped form (one computing wave per workgroup, a key tile per
+        // barrier) is fastest at about two per CU (B32 H32 Hkv8 KV4096: 85 us with 2 ranges, 92 with 8; B8 KV8192: 46 with 8, 54 with 32)
+        splits = grouped ? (int)((512 + bh - 1) / bh) : (int)((1024 + bh / 2) / bh);
     }
     if (splits > maxs) splits = maxs;
     if (splits > 64) splits = 64;
