@@ -37,14 +37,14 @@ TRAFFIC_BYTES = {
     "gemm_f16_proj_f32out": int((17048 * 2.0 + 49178) * 1024),
     "gemm_f32_proj": int((43100 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
-    "decode_bf16": int((1048890 * 2.0 + 1088) * 1024),
+    "decode_bf16": int((1048770 * 2.0 + 512) * 1024),
     "attn_f16_prefill": int((139311 * 2.0 + 132113) * 1024),
     "attn_bf16_prefill": int((139768 * 2.0 + 132113) * 1024),
     "attn_f32_prefill": int((22644 * 2.0 + 12480) * 1024),
     "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
     # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass)
-    "decode_bf16_gqa": int(((262406 + 2641) * 2.0 + 4166 + 512) * 1024),
-    "decode_f32_gqa": int(((526428 + 2641) * 2.0 + 4352 + 512) * 1024),
+    "decode_bf16_gqa": int(((262417 + 1108) * 2.0 + 1040 + 512) * 1024),
+    "decode_f32_gqa": int(((525392 + 1108) * 2.0 + 2176 + 512) * 1024),
     "gemm_f32_m16": int(((33827 + 1026) * 2.0 + 2048 + 256) * 1024),
 }
 # MI355X published dense peaks
