@@ -892,7 +892,9 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     constexpr int BM = HALF ? 128 : 256, BN = 64 * TJ, BK = 64;
     constexpr int WTM = BM / 2, WTN = 16 * TJ;
     constexpr int TI = WTM / 16;                  // 16 x 16 blocks of the wave tile: TI x TJ
-    constexpr int BROW = (HALF ? 128 : 256) * EB; // LDS pitch of a B k-row (16 or 32 chunk positions)
+    // LDS pitch of a B k-row (16 or 32 chunk positions): 512 bytes, or 256 for the 128-column tiles (with 512-byte rows the 256 x 128
+    // tile fetched 256 columns of B per k-row for the 128 it uses: 6-8 % slower on every shape that takes it)
+    constexpr int BROW = ((HALF || TJ == 2) ? 128 : 256) * EB;
     constexpr int BCH = BN / E;                   // 16-byte chunks of a k-row that hold tile columns
     constexpr int ABYTES = BM * 128, BBYTES = BK * BROW, STAGE = ABYTES + BBYTES;
     constexpr int LA = BM / 64, LB = BK * BROW / 8192, RPL = 1024 / BROW, LPR = BROW / 16;
@@ -1097,6 +1099,8 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     // the last stage (dead after the final barrier), 16-byte chunk c of a staged row at position c ^ ((row >> 1) & 7).
     {
         // (HALF: every stage is dead after the final barrier; the eight waves' 8 KiB take the first two)
+        // (the eight waves' 64 KiB may reach past a 48 KiB stage into the other one, which is just as dead; the launch allocates 128 KiB)
+        static_assert(HALF || STAGE + 8 * 8192 <= 2 * (256 * 128 + 128 * 256), "C staging must stay inside the allocation");
         unsigned char* stg = smem + (HALF ? 0 : ((KT - 1) & 1) * STAGE) + wave * 8192;
         constexpr int ROWB = WTN * OB;                // bytes of one staged row
         constexpr int CPR = ROWB / 16;                // 16-byte chunks per staged row
