@@ -1640,7 +1640,7 @@ static int smallm_kper(int N, int K)
     kper = (kper + 31) / 32 * 32;
     // K ranges that start a multiple of 4 MiB apart put the workgroups of a column block on the same memory channels
     // (1 x 8192 x 8192: 60 us with 256-row ranges, 8 MiB apart, against 43-48 us with any other size)
-    while (((long long)kper * N * 4) % (1LL << 22) == 0) kper += 32;
+    for (int tries = 0; tries < 64 && ((long long)kper * N * 4) % (1LL << 22) == 0; tries++) kper += 8;   // (bounded: a very wide N aliases at every multiple of 32)
     return kper;
 }
 

@@ -114,7 +114,10 @@ def gpu_gemm(be, a, b, m, n, k, alpha=1.0, beta=0.0, c0=None):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("m,k,n", SHAPES + [(1, 1024, 4096), (3, 4096, 4096), (8, 1000, 1001), (7, 33, 130), (1, 320, 1280), (6, 5000, 260)])
+# (the last two: row strides of 32 KiB and 128 KiB, where the K ranges are moved off multiples of 4 MiB -- at N = 32768 every range
+# size is such a multiple and the search must give up)
+@pytest.mark.parametrize("m,k,n", SHAPES + [(1, 1024, 4096), (3, 4096, 4096), (8, 1000, 1001), (7, 33, 130), (1, 320, 1280), (6, 5000, 260),
+                                            (2, 2048, 8192), (1, 512, 32768)])
 def test_gpu_small_m_overwrite(be, m, k, n):
     a, b, _ = case(m, k, n, m * 31 + k + n) if m * k + k * n < 600000 else (None, None, None)
     if a is None:
