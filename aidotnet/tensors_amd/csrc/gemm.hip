@@ -847,7 +847,8 @@ static hipError_t launch_gemm_dl(GemmArgs g, int batch, hipStream_t stream)
 
 // ---------------------------------------------------------------------------------------------
 // 256 x 256 x 64 direct-to-LDS kernel for 16-bit inputs on v_mfma_f32_16x16x32 (the form the large exact-fit problems take:
-// M % 256 == 0, N % 256 == 0, K % 64 == 0, B stored [K,N]).  Same tile, loads and LDS layout as gemm_dl_kernel<.., 256>; what
+// N a multiple of the tile width, K % 64 == 0, B stored [K,N]; M may be ragged: the rows of A past M are clamped loads of row
+// M - 1 whose products are never stored).  Same tile, loads and LDS layout as gemm_dl_kernel<.., 256>; what
 // differs is the matrix instruction.  Under load this part runs at the clock its power limit allows, and per multiply-add the
 // 16 x 16 x 32 instruction moves 20 % fewer register bytes than 32 x 32 x 16 (half the accumulator traffic, twice the
 // operand traffic): with random fp16 operands and nothing else running it sustains 1.71 PFLOP/s against 1.52, and this kernel
@@ -918,11 +919,13 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     auto b_swz = [](int row) -> int { return ((row & 3) << 2) | (((row >> 3) & 1) << 1); };
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
-    uint32_t a_lane_off[2], b_lane_off[LB];
+    // A rows past M (the last tile row of a ragged M) are clamped to row M - 1: valid loads whose products are never stored
+    uint32_t a_lane_off[LA], b_lane_off[LB];
 #pragma unroll
-    for (int par = 0; par < 2; par++) {
+    for (int i = 0; i < LA; i++) {
         const int ra = lane >> 3, pos_a = lane & 7;
-        a_lane_off[par] = (uint32_t)(ra * g.lda + (pos_a ^ ((4 * par + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
+        const int row = min(m0 + 8 * (LA * wave + i) + ra, g.M - 1) - m0;        // relative to the tile's first row, >= 0
+        a_lane_off[i] = (uint32_t)(row * g.lda + (pos_a ^ ((4 * (i & 1) + (ra >> 1)) & 7)) * E) * (uint32_t)EB;
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
@@ -931,9 +934,9 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
         if (chunk >= BCH) chunk -= LPR - BCH >= BCH ? BCH : LPR - BCH;    // a valid chunk again (its LDS position is never read)
         b_lane_off[i] = (uint32_t)(rb * g.ldb + chunk * E) * (uint32_t)EB;
     }
-    const unsigned char* a_base = A + (long long)(m0 + 8 * LA * wave_s) * g.lda * EB;
+    const unsigned char* a_base = A + (long long)m0 * g.lda * EB;
     const unsigned char* b_base = B + ((long long)(RPL * LB * wave_s) * g.ldb + n0) * EB;
-    const long long a_step = 8LL * g.lda * EB, b_step = (long long)RPL * g.ldb * EB;
+    const long long b_step = (long long)RPL * g.ldb * EB;
     const int KT = g.K / BK;
     auto issue_loads = [&](int kt, int stage) {
         const uint32_t as = lds0 + stage * STAGE + wave_s * (LA * 1024);
@@ -941,7 +944,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
         const unsigned char* a_src = a_base + (long long)kt * 128;
         const unsigned char* b_src = b_base + (long long)kt * BK * g.ldb * EB;
 #pragma unroll
-        for (int i = 0; i < LA; i++) dma16_base(a_src + i * a_step, a_lane_off[i & 1], as + i * 1024);
+        for (int i = 0; i < LA; i++) dma16_base(a_src, a_lane_off[i], as + i * 1024);
 #pragma unroll
         for (int i = 0; i < LB; i++) dma16_base(b_src + i * b_step, b_lane_off[i], bs + i * 1024);
     };
@@ -1146,8 +1149,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 const int row = u / CPR, c = u % CPR;
                 const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
                 u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
-                if constexpr (NTS) __builtin_nontemporal_store(v, dst);
-                else *dst = v;
+                if (m0 + wm * WTM + ip * 16 + row < g.M) {
+                    if constexpr (NTS) __builtin_nontemporal_store(v, dst);
+                    else *dst = v;
+                }
             }
         }
     }
@@ -1157,7 +1162,7 @@ template <typename T, typename OutT, int TJ = 4, bool HALF = false>
 static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 {
     constexpr int smem = HALF ? DL16_HALF_STAGES * (128 * 128 + 64 * 256) : 2 * (256 * 128 + 128 * 256);
-    g.tiles_m = g.M / (HALF ? 128 : 256);
+    g.tiles_m = (g.M + (HALF ? 127 : 255)) / (HALF ? 128 : 256);      // the last tile row may be partial
     g.tiles_n = g.N / (64 * TJ);
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch);
     // Non-temporal stores of C when A, B and C together exceed the 256 MB last-level cache: C then no longer displaces the operand
@@ -1723,7 +1728,7 @@ static bool dl16_applies(const GemmArgs& g)
            g.alpha == 1.0f && g.beta == 0.0f;
 }
 
-// Tile width (in 64-column units: 4, 3 or 2) of the 16 x 16 x 32 kernel for a 16-bit problem with M % 256 == 0 and K % 64 == 0, or 0
+// Tile width (in 64-column units: 4, 3 or 2) of the 16 x 16 x 32 kernel for a 16-bit problem with K % 64 == 0 (any M), or 0
 // when none of the widths divides N or the 128 x 128 / 64 x 64 tiles of the 32 x 32 x 16 kernel are expected to finish earlier.
 // Every candidate is scored as (how evenly its tiles load the 256 CUs) x (its rate per flop relative to the 256 x 256 tile): a
 // narrower tile moves more A bytes per flop (and the 256 x 128 one wastes half of its B loads); the 128 x 128 tile runs at about
@@ -1732,11 +1737,9 @@ static bool dl16_applies(const GemmArgs& g)
 static int dl16_width(int M, int N, int K, int batch)
 {
     if (K % 64 != 0) return 0;
-    if (M % 256 != 0) {
-        if (M % 128 != 0 || N % 128 != 0) return 0;
-        const long long t128 = (long long)(M / 128) * (N / 128) * batch, t64 = (long long)(M / 64) * (N / 64) * batch;
-        return DL16_HALF_EFF * cu_fill(t128) >= 0.45 * cu_fill(t64) ? 1 : 0;
-    }
+    // M may be ragged (the last tile row is partial: clamped loads, guarded stores); the rows a tile height pads count as waste
+    const long long tm256 = (M + 255) / 256, tm128 = (M + 127) / 128, tm64 = (M + 63) / 64;
+    const double use256 = (double)M / (double)(tm256 * 256), use128 = (double)M / (double)(tm128 * 128), use64 = (double)M / (double)(tm64 * 64);
     const int widths[3] = {4, 3, 2};
     const double eff[3] = {1.0, 0.94, 0.8};
     int best = 0;
@@ -1744,15 +1747,15 @@ static int dl16_width(int M, int N, int K, int batch)
     for (int i = 0; i < 3; i++) {
         const int bn = 64 * widths[i];
         if (N % bn != 0) continue;
-        const long long t = (long long)(M / 256) * (N / bn) * batch;
-        const double score = cu_fill(t) * eff[i];
+        const long long t = tm256 * (N / bn) * batch;
+        const double score = cu_fill(t) * eff[i] * use256;
         if (score > best_score) { best_score = score; best = widths[i]; }
     }
-    const long long t128 = (long long)((M + 127) / 128) * ((N + 127) / 128) * batch;
-    const long long t64 = (long long)((M + 63) / 64) * ((N + 63) / 64) * batch;
-    // the 128 x 128 tile of this kernel (code 1): whole tiles only
-    if (M % 128 == 0 && N % 128 == 0 && DL16_HALF_EFF * cu_fill(t128) > best_score) { best_score = DL16_HALF_EFF * cu_fill(t128); best = 1; }
-    if (0.55 * cu_fill(t128) > best_score || 0.45 * cu_fill(t64) > best_score) return 0;
+    const long long t128 = tm128 * ((N + 127) / 128) * batch;
+    const long long t64 = tm64 * ((N + 63) / 64) * batch;
+    // the 128 x 128 tile of this kernel (code 1): whole column tiles only
+    if (N % 128 == 0 && DL16_HALF_EFF * cu_fill(t128) * use128 > best_score) { best_score = DL16_HALF_EFF * cu_fill(t128) * use128; best = 1; }
+    if (0.55 * cu_fill(t128) * use128 > best_score || 0.45 * cu_fill(t64) * use64 > best_score) return 0;
     return best;
 }
 
@@ -1803,13 +1806,13 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 192 || tile == 193) {                 // 256 x 192 / 256 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
             const int bn = tile == 192 ? 192 : 128;
-            if (!(g.M % 256 == 0 && g.N % bn == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
+            if (!(g.N % bn == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
             return tile == 192 ? launch_gemm_dl16<T, OutT, 3>(g, batch, stream) : launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
         }
     }
     if constexpr (E == 8 && !TRANSB) {
         if (tile == 130) {                                // 128 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
-            if (!(g.M % 128 == 0 && g.N % 128 == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
+            if (!(g.N % 128 == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
             return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
         }
     }

@@ -150,7 +150,9 @@ HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7
                # skinny-M (decode projection) path: M <= 32, N % 128 == 0, K % 64 == 0
                (1, 128, 64), (5, 256, 192), (17, 384, 1024), (32, 128, 64), (8, 4096, 512), (200, 304, 128), (129, 136, 256), (1000, 1000, 256),
                # split-K through the batch dimension of the 128 x 128 kernel: few tiles over a long K (16, 8 and 2 K ranges)
-               (128, 512, 1024), (256, 1024, 4096), (384, 1152, 1536), (512, 2048, 1024)]
+               (128, 512, 1024), (256, 1024, 4096), (384, 1152, 1536), (512, 2048, 1024),
+               # a ragged M on the 16 x 16 x 32 kernel (last tile row partial; 256-, 192- and 128-wide tiles, and the 128 x 128 one)
+               (1000, 4096, 128), (300, 3072, 192), (700, 1920, 64), (3000, 384, 256), (1, 256, 64 * 3), (257, 2048, 128)]
 
 
 def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
@@ -472,7 +474,7 @@ def test_config2_square_8192_baseline_distribution_sampled_rows(be, kind):
                                         (130, 128, 128, 64), (130, 384, 640, 192), (130, 128, 256, 4096), (130, 1152, 384, 128)])
 def test_half_gemm_16x16x32_kernel_tile_widths(be, kind, tile, M, N, K):
     # the 256 x 192, 256 x 128 and 128 x 128 tiles of the 16 x 16 x 32 kernel (codes 192 / 193 / 130) and its 256 x 256 tile, forced on small whole-tile
-    # shapes: bit-exact on dyadic inputs for both output types, bias + activation epilogue, guard band, refusal of ragged shapes
+    # shapes: bit-exact on dyadic inputs for both output types, bias + activation epilogue, guard band, a ragged M, refusal of a ragged N
     be.SetGemmTile(tile)
     try:
         rng = np.random.default_rng(tile + M + 2 * N + 3 * K)
@@ -494,10 +496,14 @@ def test_half_gemm_16x16x32_kernel_tile_widths(be, kind, tile, M, N, K):
         got = c[:M * N].reshape(M, N).cpu().numpy()
         assert mixed_err(got, np.maximum(truth + bias[None, :], 0.0)) <= 1e-4
         assert bool((c[M * N:] == -7.0).all())                     # one row of guard band behind C stays untouched
+        # a ragged M is computed (rows past M are clamped loads whose products are never stored) ...
+        short = _half_gemm(be, kind, np.ascontiguousarray(ab.reshape(M, K)[:M - 5]).reshape(-1), bb, M - 5, N, K, True)
+        assert mixed_err(short, truth[:M - 5]) <= 1e-4
         if tile != 256:
             from aidotnet.tensors_amd import HipException
-            with pytest.raises(HipException):                      # these tile codes take whole tiles only
-                _half_gemm(be, kind, ab[:(M - 1) * K], bb, M - 1, N, K, True)
+            nb, _ = round_to(np.ascontiguousarray(bw.reshape(K, N)[:, :N - 8]), kind)
+            with pytest.raises(HipException):                      # ... these tile codes take whole column tiles only
+                _half_gemm(be, kind, ab, nb, M, N - 8, K, True)
     finally:
         be.SetGemmTile(0)
 
