@@ -39,6 +39,9 @@ struct GemmArgs {
     const float* bias;
     int act;
     float act_param;
+    // 16 x 16 x 32 kernel only.  > 0: C has this many columns (fewer than N, the columns past them are padding of B that is
+    // computed and dropped) and ldc is any element count, so a row of C may start off a 16-byte boundary
+    int c_cols = 0;
 };
 
 #if AIDN_GEMM_PART == 0
@@ -1150,7 +1153,23 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
                 u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
                 if (m0 + wm * WTM + ip * 16 + row < g.M) {
-                    if constexpr (NTS) __builtin_nontemporal_store(v, dst);
+                    if (g.c_cols > 0) {
+                        // rows of C at any element offset: whole chunks by one under-aligned 16-byte store, the chunk that
+                        // crosses the last column by elements
+                        typedef typename Raw<OutT>::type out_t;
+                        typedef u32x4 u32x4_elem __attribute__((aligned(2)));
+                        constexpr int PER = 16 / OB;
+                        const int col0 = n0 + wn * WTN + c * PER;
+                        if (col0 + PER <= g.c_cols) *(u32x4_elem*)dst = v;
+                        else {
+#pragma unroll
+                            for (int e = 0; e < PER; e++)
+                                if (col0 + e < g.c_cols) {
+                                    if constexpr (OB == 2) ((out_t*)dst)[e] = (out_t)(v[e >> 1] >> ((e & 1) * 16));
+                                    else ((out_t*)dst)[e] = v[e];
+                                }
+                        }
+                    } else if constexpr (NTS) __builtin_nontemporal_store(v, dst);
                     else *dst = v;
                 }
             }
@@ -1360,12 +1379,177 @@ static int splitk16_ranges(int M, int N, int K)
     return ks >= 2 && (long long)K >= 1024 ? ks : 0;
 }
 
-#if AIDN_GEMM_PART == 0
-size_t gemm_16_workspace_bytes(int M, int N, int K)
+// 16-bit problems whose rows are not 16-byte aligned (N or K not a multiple of 8) would run on 2-byte loads, an order of
+// magnitude below the vector-load kernels.  They are copied instead into zero-padded, aligned operands in the workspace
+// (K up to a multiple of 64, N up to a multiple of 128, or of 8 for a narrow N), multiplied there by the kernels for aligned
+// problems and the columns of C copied back: three extra passes over A, B and C, which a product of this size repays many
+// times over.  The zero columns of A meet zero rows of B, so the padded product holds exactly the sums of the plain one.
+struct PadPlan {
+    int Np, Kp;                                   // padded N and K
+    size_t a_off, b_off, c_off, bias_off, inner_off, total;
+};
+static size_t gemm_16_inner_workspace_bytes(int M, int N, int K)
 {
     if (skinny_applies(M, N, K)) return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
     const int ks = splitk16_ranges(M, N, K);
     return ks ? (size_t)ks * M * N * sizeof(float) : 0;
+}
+static bool pad16_plan(int M, int N, int K, PadPlan* pl)
+{
+    if (N % 8 == 0 && K % 8 == 0) return false;
+    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;        // launch-bound either way
+    const int Np = N >= 512 ? (N + 127) / 128 * 128 : (N + 7) / 8 * 8;
+    const int Kp = (K + 63) / 64 * 64;
+    auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    size_t off = 0;
+    pl->Np = Np; pl->Kp = Kp;
+    pl->a_off = off; off += up((size_t)M * Kp * 2);
+    pl->b_off = off; off += up((size_t)Kp * Np * 2);
+    pl->c_off = off; off += up((size_t)M * Np * 4);
+    pl->bias_off = off; off += up((size_t)Np * 4);
+    pl->inner_off = off; off += gemm_16_inner_workspace_bytes(M, Np, Kp);
+    pl->total = off;
+    return off <= ((size_t)4 << 30);
+}
+
+// dst [rows_dst, cols_dst] (16-byte aligned rows) <- src [rows_src, cols_src] (dense, any alignment), zeros elsewhere; E = element.
+// One thread fills one 16-byte chunk of dst from element loads.
+template <typename E>
+__global__ __launch_bounds__(256) void pad_rows_kernel(const E* __restrict__ src, E* __restrict__ dst, int rows_src, int cols_src,
+                                                       int rows_dst, int cols_dst)
+{
+    constexpr int PER = 16 / (int)sizeof(E);
+    typedef E Vec __attribute__((ext_vector_type(PER)));
+    const int per_row = cols_dst / PER;
+    const long long total = (long long)rows_dst * per_row;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += stride) {
+        const long long row = g / per_row;
+        const int c0 = (int)(g - row * per_row) * PER;
+        Vec v;
+#pragma unroll
+        for (int e = 0; e < PER; e++) v[e] = (row < rows_src && c0 + e < cols_src) ? src[row * cols_src + c0 + e] : (E)0;
+        *(Vec*)(dst + row * cols_dst + c0) = v;
+    }
+}
+
+// The same for 2-byte elements with every access a dword that is contiguous across the wave: one thread per dword of dst
+// (columns 2 i, 2 i + 1 of a row).  A source row starts on a dword boundary or 2 bytes past one; in the second case the two
+// elements come from the high half of one source dword and the low half of the next.  A dword of the source is only loaded whole
+// when both of its elements belong to the array.  grid = (ceil(cols_dst / 512), rows): no division per thread.
+#if AIDN_GEMM_PART == 0
+__global__ __launch_bounds__(256) void pad_rows16_kernel(const uint16_t* __restrict__ src, uint32_t* __restrict__ dst, int rows_src, int cols_src,
+                                                         int rows_dst, int cols_dst)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;                    // dword column of dst
+    const int per_row = cols_dst >> 1;
+    if (i >= per_row) return;
+    const uint32_t* base = (const uint32_t*)(((uintptr_t)src) & ~(uintptr_t)3);
+    const long long off0 = (((uintptr_t)src) & 2) ? 1 : 0;           // flat element index of src[0] counted from base
+    const long long end = off0 + (long long)rows_src * cols_src;     // one past the last element
+    auto dword = [&](long long k) -> uint32_t {                      // source dword k: elements 2k (low half) and 2k + 1
+        const bool lo = 2 * k >= off0 && 2 * k < end, hi = 2 * k + 1 >= off0 && 2 * k + 1 < end;
+        if (lo && hi) return base[k];
+        const uint16_t* h = (const uint16_t*)base;
+        return (lo ? (uint32_t)h[2 * k] : 0u) | (hi ? (uint32_t)h[2 * k + 1] << 16 : 0u);
+    };
+    const int col = 2 * i;
+    auto one = [&](int row) -> uint32_t {                            // guarded form: any row, any position in the array
+        uint32_t v = 0;
+        if (row < rows_src && col < cols_src) {
+            const long long f = off0 + (long long)row * cols_src + col;
+            const long long k = f >> 1;
+            if (f & 1) v = (dword(k) >> 16) | (dword(k + 1) << 16);
+            else v = dword(k);
+            if (col + 1 >= cols_src) v &= 0xFFFFu;
+        }
+        return v;
+    };
+    // four rows per step with all eight loads issued before the first use (a row is one dword per thread: the kernel is bound
+    // by memory latency unless several rows are in flight); rows whose dwords k and k + 1 lie strictly inside the array only
+    const int step = gridDim.y;
+    int row = blockIdx.y;
+    if (row == 0) { dst[i] = one(0); row += step; }
+    const uint32_t keep = col + 1 >= cols_src ? 0xFFFFu : 0xFFFFFFFFu;
+    if (col < cols_src && cols_src >= 8) {
+        for (; (long long)row + 3LL * step < (long long)rows_src - 1; row += 4 * step) {
+            uint32_t d0[4], d1[4];
+            long long f[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                f[u] = off0 + (long long)(row + u * step) * cols_src + col;
+                d0[u] = base[f[u] >> 1];
+                d1[u] = base[(f[u] >> 1) + 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const uint32_t v = (f[u] & 1) ? (d0[u] >> 16) | (d1[u] << 16) : d0[u];
+                dst[(long long)(row + u * step) * per_row + i] = v & keep;
+            }
+        }
+    }
+    for (; row < rows_dst; row += step) dst[(long long)row * per_row + i] = one(row);
+}
+#endif
+
+// dst [rows, cols] (dense, any row alignment, dst itself 16-byte aligned) <- the first cols columns of src [rows, cols_src]:
+// one thread per 16-byte chunk of the flat destination; the last, partial chunk is stored by elements.
+template <typename E>
+__global__ __launch_bounds__(256) void unpad_rows_kernel(const E* __restrict__ src, E* __restrict__ dst, long long rows, int cols, int cols_src)
+{
+    constexpr int PER = 16 / (int)sizeof(E);
+    typedef E Vec __attribute__((ext_vector_type(PER)));
+    const long long total = rows * cols;
+    const long long chunks = (total + PER - 1) / PER;
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    for (long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x; g < chunks; g += stride) {
+        const long long f0 = g * PER;
+        long long row = f0 / cols;
+        int col = (int)(f0 - row * cols);
+        Vec v;
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+            v[e] = f0 + e < total ? src[row * cols_src + col] : (E)0;
+            if (++col == cols) { col = 0; row++; }
+        }
+        if (f0 + PER <= total) *(Vec*)(dst + f0) = v;
+        else for (int e = 0; e < PER && f0 + e < total; e++) dst[f0 + e] = v[e];
+    }
+}
+
+// esize 2 or 4
+hipError_t pad_rows(hipStream_t stream, const void* src, void* dst, int rows_src, int cols_src, int rows_dst, int cols_dst, int esize);
+hipError_t unpad_rows(hipStream_t stream, const void* src, void* dst, long long rows, int cols, int cols_src, int esize);
+
+#if AIDN_GEMM_PART == 0
+static unsigned copy_grid(long long chunks)
+{
+    const long long wg = (chunks + 255) / 256;
+    return (unsigned)(wg > 256 * 16 ? 256 * 16 : wg < 1 ? 1 : wg);
+}
+hipError_t pad_rows(hipStream_t stream, const void* src, void* dst, int rows_src, int cols_src, int rows_dst, int cols_dst, int esize)
+{
+    const long long chunks = (long long)rows_dst * (cols_dst / (16 / esize));
+    if (esize == 2 && cols_dst >= 256) {
+        const unsigned gy = (unsigned)((rows_dst + 7) / 8 < 8192 ? (rows_dst + 7) / 8 : 8192);      // about eight rows per thread
+        hipLaunchKernelGGL(pad_rows16_kernel, dim3((unsigned)((cols_dst / 2 + 255) / 256), gy), dim3(256), 0, stream, (const uint16_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
+    } else if (esize == 2) hipLaunchKernelGGL((pad_rows_kernel<uint16_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint16_t*)src, (uint16_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
+    else hipLaunchKernelGGL((pad_rows_kernel<uint32_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint32_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
+    return hipGetLastError();
+}
+hipError_t unpad_rows(hipStream_t stream, const void* src, void* dst, long long rows, int cols, int cols_src, int esize)
+{
+    const long long chunks = (rows * cols + 16 / esize - 1) / (16 / esize);
+    if (esize == 2) hipLaunchKernelGGL((unpad_rows_kernel<uint16_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint16_t*)src, (uint16_t*)dst, rows, cols, cols_src);
+    else hipLaunchKernelGGL((unpad_rows_kernel<uint32_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint32_t*)src, (uint32_t*)dst, rows, cols, cols_src);
+    return hipGetLastError();
+}
+
+size_t gemm_16_workspace_bytes(int M, int N, int K)
+{
+    PadPlan pl;
+    if (pad16_plan(M, N, K, &pl)) return pl.total;
+    return gemm_16_inner_workspace_bytes(M, N, K);
 }
 #endif
 
@@ -1940,6 +2124,36 @@ template <typename T>
 static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
                                 int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
 {
+    PadPlan pl;
+    if (force_tile == 0 && workspace && aligned16(C) && aligned16(workspace) && pad16_plan(M, N, K, &pl)) {
+        unsigned char* w = (unsigned char*)workspace;
+        const bool padA = pl.Kp != K, padC = pl.Np != N;
+        const uint16_t* Ap = A;
+        if (padA) {
+            if (hipError_t e = pad_rows(stream, A, w + pl.a_off, M, K, M, pl.Kp, 2)) return e;
+            Ap = (const uint16_t*)(w + pl.a_off);
+        }
+        if (hipError_t e = pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 2)) return e;
+        const float* bp = bias;
+        if (bias && padC) {
+            if (hipError_t e = pad_rows(stream, bias, w + pl.bias_off, 1, N, 1, pl.Np, 4)) return e;
+            bp = (const float*)(w + pl.bias_off);
+        }
+        if (padC && pl.Np % 128 == 0 && pl.Kp < (1 << 21) && pl.Np < (1 << 21)) {
+            // the 16 x 16 x 32 kernel stores the N real columns straight into the caller's C
+            GemmArgs gp{Ap, w + pl.b_off, C, M, pl.Np, pl.Kp, pl.Kp, pl.Np, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bp, act, act_param};
+            gp.c_cols = N;
+            const int wd = dl16_width(M, pl.Np, pl.Kp, 1);
+            if (wd == 4) return out32 ? launch_gemm_dl16<T, float, 4>(gp, 1, stream) : launch_gemm_dl16<T, T, 4>(gp, 1, stream);
+            if (wd == 3) return out32 ? launch_gemm_dl16<T, float, 3>(gp, 1, stream) : launch_gemm_dl16<T, T, 3>(gp, 1, stream);
+            if (wd == 2) return out32 ? launch_gemm_dl16<T, float, 2>(gp, 1, stream) : launch_gemm_dl16<T, T, 2>(gp, 1, stream);
+            if (wd == 1) return out32 ? launch_gemm_dl16<T, float, 2, true>(gp, 1, stream) : launch_gemm_dl16<T, T, 2, true>(gp, 1, stream);
+        }
+        void* Cp = padC ? (void*)(w + pl.c_off) : C;
+        if (hipError_t e = gemm_16_typed<T>(stream, Ap, (const uint16_t*)(w + pl.b_off), Cp, out32, M, pl.Np, pl.Kp, 0,
+                                            pl.total > pl.inner_off ? (void*)(w + pl.inner_off) : nullptr, bp, act, act_param)) return e;
+        return padC ? unpad_rows(stream, Cp, C, M, N, pl.Np, out32 ? 4 : 2) : hipSuccess;
+    }
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
     if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         float* ws = (float*)workspace;

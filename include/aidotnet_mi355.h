@@ -120,7 +120,10 @@ AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A,
  * round-to-nearest-even narrow, the arithmetic of the CPU kernel (Engines/Simd/HalfKernels.cs:35-99).
  * The bf16 pair has no member in the reference's backend interface today (its planner widens
  * bf16 tensors to fp32, Engines/Gpu/GpuPrecisionPolicy.cs:497-532); it follows the CPU kernel
- * Engines/Simd/BFloat16Kernels.cs:144-211 and NumericOperations/BFloat16.cs:64-90. */
+ * Engines/Simd/BFloat16Kernels.cs:144-211 and NumericOperations/BFloat16.cs:64-90.
+ * Any M, N and K are accepted.  When N or K is not a multiple of 8 (rows that are not whole 16-byte chunks) a product of some size
+ * is computed from zero-padded copies of A and B held in the stream's workspace -- same sums, three more passes over the
+ * operands; a weight of such a width that is used many times is better stored padded by the caller. */
 AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K);
 AIDN_API int aidn_mi355_hgemm_f16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K);
 AIDN_API int aidn_mi355_bf16gemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K);

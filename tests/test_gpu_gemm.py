@@ -152,7 +152,11 @@ HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7
                # split-K through the batch dimension of the 128 x 128 kernel: few tiles over a long K (16, 8 and 2 K ranges)
                (128, 512, 1024), (256, 1024, 4096), (384, 1152, 1536), (512, 2048, 1024),
                # a ragged M on the 16 x 16 x 32 kernel (last tile row partial; 256-, 192- and 128-wide tiles, and the 128 x 128 one)
-               (1000, 4096, 128), (300, 3072, 192), (700, 1920, 64), (3000, 384, 256), (1, 256, 64 * 3), (257, 2048, 128)]
+               (1000, 4096, 128), (300, 3072, 192), (700, 1920, 64), (3000, 384, 256), (1, 256, 64 * 3), (257, 2048, 128),
+               # rows that are not whole 16-byte chunks (odd N and / or K), large enough to be copied into padded operands: narrow N
+               # (padded C, copied back), wide N (the kernel stores the real columns), odd K only, skinny and split-K inner problems
+               (300, 301, 299), (512, 1001, 300), (1000, 1025, 130), (2049, 2051, 70), (700, 1024, 77), (16, 1001, 515), (256, 1100, 1030),
+               (130, 4099, 257)]
 
 
 def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
@@ -279,6 +283,34 @@ def test_half_gemm_16bit_output_guard_band_and_odd_offset(be, kind, M, N, K):
         torch.cuda.synchronize()
         assert np.array_equal(bits16(flat[lead:lead + M * N]).reshape(M, N), want16.reshape(M, N)), lead
         assert bool((flat[:lead].float() == -7.0).all()) and bool((flat[lead + M * N:].float() == -7.0).all()), lead
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(300, 301, 299), (640, 1001, 300), (1000, 2051, 131), (520, 1024, 77)])
+def test_half_gemm_unaligned_rows_guard_band_odd_operand_offsets_and_epilogue(be, kind, M, N, K):
+    # odd N / K: the operands are copied into padded, aligned buffers.  A and B may themselves start on an odd element (the copy then
+    # begins in the high half of a dword); elements after the matrix must stay untouched; bias and activation ride along
+    rng = np.random.default_rng(M + N + K)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+    ab, _ = round_to(a, kind); bb, _ = round_to(b, kind)
+    want16, want32 = (oracle.hgemm if kind == "f16" else oracle.bf16gemm)(ab, bb, M, K, N)
+    for lead in (0, 1, 3):
+        fa = torch.zeros(lead + M * K, dtype=TORCH16[kind], device="cuda"); fa[lead:] = from_bits16(ab, TORCH16[kind]).reshape(-1)
+        fb = torch.zeros(lead + K * N, dtype=TORCH16[kind], device="cuda"); fb[lead:] = from_bits16(bb, TORCH16[kind]).reshape(-1)
+        A = be.WrapTensor(fa[lead:]); B = be.WrapTensor(fb[lead:])
+        c16 = torch.full(((M + 1) * N,), -7.0, device="cuda").to(TORCH16[kind])
+        (be.Hgemm if kind == "f16" else be.Bf16Gemm)(A, B, be.WrapTensor(c16), M, N, K)
+        assert np.array_equal(bits16(c16[:M * N]).reshape(M, N), want16.reshape(M, N)), lead
+        assert bool((c16[M * N:].float() == -7.0).all()), lead
+        c32 = torch.full(((M + 1) * N,), -7.0, device="cuda")
+        (be.GemmFp16In32fOut if kind == "f16" else be.GemmBf16In32fOut)(A, B, be.WrapTensor(c32), M, N, K)
+        assert np.array_equal(c32[:M * N].cpu().numpy().reshape(M, N), want32.reshape(M, N)), lead
+        assert bool((c32[M * N:] == -7.0).all()), lead
+    bias = dyadic(rng, (N,), hi=8).astype(np.float32)
+    c32 = torch.full(((M + 1) * N,), -7.0, device="cuda")
+    be.GemmBiasActivationHalf(kind, A, B, be.WrapTensor(torch.from_numpy(bias).cuda()), be.WrapTensor(c32), M, N, K, 1, 0.0, outputIsFp32=True)
+    assert np.array_equal(c32[:M * N].cpu().numpy().reshape(M, N), np.maximum(want32.reshape(M, N) + bias[None, :], 0.0))
+    assert bool((c32[M * N:] == -7.0).all())
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
