@@ -39,8 +39,9 @@ struct GemmArgs {
     const float* bias;
     int act;
     float act_param;
-    // 16 x 16 x 32 kernel only.  > 0: C has this many columns (fewer than N, the columns past them are padding of B that is
-    // computed and dropped) and ldc is any element count, so a row of C may start off a 16-byte boundary
+    // direct-to-LDS kernels only (the 16 x 16 x 32 one and the instances of the 32 x 32 one with edge handling).  > 0: C has this
+    // many columns (fewer than N, the columns past them are padding of B that is computed and dropped) and ldc is any element
+    // count, so a row of C may start off a 16-byte boundary
     int c_cols = 0;
 };
 
@@ -788,7 +789,7 @@ __global__ __launch_bounds__((TILE == 256 ? 512 : 256) * KSW, TILE == 256 ? 1 : 
         for (int ij = 0; ij < TM * TN; ij++) {
             const int i = ij / TN, j = ij - i * TN;
             const int col = n0 + wn * WTN + j * 32 + l32;
-            if (EDGE && col >= g.N) continue;
+            if (EDGE && col >= (g.c_cols > 0 ? g.c_cols : g.N)) continue;
             const float bias = g.bias ? g.bias[col] : 0.0f;
             f32x16 v = acc[0][0];
 #pragma unroll
@@ -817,7 +818,7 @@ __global__ __launch_bounds__((TILE == 256 ? 512 : 256) * KSW, TILE == 256 ? 1 : 
 #pragma unroll
         for (int j = 0; j < TN; j++) {
             const int col = n0 + wn * WTN + j * 32 + l32;
-            const bool col_ok = !EDGE || col < g.N;
+            const bool col_ok = !EDGE || col < (g.c_cols > 0 ? g.c_cols : g.N);
             if (fused) {                                  // bias and / or activation folded into the store
                 const float bias = (g.bias && col_ok) ? g.bias[col] : 0.0f;
 #pragma unroll
@@ -1490,6 +1491,26 @@ __global__ __launch_bounds__(256) void pad_rows16_kernel(const uint16_t* __restr
     }
     for (; row < rows_dst; row += step) dst[(long long)row * per_row + i] = one(row);
 }
+
+// 4-byte elements: one thread per element of a dst row, four rows in flight; grid = (ceil(cols_dst / 256), rows).
+__global__ __launch_bounds__(256) void pad_rows32_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, int rows_src, int cols_src,
+                                                         int rows_dst, int cols_dst)
+{
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= cols_dst) return;
+    const int step = gridDim.y;
+    int row = blockIdx.y;
+    if (i < cols_src) {
+        for (; (long long)row + 3LL * step < rows_src; row += 4 * step) {
+            uint32_t d[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) d[u] = src[(long long)(row + u * step) * cols_src + i];
+#pragma unroll
+            for (int u = 0; u < 4; u++) dst[(long long)(row + u * step) * cols_dst + i] = d[u];
+        }
+    }
+    for (; row < rows_dst; row += step) dst[(long long)row * cols_dst + i] = (row < rows_src && i < cols_src) ? src[(long long)row * cols_src + i] : 0u;
+}
 #endif
 
 // dst [rows, cols] (dense, any row alignment, dst itself 16-byte aligned) <- the first cols columns of src [rows, cols_src]:
@@ -1534,7 +1555,10 @@ hipError_t pad_rows(hipStream_t stream, const void* src, void* dst, int rows_src
         const unsigned gy = (unsigned)((rows_dst + 7) / 8 < 8192 ? (rows_dst + 7) / 8 : 8192);      // about eight rows per thread
         hipLaunchKernelGGL(pad_rows16_kernel, dim3((unsigned)((cols_dst / 2 + 255) / 256), gy), dim3(256), 0, stream, (const uint16_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
     } else if (esize == 2) hipLaunchKernelGGL((pad_rows_kernel<uint16_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint16_t*)src, (uint16_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
-    else hipLaunchKernelGGL((pad_rows_kernel<uint32_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint32_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
+    else if (cols_dst >= 128) {
+        const unsigned gy = (unsigned)((rows_dst + 7) / 8 < 8192 ? (rows_dst + 7) / 8 : 8192);
+        hipLaunchKernelGGL(pad_rows32_kernel, dim3((unsigned)((cols_dst + 255) / 256), gy), dim3(256), 0, stream, (const uint32_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
+    } else hipLaunchKernelGGL((pad_rows_kernel<uint32_t>), dim3(copy_grid(chunks)), dim3(256), 0, stream, (const uint32_t*)src, (uint32_t*)dst, rows_src, cols_src, rows_dst, cols_dst);
     return hipGetLastError();
 }
 hipError_t unpad_rows(hipStream_t stream, const void* src, void* dst, long long rows, int cols, int cols_src, int esize)
@@ -1840,8 +1864,28 @@ size_t gemm_smallm_workspace_bytes(int M, int N, int K)
     const int kper = smallm_kper(N, K);
     return (size_t)((K + kper - 1) / kper) * M * N * sizeof(float);
 }
+// fp32 problems whose rows are not whole 16-byte chunks (K, or N with B [K,N], not a multiple of 4): zero-padded copies of A and B
+// in the workspace (K up to a multiple of 32, N up to a multiple of 4) feed the direct-to-LDS kernel, whose element stores put the N
+// real columns straight into the caller's C.  Same sums as the plain product: the padding contributes exact zeros.
+struct Pad32Plan { int Np, Kp; size_t a_off, b_off, total; };
+static bool pad32_plan(int M, int N, int K, int transB, Pad32Plan* pl)
+{
+    if (K % 4 == 0 && (transB || N % 4 == 0)) return false;
+    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;
+    pl->Kp = (K + 31) / 32 * 32;
+    pl->Np = transB ? N : (N + 3) / 4 * 4;
+    if (pl->Kp >= (1 << 21) || pl->Np >= (1 << 21)) return false;
+    auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
+    pl->a_off = 0;
+    pl->b_off = up((size_t)M * pl->Kp * 4);
+    pl->total = pl->b_off + up((size_t)(transB ? N : pl->Kp) * (transB ? pl->Kp : pl->Np) * 4);
+    return pl->total <= ((size_t)4 << 30);
+}
+
 size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB)
 {
+    Pad32Plan pl;
+    if (!(!transB && smallm_applies(M, N, K)) && pad32_plan(M, N, K, transB, &pl)) return pl.total;
     if (!transB && smallm_applies(M, N, K)) return gemm_smallm_workspace_bytes(M, N, K);
     if (!transB && skinny32_applies(M, N, K)) return (size_t)skinny32_ksplit(N, K) * M * N * sizeof(float);
     const int ks = splitk32_ranges(M, N, K);
@@ -2005,7 +2049,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
-            const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % (8 * E) == 0;
+            const bool exact_fit = g.M % 64 == 0 && g.N % 64 == 0 && g.K % (8 * E) == 0 && g.c_cols == 0;
             if constexpr (E == 4 && !TRANSB) {
                 // about one tile per CU: the eight-wave form (two k-step groups), so that every SIMD has a second wave to switch to
                 if (exact_fit && tiles(64, 64) <= 512) return launch_gemm_dl<T, OutT, false, 64, TRANSB, 2>(g, batch, stream);
@@ -2019,7 +2063,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
             if (Elem<OutT>::BYTES != 4 && (g.alpha != 1.0f || g.beta != 0.0f)) return hipErrorInvalidValue;
             const int edge = tile == 256 ? 256 : 128;
-            const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0;
+            const bool exact_fit = g.M % edge == 0 && g.N % edge == 0 && g.K % (8 * E) == 0 && g.c_cols == 0;
             // (bf16 output with ragged edges on the 256 x 256 tile: that one instance does not fit the register file -- the
             // compiler moves accumulators to scratch memory -- so such problems take the 128 x 128 tile)
             constexpr bool kSpills256Edge = std::is_same<T, bf16_t>::value && std::is_same<OutT, bf16_t>::value;
@@ -2036,6 +2080,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         }
     }
     if (tile == 129) tile = 128;
+    if (g.c_cols > 0) return hipErrorInvalidValue;        // only the direct-to-LDS kernels above know that C is narrower than N
     // 16-byte aligned operands whose K the K-tile divides take the instance without bounds checks in its loop (no zero fill
     // is needed; rows and column blocks past the end are clamped loads whose products are never stored)
     auto exact = [&](int bt) { return vec && g.N >= E && g.K % (gemm_k_chunks(bt, bt) * E) == 0; };
@@ -2065,6 +2110,19 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
     if (force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
         return launch_smallm<false>(g, stream, (float*)workspace);
+    Pad32Plan pl;
+    if (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && (pl.Kp != K || aligned16(A))) {
+        unsigned char* w = (unsigned char*)workspace;
+        const float* Ap = A;
+        if (pl.Kp != K) {
+            if (hipError_t e = pad_rows(stream, A, w + pl.a_off, M, K, M, pl.Kp, 4)) return e;
+            Ap = (const float*)(w + pl.a_off);
+        }
+        if (hipError_t e = transB ? pad_rows(stream, B, w + pl.b_off, N, K, N, pl.Kp, 4) : pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 4)) return e;
+        GemmArgs gp{Ap, w + pl.b_off, C, M, pl.Np, pl.Kp, pl.Kp, transB ? pl.Kp : pl.Np, N, 0, 0, 0, alpha, beta, 0, 0, bias, act, act_param};
+        if (pl.Np != N) gp.c_cols = N;
+        return transB ? dispatch_gemm<float, float, true>(gp, 1, stream, 0) : dispatch_gemm<float, float, false>(gp, 1, stream, 0);
+    }
     if (force_tile == 0 && workspace && !transB && batch == 1 && skinny32_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         int ks;
         const int kper = 32 * skinny_plan(N / 128, K / 32, &ks);

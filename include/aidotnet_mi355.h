@@ -77,7 +77,9 @@ AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream);
  * and fp16-weight entry points below.  With 9 <= M <= 32 (B [K,N], N a multiple of 128, K a multiple of 32) the weight matrix is
  * likewise streamed once, through a 32-row MFMA kernel, and larger products whose tiles would not fill the chip over a long K
  * (K >= 1024, K a multiple of 32, either layout of B) run their K ranges side by side; both keep fp32 partials in the context
- * workspace and sum them in range order, so results are repeatable run to run (this entry point and the bias/activation one). */
+ * workspace and sum them in range order, so results are repeatable run to run (this entry point and the bias/activation one).
+ * Rows that are not whole 16-byte chunks (K, or N with B [K,N], not a multiple of 4): a product of some size is computed from
+ * zero-padded copies of A and B in the workspace (same sums; C is written in place). */
 AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const float* B, float* C,
                      int M, int N, int K, float alpha, float beta, int transB);
 

@@ -22,7 +22,9 @@ SHAPES = [(1, 1, 1), (7, 13, 11), (96, 130, 80), (37, 53, 71), (13, 10, 17), (4,
           (1, 64, 1), (64, 64, 32), (65, 63, 33), (128, 128, 64), (129, 127, 65), (256, 256, 64), (200, 300, 100),
           (32, 4096, 128), (8, 512, 1030), (512, 512, 512),
           # ragged M / N with a K the K-tile divides: the branch-free loop with clamped loads
-          (200, 300, 128), (129, 132, 256), (1000, 1000, 256), (65, 8, 512)]
+          (200, 300, 128), (129, 132, 256), (1000, 1000, 256), (65, 8, 512),
+          # rows that are not whole 16-byte chunks, large enough for the padded operand copies (odd N, odd K, both; B in either layout)
+          (300, 301, 299), (512, 1001, 300), (700, 1024, 77), (130, 2050, 258), (2049, 515, 70)]
 
 
 @pytest.fixture(scope="module")
@@ -84,6 +86,26 @@ def test_sgemm_alpha_beta_and_poisoned_output(be):
     host = big.cpu().numpy()
     assert np.array_equal(host[:M * N].reshape(M, N), oracle.sgemm(a, b, M, K, N))
     assert np.isnan(host[M * N:]).all()
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 301, 299), (640, 1001, 300), (520, 1024, 77)])
+def test_sgemm_unaligned_rows_alpha_beta_guard_band_and_epilogue(be, M, N, K):
+    # odd N / K on padded operand copies: alpha / beta read and write the caller's C in place, the elements after the matrix
+    # stay untouched, bias and activation are taken from the unpadded bias
+    rng = np.random.default_rng(M + N + K)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4); c0 = dyadic(rng, (M, N), hi=4)
+    want = oracle.sgemm(a, b, M, K, N, threads=4)
+    for transB in (False, True):
+        bm = np.ascontiguousarray(b.T) if transB else b
+        c = torch.full(((M + 1) * N,), -7.0, device="cuda"); c[:M * N] = dev(c0).reshape(-1)
+        (be.MatMulTransposed if transB else be.Gemm)(be.WrapTensor(dev(a)), be.WrapTensor(dev(bm)), be.WrapTensor(c), M, N, K, 0.5, 2.0)
+        assert np.array_equal(c[:M * N].cpu().numpy().reshape(M, N), np.float32(0.5) * want + np.float32(2.0) * c0), transB
+        assert bool((c[M * N:] == -7.0).all()), transB
+    bias = dyadic(rng, (N,), hi=8)
+    c = torch.full(((M + 1) * N,), -7.0, device="cuda")
+    be.GemmBiasActivationInto(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(dev(bias)), be.WrapTensor(c), M, N, K, 1)
+    assert np.array_equal(c[:M * N].cpu().numpy().reshape(M, N), np.maximum(want + bias[None, :], 0.0))
+    assert bool((c[M * N:] == -7.0).all())
 
 
 def test_sgemm_identity_known_answer(be):
