@@ -28,6 +28,17 @@
 
 namespace aidn {
 
+// f(std::integral_constant<int, I>) for I = BEGIN, BEGIN + STEP, ... < END: a loop the compiler cannot leave rolled (register
+// arrays indexed by the loop variable need constant indices)
+template <int BEGIN, int END, int STEP, typename F>
+__device__ __forceinline__ void static_for(F&& f)
+{
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + STEP, END, STEP>(f);
+    }
+}
+
 struct GemmArgs {
     const void* A; const void* B; void* C;
     int M, N, K;
@@ -1124,8 +1135,9 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
             if (g.bias) bias4[j] = *(const f32x4*)(g.bias + n0 + wn * WTN + 16 * j + 4 * g4);
         }
         unsigned char* Cw = (unsigned char*)g.C + (bz * g.sC + (long long)(m0 + wm * WTM) * g.ldc + n0 + wn * WTN) * OB;
-#pragma unroll
-        for (int ip = 0; ip < TI; ip += IPR) {
+        const bool whole_tile = __builtin_amdgcn_readfirstlane(m0 + (HALF ? 128 : 256) <= g.M && g.c_cols == 0);
+        static_for<0, TI, IPR>([&](auto ip_const) {
+            constexpr int ip = decltype(ip_const)::value;
 #pragma unroll
             for (int ii = 0; ii < IPR; ii++) {
 #pragma unroll
@@ -1147,13 +1159,29 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                     }
                 }
             }
+            // a workgroup whose tile lies inside the matrix (every one but the last tile row of a ragged M) stores without a
+            // test per row: with the test the compiler serialises LDS read and store of every chunk, which costs the short-K
+            // shapes 3-5 %
+            if (whole_tile) {
 #pragma unroll
-            for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
-                const int u = q * 64 + lane;
-                const int row = u / CPR, c = u % CPR;
-                const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
-                u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
-                if (m0 + wm * WTM + ip * 16 + row < g.M) {
+                for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
+                    const int u = q * 64 + lane;
+                    const int row = u / CPR, c = u % CPR;
+                    const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
+                    u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
+                    if constexpr (NTS) __builtin_nontemporal_store(v, dst);
+                    else *dst = v;
+                }
+            } else {
+                // (a rolled loop: nothing in it is indexed by q at compile time, and unrolled it grows the epilogue so much that
+                // the compiler stops unrolling the loop over ip, whose accumulator indices must be constants)
+#pragma unroll 1
+                for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
+                    const int u = q * 64 + lane;
+                    const int row = u / CPR, c = u % CPR;
+                    const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
+                    u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
+                    if (m0 + wm * WTM + ip * 16 + row >= g.M) continue;
                     if (g.c_cols > 0) {
                         // rows of C at any element offset: whole chunks by one under-aligned 16-byte store, the chunk that
                         // crosses the last column by elements
@@ -1170,11 +1198,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                                     else ((out_t*)dst)[e] = v[e];
                                 }
                         }
-                    } else if constexpr (NTS) __builtin_nontemporal_store(v, dst);
-                    else *dst = v;
+                    } else *dst = v;
                 }
             }
-        }
+        });
     }
 }
 
