@@ -1395,16 +1395,72 @@ static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &k
 // Split-K for 16-bit problems whose 128 x 128 tiles fill less than half the chip over a long K (M <= 512 against a 4096-wide
 // weight): K ranges run as the batch dimension of the 128 x 128 kernel into fp32 partials, summed in range order by
 // skinny_reduce_kernel (deterministic; bias and activation there).  Returns the number of ranges, 0 = not worth it.
-static int splitk16_ranges(int M, int N, int K)
+static int dl16_width(int M, int N, int K, int batch, double* score_out = nullptr);
+// Share of a split-K product's time that is the product: the fp32 partials are written and read once per range, 8 bytes per output
+// element and range at about 4 TB/s, against 2 K flops per element at about 1.4 PFLOP/s (512 x 8192 x 8192 in four ranges: 49 us of
+// product, 33 us of partials)
+static double splitk16_partials_factor(int K, int ks) { return 1.0 / (1.0 + 1000.0 * ks / K); }
+static int splitk16_ranges(int M, int N, int K, int* big_tile = nullptr)
 {
-    if (M % 128 != 0 || N % 128 != 0 || K % 64 != 0) return 0;
-    const long long t = (long long)(M / 128) * (N / 128);
-    if (t > 128) return 0;                    // up to half a chip of tiles
-    int ks = (int)(256 / t);
-    if (ks > 16) ks = 16;
-    while (ks > 1 && (K % (ks * 64) != 0 || K / ks < 512)) ks--;
-    // the partials cost 8 bytes of traffic per output element and range; the product must be worth it
-    return ks >= 2 && (long long)K >= 1024 ? ks : 0;
+    if (big_tile) *big_tile = 0;
+    if (N % 128 != 0 || K % 64 != 0) return 0;
+    auto ranges = [&](long long t, int min_k) {
+        int ks = (int)(256 / t);
+        if (ks > 16) ks = 16;
+        while (ks > 1 && (K % (ks * 64) != 0 || K / ks < min_k)) ks--;
+        return ks;
+    };
+    // (a ragged M: the last tile row is partial)
+    const long long t = (long long)((M + 127) / 128) * (N / 128);
+    if (t <= 128) {                           // up to half a chip of 128 x 128 tiles
+        const int ks = ranges(t, 512);
+        // the partials cost 8 bytes of traffic per output element and range; the product must be worth it
+        // (a ragged M only from K = 2048 on: below, the second launch costs what the ranges save -- 1000 x 1024 x 1024 8 -> 15 us)
+        return ks >= 2 && (long long)K >= (M % 128 == 0 ? 1024 : 2048) ? ks : 0;
+    }
+    // Larger problems whose 256 x 256 tiles still fill at most half the chip over a long K (M about 1000 against an 8192-wide
+    // weight with K = 28672): narrower tiles would fill the chip but move twice the operand bytes per flop through the L2, which
+    // is what bounds them at this K; K ranges of the 256 x 256 tile keep its traffic.
+    if (N % 256 != 0) return 0;
+    const long long t256 = (long long)((M + 255) / 256) * (N / 256);
+    if (t256 > 128 || K < 4096) return 0;
+    const int ks = ranges(t256, 2048);
+    if (ks < 2 || !big_tile) return 0;
+    // against the best single launch, by the scores of the tile choice (CU fill x rate per flop x share of real rows)
+    double single = 0.0;
+    dl16_width(M, N, K, 1, &single);
+    const double split = cu_fill(t256 * ks) * ((double)M / (double)(((M + 255) / 256) * 256)) * splitk16_partials_factor(K, ks);
+    if (split <= 1.05 * single) return 0;
+    *big_tile = 1;
+    return ks;
+}
+
+// Rows of a tall 16-bit problem to run as a launch of their own: with N / 256 tile columns that divide the 256 CUs, whole rounds of
+// 256 x 256 tiles cover a multiple of 256 * 256 / (N / 256) rows at the full rate; the rows that would start a partly filled round
+// (3000 rows against an 8192-wide weight: 1.5 rounds) are better served by whatever suits them alone -- narrower tiles, or K
+// ranges of the 256 x 256 tile.  Returns the row count of the first launch, 0 = one launch.  Both estimates are rows / score.
+static int msplit16_rows(int M, int N, int K)
+{
+    if (N % 256 != 0 || K % 64 != 0 || 256 % (N / 256) != 0) return 0;
+    const int rows_per_round = 256 / (N / 256) * 256;
+    const int first = M / rows_per_round * rows_per_round;
+    const int rest = M - first;
+    if (first == 0 || rest == 0) return 0;
+    auto score = [&](int m) {
+        double single = 0.0;
+        dl16_width(m, N, K, 1, &single);
+        int big = 0;
+        const int ks = splitk16_ranges(m, N, K, &big);
+        if (ks && big) {
+            const long long t256 = (long long)((m + 255) / 256) * (N / 256);
+            const double split = cu_fill(t256 * ks) * ((double)m / (double)(((m + 255) / 256) * 256)) * splitk16_partials_factor(K, ks);
+            if (split > single) single = split;
+        }
+        return single;
+    };
+    const double whole = score(M), tail = score(rest);
+    if (whole <= 0.0 || tail <= 0.0) return 0;
+    return (double)first + (double)rest / tail < 0.92 * (double)M / whole ? first : 0;
 }
 
 // 16-bit problems whose rows are not 16-byte aligned (N or K not a multiple of 8) would run on 2-byte loads, an order of
@@ -1419,7 +1475,12 @@ struct PadPlan {
 static size_t gemm_16_inner_workspace_bytes(int M, int N, int K)
 {
     if (skinny_applies(M, N, K)) return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
-    const int ks = splitk16_ranges(M, N, K);
+    if (const int first = msplit16_rows(M, N, K)) {
+        const size_t a = gemm_16_inner_workspace_bytes(first, N, K), b = gemm_16_inner_workspace_bytes(M - first, N, K);
+        return a > b ? a : b;
+    }
+    int big;
+    const int ks = splitk16_ranges(M, N, K, &big);
     return ks ? (size_t)ks * M * N * sizeof(float) : 0;
 }
 static bool pad16_plan(int M, int N, int K, PadPlan* pl)
@@ -1989,8 +2050,9 @@ static bool dl16_applies(const GemmArgs& g)
 // narrower tile moves more A bytes per flop (and the 256 x 128 one wastes half of its B loads); the 128 x 128 tile runs at about
 // 0.55 and the 64 x 64 tile at about 0.45 of the 256 x 256 rate (2048^3: 128 tiles of 256 x 128 take 36 us, 256 tiles of 128 x 128 29 us).
 #define DL16_HALF_EFF 0.7
-static int dl16_width(int M, int N, int K, int batch)
+static int dl16_width(int M, int N, int K, int batch, double* score_out)
 {
+    if (score_out) *score_out = 0.0;
     if (K % 64 != 0) return 0;
     // M may be ragged (the last tile row is partial: clamped loads, guarded stores); the rows a tile height pads count as waste
     const long long tm256 = (M + 255) / 256, tm128 = (M + 127) / 128, tm64 = (M + 63) / 64;
@@ -2010,7 +2072,9 @@ static int dl16_width(int M, int N, int K, int batch)
     const long long t64 = tm64 * ((N + 63) / 64) * batch;
     // the 128 x 128 tile of this kernel (code 1): whole column tiles only
     if (N % 128 == 0 && DL16_HALF_EFF * cu_fill(t128) * use128 > best_score) { best_score = DL16_HALF_EFF * cu_fill(t128) * use128; best = 1; }
-    if (0.55 * cu_fill(t128) * use128 > best_score || 0.45 * cu_fill(t64) * use64 > best_score) return 0;
+    const double s128 = 0.55 * cu_fill(t128) * use128, s64 = 0.45 * cu_fill(t64) * use64;
+    if (score_out) *score_out = best_score > s128 ? (best_score > s64 ? best_score : s64) : (s128 > s64 ? s128 : s64);
+    if (s128 > best_score || s64 > best_score) return 0;
     return best;
 }
 
@@ -2244,15 +2308,24 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
         float* ws = (float*)workspace;
         return out32 ? launch_skinny<T, float>(g, stream, ws) : launch_skinny<T, T>(g, stream, ws);
     }
+    if (force_tile == 0 && dl16_applies<float>(g)) {
+        if (const int first = msplit16_rows(M, N, K)) {
+            // the rows of the whole rounds, then the rest (stream order; the two share the workspace one after the other)
+            if (hipError_t e = gemm_16_typed<T>(stream, A, B, C, out32, first, N, K, 0, workspace, bias, act, act_param)) return e;
+            return gemm_16_typed<T>(stream, A + (size_t)first * K, B, (unsigned char*)C + (size_t)first * N * (out32 ? 4 : 2), out32, M - first, N, K, 0,
+                                    workspace, bias, act, act_param);
+        }
+    }
     if (force_tile == 0 && workspace) {
-        const int ks = splitk16_ranges(M, N, K);
+        int big = 0;
+        const int ks = splitk16_ranges(M, N, K, &big);
         if (ks) {
             GemmArgs gp = g;
             gp.C = workspace; gp.K = K / ks; gp.ldc = N;
             gp.sA = K / ks; gp.sB = (long long)(K / ks) * N; gp.sC = (long long)M * N;
             gp.bias = nullptr; gp.act = 0;
             if (dl16_applies<float>(gp)) {
-                if (hipError_t e = launch_gemm_dl16<T, float, 2, true>(gp, ks, stream)) return e;
+                if (hipError_t e = big ? launch_gemm_dl16<T, float, 4>(gp, ks, stream) : launch_gemm_dl16<T, float, 2, true>(gp, ks, stream)) return e;
                 const long long total = (long long)M * N;
                 const unsigned grid = (unsigned)((total + 255) / 256);
                 if (out32) hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)workspace, C, M, N, ks, bias, act, act_param, 1.0f, 0.0f);

@@ -336,6 +336,29 @@ def test_half_gemm_unaligned_rows_guard_band_odd_operand_offsets_and_epilogue(be
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("M,N,K", [(1224, 16384, 64), (3000, 8192, 64),          # whole rounds of 256 x 256 tiles, then the rest as its own launch
+                                   (1000, 8192, 4096), (384, 8192, 8192),         # K ranges of the 256 x 256 tile (2 and 4)
+                                   (1000, 768, 3072), (200, 1024, 2048)])         # K ranges of the 128 x 128 tile under a ragged M
+def test_half_gemm_row_split_and_k_ranges_sampled_rows_exact(be, kind, M, N, K):
+    # dyadic inputs: every summation order gives the same fp32 bits, so sampled rows must equal the float64 product exactly
+    rng = np.random.default_rng(M + N + K)
+    a = dyadic(rng, (M, K), hi=4); b = dyadic(rng, (K, N), hi=4)
+    ab, aw = round_to(a, kind); bb, bw = round_to(b, kind)
+    rows = np.unique(np.r_[0:3, 127:130, 255:258, M // 2, M - 3:M, np.arange(1023, M, 1024), np.arange(1024, M, 1024), np.arange(2047, M, 2048)])
+    rows = rows[rows < M]
+    truth = (aw[rows].astype(np.float64) @ bw.astype(np.float64)).astype(np.float32)
+    got32 = _half_gemm(be, kind, ab, bb, M, N, K, True)
+    assert np.array_equal(got32[rows], truth)
+    assert np.isfinite(got32).all()
+    got16 = _half_gemm(be, kind, ab, bb, M, N, K, False)
+    narrow = oracle.f32_to_f16 if kind == "f16" else oracle.f32_to_bf16
+    assert np.array_equal(got16[rows], narrow(truth).reshape(truth.shape))
+    # every row, cheaply: the column sums of C equal (column sums of A) B
+    colsum = aw.astype(np.float64).sum(axis=0) @ bw.astype(np.float64)
+    assert np.array_equal(got32.astype(np.float64).sum(axis=0), colsum)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
 def test_half_gemm_ragged_large_shape_takes_the_large_tile(be, kind):
     # 3000 x 3080 x 512: 156 tiles of 256 x 256, chosen automatically; sampled rows against the float64 truth
     M, N, K = 3000, 3080, 512
