@@ -1894,8 +1894,15 @@ __global__ __launch_bounds__(256, 1) void gemm_skinny32_kernel(const GemmArgs g,
 {
     const long long wg = (long long)((M + tile - 1) / tile) * ((N + tile - 1) / tile) * batch * ks;
     const double rounds = wg <= 2048 ? (double)((wg + 255) / 256) : (double)wg / 256.0 + 0.5;
-    const double eff = tile == 64 ? 0.75 : 0.88;
-    const double tile_us = 2.0 * tile * tile * (double)(K / ks) / (0.614e6 * eff) + 1.5;
+    // the 64 x 64 tile comes close to the rate of the larger ones once several workgroups share a CU (3000 x 4096 x 4096: 3008 tiles
+    // at 0.88 of the pipe; with operands beyond the caches its doubled traffic per flop costs a few per cent), and 0.75 with one
+    // per CU, where a lone wave per SIMD overlaps nothing
+    const double eff = tile == 64 ? (wg >= 1024 ? 0.85 : wg >= 512 ? 0.80 : 0.75) : 0.88;
+    double tile_us = 2.0 * tile * tile * (double)(K / ks) / (0.614e6 * eff) + 1.5;
+    // measured, not understood: the 128 x 128 instance with edge handling takes 922 us where the plain one takes 721 us on 768
+    // tiles (M = 2945..3071 against 3072, N = K = 4096; one ragged row is enough), 3 % more on 256 tiles (M = 1023) and nothing
+    // extra on 1536 tiles (3000 x 8192 x 8192); the 64 x 64 instance shows no such step
+    if (tile == 128 && (M % 128 != 0 || N % 128 != 0)) tile_us *= wg > 512 && wg <= 1024 ? 1.25 : 1.03;
     double t = rounds * tile_us;
     if (ks > 1) t += 3.0 + (double)(ks + 2) * M * N * 4.0 / 3.0e6;
     return t;
