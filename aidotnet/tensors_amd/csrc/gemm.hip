@@ -1237,19 +1237,20 @@ static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 // ---------------------------------------------------------------------------------------------
 // Skinny-M path (decode projections): M <= 32, 16-bit, B stored [K,N], N % 128 == 0, K % 64 == 0.
 // HBM-bound: B (K x N) is read exactly once.  grid = (N / 128, KS), about one workgroup per CU: each workgroup streams a
-// 128-column slab of B over its K range with the direct global->LDS load through a ring of SKINNY_STAGES 20 KB stages, filled
-// SKINNY_STAGES - 1 K-tiles ahead (120 KB in flight per CU: one memory round trip covers a whole K range of up to six tiles,
-// where a two-stage ring paid one round trip per tile), computes a 32 x 128 partial product on MFMA (A rows beyond M are
+// 128-column slab of B over its K range with the direct global->LDS load through a ring of NS 20 KB stages, filled NS - 1
+// K-tiles ahead -- seven stages and one workgroup per CU (120 KB in flight per CU: one memory round trip covers a whole K range of
+// up to six tiles, where a two-stage ring paid one round trip per tile), or three stages and two workgroups per CU for wide
+// weights (launch_skinny) --, computes a 32 x 128 partial product on MFMA (A rows beyond M are
 // clamped duplicates that are never stored) and writes it to an fp32 workspace that skinny_reduce_kernel sums in split order
 // (deterministic) and narrows.  Loads complete in issue order, so "tile kt has landed" is a count of younger loads.
 //   B tile [64 k][256 B]: chunk c of row k at position c ^ ((k & 3) << 2)   (transposing reads)
 //   A tile [32 m][128 B]: chunk c of row m at position c ^ ((m >> 1) & 7)   (b128 reads)
 #define SKINNY_STAGES 7
-template <typename T>
-__global__ __launch_bounds__(256, 1) void gemm_skinny_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
+template <typename T, int NS>
+__global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_skinny_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
 {
     typedef uint16_t raw_t;
-    constexpr int BK = 64, NS = SKINNY_STAGES, AHEAD = NS - 1;
+    constexpr int BK = 64, AHEAD = NS - 1;
     constexpr int ABYTES = 32 * 128, BBYTES = BK * 256, STAGE = ABYTES + BBYTES;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];      // NS stages
 
@@ -1375,22 +1376,27 @@ static double cu_fill(long long tiles) { return (double)tiles / (double)(((tiles
 // K ranges of the skinny paths: `tiles` K-tiles over `slabs` column slabs, one workgroup per CU at a time.  Returns the K-tiles per
 // range (the last range may be shorter); *ks = number of ranges.  Scored as (how evenly slabs x ranges load the 256 CUs) x (the
 // share of a workgroup's time that is not its first memory round trip, about three K-tiles' worth).
-static int skinny_plan(int slabs, int tiles, int* ks_out)
+static int skinny_plan(int slabs, int tiles, int* ks_out, int per_cu = 1, double* score_out = nullptr)
 {
     int best_kper = tiles, best_ks = 1;
     double best = -1.0;
+    const long long slots = 256LL * per_cu;
+    // (two workgroups per CU: one's first round trip runs under the other's stream, so it counts half)
+    const double ramp = per_cu == 1 ? 3.0 : 1.5;
     for (int ks = 1; ks <= 32 && ks <= tiles; ks++) {
         const int kper = (tiles + ks - 1) / ks;
         const int kse = (tiles + kper - 1) / kper;
         if (kper < 4 && ks > 1) break;
         const long long wg = (long long)slabs * kse;
-        const double score = cu_fill(wg) * (double)kper / (kper + 3.0);
+        const double fill = (double)wg / (double)(((wg + slots - 1) / slots) * slots);
+        const double score = fill * (double)kper / (kper + ramp);
         if (score > best * 1.02) { best = score; best_kper = kper; best_ks = kse; }
     }
     *ks_out = best_ks;
+    if (score_out) *score_out = best;
     return best_kper;
 }
-static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &ks); return ks; }
+static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &ks, N / 128 > 64 ? 2 : 1); return ks; }
 
 // Split-K for 16-bit problems whose 128 x 128 tiles fill less than half the chip over a long K (M <= 512 against a 4096-wide
 // weight): K ranges run as the batch dimension of the 128 x 128 kernel into fp32 partials, summed in range order by
@@ -1669,11 +1675,22 @@ template <typename T, typename OutT>
 static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
 {
     int ks;
-    const int kper = 64 * skinny_plan(g.N / 128, g.K / 64, &ks);
-    constexpr int smem = SKINNY_STAGES * (32 * 128 + 64 * 256);
-    static unsigned long long attr_done = 0;
-    if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny_kernel<T>, smem, &attr_done)) return e0;
-    hipLaunchKernelGGL((gemm_skinny_kernel<T>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), smem, stream, g, ws, ks, kper);
+    // more than 64 column slabs: the three-stage form, two workgroups per CU (a workgroup's first memory round trip and its last
+    // tiles run under the other's stream: 32 x 11008 x 4096 24.5 -> 22.9 us, 32 x 128256 x 4096 193 -> 187 us); with fewer slabs the
+    // K ranges of that plan get too short (32 x 4096 x 4096 12.3 -> 14.1 us) and the seven-stage form, one per CU, stays
+    const bool three = g.N / 128 > 64;
+    const int kper = 64 * skinny_plan(g.N / 128, g.K / 64, &ks, three ? 2 : 1);
+    if (three) {
+        constexpr int smem = 3 * (32 * 128 + 64 * 256);
+        static unsigned long long attr_done3 = 0;
+        if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny_kernel<T, 3>, smem, &attr_done3)) return e0;
+            hipLaunchKernelGGL((gemm_skinny_kernel<T, 3>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), smem, stream, g, ws, ks, kper);
+    } else {
+        constexpr int smem = SKINNY_STAGES * (32 * 128 + 64 * 256);
+        static unsigned long long attr_done = 0;
+        if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny_kernel<T, SKINNY_STAGES>, smem, &attr_done)) return e0;
+        hipLaunchKernelGGL((gemm_skinny_kernel<T, SKINNY_STAGES>), dim3((unsigned)(g.N / 128), (unsigned)ks), dim3(256), smem, stream, g, ws, ks, kper);
+    }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     long long total = (long long)g.M * g.N;
@@ -1790,7 +1807,7 @@ __global__ __launch_bounds__(256) void gemm_smallm_kernel(const GemmArgs g, floa
 // ---------------------------------------------------------------------------------------------
 // Skinny-M fp32 path: 9 <= M <= 32, B stored [K,N], N % 128 == 0, K % 32 == 0 -- the fp32 form of gemm_skinny_kernel.
 // HBM-bound: B is read exactly once.  grid = (N / 128, KS); a workgroup streams a 128-column slab of B over its K range through
-// the same ring of SKINNY_STAGES 20 KB stages (32 k-rows of 512 bytes of B and 32 rows of 128 bytes of A per stage, five
+// a ring of NS (three: two workgroups per CU) 20 KB stages (32 k-rows of 512 bytes of B and 32 rows of 128 bytes of A per stage, five
 // direct-to-LDS loads per wave and K-tile), each wave multiplies the 32 x 32 block of its 32 columns on the fp32 MFMA (a 64-row
 // tile of the general kernel would spend three quarters of its matrix work on padding and run at a quarter of the memory rate)
 // and stores the partial product for skinny_reduce_kernel.
@@ -1798,9 +1815,10 @@ __global__ __launch_bounds__(256) void gemm_smallm_kernel(const GemmArgs g, floa
 //   A tile [32 m][128 B]: chunk c of row m at position c ^ ((m >> 1) & 7)          (b128 reads)
 // The k index of MFMA step i of 8-k group j is 8 j + 4 h + i for both operands (h = lane half).
 #if AIDN_GEMM_PART == 0
-__global__ __launch_bounds__(256, 1) void gemm_skinny32_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
+template <int NS>
+__global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_skinny32_kernel(const GemmArgs g, float* __restrict__ ws, int ksplit, int kper)
 {
-    constexpr int BK = 32, NS = SKINNY_STAGES, AHEAD = NS - 1;
+    constexpr int BK = 32, AHEAD = NS - 1;
     constexpr int ABYTES = 32 * 128, BBYTES = BK * 512, STAGE = ABYTES + BBYTES;
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];      // NS stages
 
@@ -1882,7 +1900,12 @@ __global__ __launch_bounds__(256, 1) void gemm_skinny32_kernel(const GemmArgs g,
 
 [[maybe_unused]] static bool skinny32_applies(int M, int N, int K) { return M > 8 && M <= 32 && N % 128 == 0 && K % 32 == 0 && N >= 128; }
 
-[[maybe_unused]] static int skinny32_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 32, &ks); return ks; }
+// The fp32 skinny kernel runs a three-stage ring, two workgroups per CU: a workgroup's first memory round trip and its last tiles
+// run under the other's stream (against seven stages and one per CU: 16 x 8192 x 8192 57.3 -> 48.3 us, 16 x 28672 x 8192 204 -> 171 us,
+// 16 x 11008 x 4096 50.3 -> 41.1 us, 16 x 4096 x 4096 20.1 -> 18.4 us).  K-tiles per range; *ks ranges.
+#define SKINNY32_STAGES 3
+[[maybe_unused]] static int skinny32_plan(int N, int K, int* ks) { return skinny_plan(N / 128, K / 32, ks, 2); }
+[[maybe_unused]] static int skinny32_ksplit(int N, int K) { int ks; skinny32_plan(N, K, &ks); return ks; }
 
 // fp32: estimated run time (microseconds) of the direct-to-LDS kernel with `tile` x `tile` tiles when K is cut into `ks` ranges
 // that run as batches.  A CU works through its tiles at the same total rate whether it holds one or two at a time, so the time
@@ -2223,11 +2246,11 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
     }
     if (force_tile == 0 && workspace && !transB && batch == 1 && skinny32_applies(M, N, K) && aligned16(A) && aligned16(B)) {
         int ks;
-        const int kper = 32 * skinny_plan(N / 128, K / 32, &ks);
-        constexpr int smem = SKINNY_STAGES * (32 * 128 + 32 * 512);
+        const int kper = 32 * skinny32_plan(N, K, &ks);
+        constexpr int smem = SKINNY32_STAGES * (32 * 128 + 32 * 512);
         static unsigned long long attr_done = 0;
-        if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny32_kernel, smem, &attr_done)) return e0;
-        hipLaunchKernelGGL(gemm_skinny32_kernel, dim3((unsigned)(N / 128), (unsigned)ks), dim3(256), smem, stream, g, (float*)workspace, ks, kper);
+        if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny32_kernel<SKINNY32_STAGES>, smem, &attr_done)) return e0;
+        hipLaunchKernelGGL(gemm_skinny32_kernel<SKINNY32_STAGES>, dim3((unsigned)(N / 128), (unsigned)ks), dim3(256), smem, stream, g, (float*)workspace, ks, kper);
         if (hipError_t e = hipGetLastError()) return e;
         const long long total = (long long)M * N;
         hipLaunchKernelGGL((skinny_reduce_kernel<float>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (const float*)workspace,
