@@ -404,9 +404,9 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
 {
     Ctx* c = (Ctx*)ctx;
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
-    if (tile != 0 && tile != 64 && tile != 65 && tile != 128 && tile != 129 && tile != 130 && tile != 192 && tile != 193 && tile != 256)
+    if (tile != 0 && tile != 64 && tile != 65 && tile != 128 && tile != 129 && tile != 130 && tile != 131 && tile != 192 && tile != 193 && tile != 256)
         return fail(c, AIDN_ERR_INVALID_ARGUMENT, "tile must be 0, 64, 65 (64, direct-to-LDS kernel), 128, 129 (128, direct-to-LDS kernel), "
-                                                  "130 (128 x 128, 16-bit 16x16x32 kernel), 192 (256 x 192, 16-bit), 193 (256 x 128, 16-bit) or 256");
+                                                  "130 / 131 (128 x 128, 16-bit 16x16x32 kernel, four- / two-stage ring), 192 (256 x 192, 16-bit), 193 (256 x 128, 16-bit) or 256");
     c->force_tile = tile;
     return AIDN_OK;
 }

@@ -899,7 +899,7 @@ template <> struct Mma16<bf16_t> {
 #define DL16_HALF_STAGES 4
 // NTS: C is written with non-temporal stores (a compile-time switch: as a run-time branch the two stores are merged by the compiler
 // and the hint is lost).
-template <typename T, typename OutT, int TJ = 4, bool HALF = false, bool NTS = false>
+template <typename T, typename OutT, int TJ = 4, bool HALF = false, bool NTS = false, int HS = DL16_HALF_STAGES>
 __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 {
     static_assert(!HALF || TJ == 2, "the 128-row tile is built for 128 columns");
@@ -995,10 +995,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
 #pragma unroll
         for (int j = 0; j < TJ; j++) acc[i][j] = f32x4_acc{0.0f, 0.0f, 0.0f, 0.0f};
 
-    constexpr int NS = HALF ? DL16_HALF_STAGES : 2;
+    constexpr int NS = HALF ? HS : 2;
     // wait until at most `tiles` of this wave's tile loads (LA + LB instructions each) are outstanding, and for its LDS reads
     auto wait_tiles = [&](int tiles) {
-        static_assert(!HALF || (LA + LB == 4 && NS == 4), "the wait counts below are for four loads per tile and a four-stage ring");
+        static_assert(!HALF || (LA + LB == 4 && NS <= 4), "the wait counts below are for four loads per tile and a four-stage ring");
         if (tiles <= 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else if (tiles == 1) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
@@ -1205,10 +1205,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
     }
 }
 
-template <typename T, typename OutT, int TJ = 4, bool HALF = false>
+template <typename T, typename OutT, int TJ = 4, bool HALF = false, int HS = DL16_HALF_STAGES>
 static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
 {
-    constexpr int smem = HALF ? DL16_HALF_STAGES * (128 * 128 + 64 * 256) : 2 * (256 * 128 + 128 * 256);
+    constexpr int smem = HALF ? HS * (128 * 128 + 64 * 256) : 2 * (256 * 128 + 128 * 256);
     g.tiles_m = (g.M + (HALF ? 127 : 255)) / (HALF ? 128 : 256);      // the last tile row may be partial
     g.tiles_n = g.N / (64 * TJ);
     const dim3 grid((unsigned)(g.tiles_m * g.tiles_n), 1, (unsigned)batch);
@@ -1227,7 +1227,7 @@ static hipError_t launch_gemm_dl16(GemmArgs g, int batch, hipStream_t stream)
             return hipGetLastError();
         }
     }
-    auto kern = gemm_dl16_kernel<T, OutT, TJ, HALF, false>;
+    auto kern = gemm_dl16_kernel<T, OutT, TJ, HALF, false, HS>;
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     hipLaunchKernelGGL(kern, grid, dim3(512), smem, stream, g);
@@ -1396,7 +1396,7 @@ static int skinny_plan(int slabs, int tiles, int* ks_out, int per_cu = 1, double
     if (score_out) *score_out = best;
     return best_kper;
 }
-static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &ks, N / 128 > 64 ? 2 : 1); return ks; }
+static int skinny_ksplit(int N, int K) { int ks; skinny_plan(N / 128, K / 64, &ks, N / 128 > 64 && K <= 4096 ? 2 : 1); return ks; }
 
 // Split-K for 16-bit problems whose 128 x 128 tiles fill less than half the chip over a long K (M <= 512 against a 4096-wide
 // weight): K ranges run as the batch dimension of the 128 x 128 kernel into fp32 partials, summed in range order by
@@ -1675,10 +1675,10 @@ template <typename T, typename OutT>
 static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
 {
     int ks;
-    // more than 64 column slabs: the three-stage form, two workgroups per CU (a workgroup's first memory round trip and its last
+    // more than 64 column slabs over a K of at most 4096 (16 x 28672 x 8192 went 77 -> 88 us): the three-stage form, two workgroups per CU (a workgroup's first memory round trip and its last
     // tiles run under the other's stream: 32 x 11008 x 4096 24.5 -> 22.9 us, 32 x 128256 x 4096 193 -> 187 us); with fewer slabs the
     // K ranges of that plan get too short (32 x 4096 x 4096 12.3 -> 14.1 us) and the seven-stage form, one per CU, stays
-    const bool three = g.N / 128 > 64;
+    const bool three = g.N / 128 > 64 && g.K <= 4096;
     const int kper = 64 * skinny_plan(g.N / 128, g.K / 64, &ks, three ? 2 : 1);
     if (three) {
         constexpr int smem = 3 * (32 * 128 + 64 * 256);
@@ -2080,6 +2080,7 @@ static bool dl16_applies(const GemmArgs& g)
 // narrower tile moves more A bytes per flop (and the 256 x 128 one wastes half of its B loads); the 128 x 128 tile runs at about
 // 0.55 and the 64 x 64 tile at about 0.45 of the 256 x 256 rate (2048^3: 128 tiles of 256 x 128 take 36 us, 256 tiles of 128 x 128 29 us).
 #define DL16_HALF_EFF 0.7
+#define DL16_HALF2_EFF 0.82
 static int dl16_width(int M, int N, int K, int batch, double* score_out)
 {
     if (score_out) *score_out = 0.0;
@@ -2102,6 +2103,17 @@ static int dl16_width(int M, int N, int K, int batch, double* score_out)
     const long long t64 = tm64 * ((N + 63) / 64) * batch;
     // the 128 x 128 tile of this kernel (code 1): whole column tiles only
     if (N % 128 == 0 && DL16_HALF_EFF * cu_fill(t128) * use128 > best_score) { best_score = DL16_HALF_EFF * cu_fill(t128) * use128; best = 1; }
+    // the same tile on a two-stage ring, two workgroups per CU (code 5): with more tiles than CUs and a K of at most 6144 one
+    // workgroup's first loads, barrier waits and store phase run under the other's MFMAs (8192 x 768 x 3072 50.4 -> 41.8 us,
+    // 512 x 12288 x 4096 64.8 -> 54.4 us, 384 x 13824 x 5120 79.8 -> 65.8 us); one tile per CU (2048^3 20.7 -> 27.6 us) and long K
+    // (384 x 28672 x 8192 228 -> 265 us) need the deeper ring
+    // (beyond one round of 512 resident workgroups only when the last round is nearly full: a workgroup alone on its CU has nothing
+    // to hide the two-stage ring's waits behind -- 3000 x 4096 x 4096, 768 tiles: 83 -> 106 us)
+    const double fill2 = (double)t128 / (double)(((t128 + 511) / 512) * 512);
+    if (N % 128 == 0 && t128 > 256 && K <= 6144 && (t128 <= 512 || fill2 >= 0.85)) {
+        const double s2 = DL16_HALF2_EFF * (t128 <= 512 ? cu_fill(t128) : fill2) * use128;
+        if (s2 > best_score) { best_score = s2; best = 5; }
+    }
     const double s128 = 0.55 * cu_fill(t128) * use128, s64 = 0.45 * cu_fill(t64) * use64;
     if (score_out) *score_out = best_score > s128 ? (best_score > s64 ? best_score : s64) : (s128 > s64 ? s128 : s64);
     if (s128 > best_score || s64 > best_score) return 0;
@@ -2133,6 +2145,7 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
                         if (w == 3) return launch_gemm_dl16<T, OutT, 3>(g, batch, stream);
                         if (w == 2) return launch_gemm_dl16<T, OutT, 2>(g, batch, stream);
                         if (w == 1) return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
+                        if (w == 5) return launch_gemm_dl16<T, OutT, 2, true, 2>(g, batch, stream);
                     }
                 }
                 if constexpr (E == 4) {
@@ -2160,12 +2173,16 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
         }
     }
     if constexpr (E == 8 && !TRANSB) {
+        if (tile == 131) {                                // the same on the two-stage ring (two workgroups per CU)
+            if (!(g.N % 128 == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
+            return launch_gemm_dl16<T, OutT, 2, true, 2>(g, batch, stream);
+        }
         if (tile == 130) {                                // 128 x 128 tiles of the 16 x 16 x 32 kernel (whole tiles only)
             if (!(g.N % 128 == 0 && g.K % 64 == 0 && dl16_applies<OutT>(g))) return hipErrorInvalidValue;
             return launch_gemm_dl16<T, OutT, 2, true>(g, batch, stream);
         }
     }
-    if (tile == 192 || tile == 193 || tile == 130) return hipErrorInvalidValue;
+    if (tile == 192 || tile == 193 || tile == 130 || tile == 131) return hipErrorInvalidValue;
     if constexpr (E == 4 || !TRANSB) {
         if (tile == 65) {                                 // 64 x 64 tiles on the direct-to-LDS kernel
             if (!(vec && (TRANSB || g.N >= E) && g.lda < (1 << 21) && g.ldb < (1 << 21))) return hipErrorInvalidValue;
@@ -2327,6 +2344,7 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
             if (wd == 3) return out32 ? launch_gemm_dl16<T, float, 3>(gp, 1, stream) : launch_gemm_dl16<T, T, 3>(gp, 1, stream);
             if (wd == 2) return out32 ? launch_gemm_dl16<T, float, 2>(gp, 1, stream) : launch_gemm_dl16<T, T, 2>(gp, 1, stream);
             if (wd == 1) return out32 ? launch_gemm_dl16<T, float, 2, true>(gp, 1, stream) : launch_gemm_dl16<T, T, 2, true>(gp, 1, stream);
+            if (wd == 5) return out32 ? launch_gemm_dl16<T, float, 2, true, 2>(gp, 1, stream) : launch_gemm_dl16<T, T, 2, true, 2>(gp, 1, stream);
         }
         void* Cp = padC ? (void*)(w + pl.c_off) : C;
         if (hipError_t e = gemm_16_typed<T>(stream, Ap, (const uint16_t*)(w + pl.b_off), Cp, out32, M, pl.Np, pl.Kp, 0,

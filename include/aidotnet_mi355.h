@@ -300,8 +300,8 @@ AIDN_API int aidn_mi355_mha_fwd_packed_bf16(void* ctx, void* stream, const uint1
                                    const float* mask, int mask_mode, uint16_t* output, int B, int S, int dModel, int heads);
 
 /* ---- test / tuning hook --------------------------------------------------------------------------------
- * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel; 192 / 193 / 130 = the 256 x 192 /
- * 256 x 128 / 128 x 128 tiles of the 16-bit 16x16x32 kernel, whole tiles only; 0 = automatic choice) for subsequent calls on this context, so the parity suite can exercise every kernel instance.  No counterpart in the
+ * Forces the GEMM tile edge (64, 128 or 256; 129 / 65 = 128 / 64 on the direct-to-LDS kernel; 192 / 193 / 130 / 131 = the 256 x 192 /
+ * 256 x 128 / 128 x 128 (four-stage ring) / 128 x 128 (two-stage ring) tiles of the 16-bit 16x16x32 kernel, whole column tiles only; 0 = automatic choice) for subsequent calls on this context, so the parity suite can exercise every kernel instance.  No counterpart in the
  * reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
 /* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast

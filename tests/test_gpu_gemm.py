@@ -338,7 +338,8 @@ def test_half_gemm_unaligned_rows_guard_band_odd_operand_offsets_and_epilogue(be
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("M,N,K", [(1224, 16384, 64), (3000, 8192, 64),          # whole rounds of 256 x 256 tiles, then the rest as its own launch
                                    (1000, 8192, 4096), (384, 8192, 8192),         # K ranges of the 256 x 256 tile (2 and 4)
-                                   (1000, 768, 3072), (200, 1024, 2048)])         # K ranges of the 128 x 128 tile under a ragged M
+                                   (1000, 768, 3072), (200, 1024, 2048),          # K ranges of the 128 x 128 tile under a ragged M
+                                   (8192, 768, 256), (2000, 2304, 192)])          # more 128 x 128 tiles than CUs over a short K: the two-stage ring
 def test_half_gemm_row_split_and_k_ranges_sampled_rows_exact(be, kind, M, N, K):
     # dyadic inputs: every summation order gives the same fp32 bits, so sampled rows must equal the float64 product exactly
     rng = np.random.default_rng(M + N + K)
@@ -548,7 +549,9 @@ def test_config2_square_8192_baseline_distribution_sampled_rows(be, kind):
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("tile,M,N,K", [(192, 256, 192, 64), (192, 512, 576, 192), (192, 256, 768, 4096), (193, 256, 128, 64),
                                         (193, 768, 384, 320), (193, 256, 640, 2048), (256, 512, 768, 128),
-                                        (130, 128, 128, 64), (130, 384, 640, 192), (130, 128, 256, 4096), (130, 1152, 384, 128)])
+                                        (130, 128, 128, 64), (130, 384, 640, 192), (130, 128, 256, 4096), (130, 1152, 384, 128),
+                                        # the 128 x 128 tile on the two-stage ring (two workgroups per CU)
+                                        (131, 128, 128, 64), (131, 384, 640, 192), (131, 128, 256, 4096), (131, 1152, 384, 128), (131, 2048, 2304, 320)])
 def test_half_gemm_16x16x32_kernel_tile_widths(be, kind, tile, M, N, K):
     # the 256 x 192, 256 x 128 and 128 x 128 tiles of the 16 x 16 x 32 kernel (codes 192 / 193 / 130) and its 256 x 256 tile, forced on small whole-tile
     # shapes: bit-exact on dyadic inputs for both output types, bias + activation epilogue, guard band, a ragged M, refusal of a ragged N
