@@ -1947,7 +1947,7 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_skinny32_kernel(con
 [[maybe_unused]] static int splitk32_ranges(int M, int N, int K)
 {
     if (K < 1024 || K % 32 != 0) return 1;
-    double best = f32_time_us(M, N, K, 1, f32_tile(M, N, K, 1, true), 1) * 0.85;
+    double best = f32_time_us(M, N, K, 1, f32_tile(M, N, K, 1, true), 1) * 0.95;
     int best_ks = 1;
     const int cand[7] = {2, 3, 4, 6, 8, 12, 16};
     for (int i = 0; i < 7; i++) {
