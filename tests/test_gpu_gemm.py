@@ -24,7 +24,7 @@ SHAPES = [(1, 1, 1), (7, 13, 11), (96, 130, 80), (37, 53, 71), (13, 10, 17), (4,
           # ragged M / N with a K the K-tile divides: the branch-free loop with clamped loads
           (200, 300, 128), (129, 132, 256), (1000, 1000, 256), (65, 8, 512),
           # rows that are not whole 16-byte chunks, large enough for the padded operand copies (odd N, odd K, both; B in either layout)
-          (300, 301, 299), (512, 1001, 300), (700, 1024, 77), (130, 2050, 258), (2049, 515, 70)]
+          (300, 301, 299), (512, 1001, 300), (700, 1024, 77), (130, 2050, 258), (2049, 515, 70), (70000, 20, 131)]
 
 
 @pytest.fixture(scope="module")
@@ -339,7 +339,8 @@ def test_half_gemm_unaligned_rows_guard_band_odd_operand_offsets_and_epilogue(be
 @pytest.mark.parametrize("M,N,K", [(1224, 16384, 64), (3000, 8192, 64),          # whole rounds of 256 x 256 tiles, then the rest as its own launch
                                    (1000, 8192, 4096), (384, 8192, 8192),         # K ranges of the 256 x 256 tile (2 and 4)
                                    (1000, 768, 3072), (200, 1024, 2048),          # K ranges of the 128 x 128 tile under a ragged M
-                                   (8192, 768, 256), (2000, 2304, 192)])          # more 128 x 128 tiles than CUs over a short K: the two-stage ring
+                                   (8192, 768, 256), (2000, 2304, 192),           # more 128 x 128 tiles than CUs over a short K: the two-stage ring
+                                   (70000, 24, 257), (300, 70001, 40)])           # padded copies with more rows / dword columns than one grid pass covers
 def test_half_gemm_row_split_and_k_ranges_sampled_rows_exact(be, kind, M, N, K):
     # dyadic inputs: every summation order gives the same fp32 bits, so sampled rows must equal the float64 product exactly
     rng = np.random.default_rng(M + N + K)
