@@ -24,7 +24,7 @@ SHAPES = [(1, 1, 1), (7, 13, 11), (96, 130, 80), (37, 53, 71), (13, 10, 17), (4,
           # ragged M / N with a K the K-tile divides: the branch-free loop with clamped loads
           (200, 300, 128), (129, 132, 256), (1000, 1000, 256), (65, 8, 512),
           # rows that are not whole 16-byte chunks, large enough for the padded operand copies (odd N, odd K, both; B in either layout)
-          (300, 301, 299), (512, 1001, 300), (700, 1024, 77), (130, 2050, 258), (2049, 515, 70), (70000, 20, 131)]
+          (300, 301, 299), (512, 1001, 300), (700, 1024, 77), (130, 2050, 258), (2049, 515, 70), (70000, 20, 131), (600, 301, 299), (40, 1030, 1027)]
 
 
 @pytest.fixture(scope="module")
@@ -175,10 +175,11 @@ HALF_SHAPES = [(4, 32, 8), (16, 24, 20), (3, 5, 7), (1, 64, 1), (96, 96, 96), (7
                (128, 512, 1024), (256, 1024, 4096), (384, 1152, 1536), (512, 2048, 1024),
                # a ragged M on the 16 x 16 x 32 kernel (last tile row partial; 256-, 192- and 128-wide tiles, and the 128 x 128 one)
                (1000, 4096, 128), (300, 3072, 192), (700, 1920, 64), (3000, 384, 256), (1, 256, 64 * 3), (257, 2048, 128),
-               # rows that are not whole 16-byte chunks (odd N and / or K), large enough to be copied into padded operands: narrow N
+               # rows that are not whole 16-byte chunks (odd N and / or K): read in place by element-aligned 16-byte loads (few rows over a
+               # short K) or copied into padded operands: narrow N
                # (padded C, copied back), wide N (the kernel stores the real columns), odd K only, skinny and split-K inner problems
                (300, 301, 299), (512, 1001, 300), (1000, 1025, 130), (2049, 2051, 70), (700, 1024, 77), (16, 1001, 515), (256, 1100, 1030),
-               (130, 4099, 257)]
+               (130, 4099, 257), (600, 301, 299), (16, 1001, 1100), (40, 4099, 1027)]
 
 
 def _half_gemm(be, kind, abits, bbits, M, N, K, out32):
