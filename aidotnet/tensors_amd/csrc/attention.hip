@@ -56,6 +56,13 @@ __device__ __forceinline__ u32x4 ld16(const typename Raw2<T>::type* p, int valid
     u32x4 v = {0u, 0u, 0u, 0u};
     if (valid <= 0) return v;
     if (vec && valid >= Elem<T>::PER16) return *(const u32x4*)p;
+    if (valid >= Elem<T>::PER16) {
+        // rows off the 16-byte grid: a whole chunk is still one load, only element-aligned (the hardware takes such loads)
+        typedef u32x4 u32x4_a4 __attribute__((aligned(4)));
+        typedef u32x4 u32x4_a2 __attribute__((aligned(2)));
+        if constexpr (Elem<T>::BYTES == 4) return *(const u32x4_a4*)p;
+        else return *(const u32x4_a2*)p;
+    }
     if constexpr (Elem<T>::BYTES == 4) {
 #pragma unroll
         for (int e = 0; e < 4; e++) if (e < valid) v[e] = p[e];
