@@ -328,6 +328,50 @@ class Mi355Backend:
                        1 if outputIsFp32 else 0, m, n, k, int(activation), float(alpha)))
         self._done()
 
+    # ------------------------------------------------------------------ pre-packed weight operand
+    _PACK_KIND = {"f32": 0, "f16": 1, "bf16": 2}
+
+    def PackB(self, kind: str, B: GpuBuffer, K: int, N: int, transB: bool = False) -> GpuBuffer:
+        """Packs a weight matrix once for GemmPackedB -- the GPU form of the reference's cached packed B
+        (``SimdGemm.SgemmWithCachedB`` / ``PrePackedB``, src/AiDotNet.Tensors/Engines/Simd/SimdGemm.cs:327-684, 1030-1159).
+        Returns a byte buffer the caller owns; repack when the weight changes."""
+        if kind not in self._PACK_KIND:
+            raise NotSupportedException("PackB: kind must be 'f32', 'f16' or 'bf16'")
+        self._need(B, "B"); self._positive(K=K, N=N)
+        es = 4 if kind == "f32" else 2
+        self._capacity(B, K * N * es, "B", "PackB")
+        nbytes = int(self._lib.aidn_mi355_packed_b_bytes(self._PACK_KIND[kind], K, N, 1 if transB else 0))
+        if nbytes <= 0:
+            raise NotSupportedException("PackB: no packed layout for this kind / shape")
+        packed = self.AllocateByteBuffer(nbytes)
+        self._check(self._lib.aidn_mi355_pack_b(self._ctx, self._stream(), self._PACK_KIND[kind], B.Handle, K, N,
+                                                1 if transB else 0, packed.Handle))
+        self._done()
+        return packed
+
+    def GemmPackedB(self, kind: str, A: GpuBuffer, packedB: GpuBuffer, bias: Optional[GpuBuffer], C: GpuBuffer,
+                    M: int, N: int, K: int, transB: bool = False, activation: int = 0, alpha: float = 0.0,
+                    outputIsFp32: bool = True) -> None:
+        """C = act(A * B + bias) with B given as PackB's result; the values are those of the plain GEMM entry points."""
+        if kind not in self._PACK_KIND:
+            raise NotSupportedException("GemmPackedB: kind must be 'f32', 'f16' or 'bf16'")
+        op = "GemmPackedB"
+        self._need(A, "A"); self._need(packedB, "packedB"); self._need(C, "C")
+        self._positive(M=M, N=N, K=K)
+        es = 4 if kind == "f32" else 2
+        out32 = True if kind == "f32" else bool(outputIsFp32)
+        self._capacity(A, M * K * es, "A", op); self._capacity(C, M * N * (4 if out32 else 2), "C", op)
+        nbytes = int(self._lib.aidn_mi355_packed_b_bytes(self._PACK_KIND[kind], K, N, 1 if transB else 0))
+        if nbytes <= 0:
+            raise NotSupportedException("GemmPackedB: no packed layout for this kind / shape")
+        self._capacity(packedB, nbytes, "packedB", op)
+        if bias is not None:
+            self._capacity(bias, N * 4, "bias", op)
+        self._check(self._lib.aidn_mi355_gemm_packed_b(self._ctx, self._stream(), self._PACK_KIND[kind], A.Handle, packedB.Handle,
+                                                       bias.Handle if bias is not None else None, C.Handle, 1 if out32 else 0,
+                                                       M, N, K, 1 if transB else 0, int(activation), float(alpha)))
+        self._done()
+
     # ------------------------------------------------------------------ rotary position embedding
     def RopeInterleaved(self, input: GpuBuffer, cos: GpuBuffer, sin: GpuBuffer, output: GpuBuffer,
                         rows: int, headDim: int, seqLen: int, startPosition: int, kind: str = "f32") -> None:

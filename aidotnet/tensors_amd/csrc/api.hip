@@ -494,6 +494,51 @@ AIDN_API int aidn_mi355_bf16gemm_bias_act(void* ctx, void* stream, const uint16_
                                  int out_is_f32, int M, int N, int K, int activation, float act_param)
 { return gemm16_common(ctx, stream, 1, A, B, C, out_is_f32 != 0, M, N, K, bias, activation, act_param); }
 
+// ---- pre-packed weight operand: kind 0 fp32 (B [K,N], or [N,K] with transB), 1 fp16, 2 bf16 (B [K,N])
+AIDN_API uint64_t aidn_mi355_packed_b_bytes(int kind, int K, int N, int transB)
+{
+    if (kind == 0) return aidn::gemm_f32_packed_b_bytes(N, K, transB != 0);
+    if ((kind == 1 || kind == 2) && !transB) return aidn::gemm_16_packed_b_bytes(N, K);
+    return 0;
+}
+AIDN_API int aidn_mi355_pack_b(void* ctx, void* stream, int kind, const void* B, int K, int N, int transB, void* packed)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!B || !packed) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "pack_b: B and packed must not be null");
+    if (K <= 0 || N <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "pack_b: dimensions must be positive");
+    if (kind < 0 || kind > 2 || (kind != 0 && transB)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "pack_b: kind 0 (fp32), 1 (fp16) or 2 (bf16); transB only for fp32");
+    if (aidn_mi355_packed_b_bytes(kind, K, N, transB) == 0) return fail(c, AIDN_ERR_UNSUPPORTED, "pack_b: dimensions beyond the packed layout");
+    if ((((uintptr_t)packed) & 15u) != 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "pack_b: packed must be 16-byte aligned");
+    if (kind == 0) return hip_status(c, aidn::gemm_f32_pack_b((hipStream_t)stream, (const float*)B, K, N, transB != 0, packed), "pack_b");
+    return hip_status(c, aidn::gemm_16_pack_b((hipStream_t)stream, (const uint16_t*)B, K, N, packed), "pack_b");
+}
+AIDN_API int aidn_mi355_gemm_packed_b(void* ctx, void* stream, int kind, const void* A, const void* packedB, const float* bias, void* C,
+                             int out_is_f32, int M, int N, int K, int transB, int activation, float act_param)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !packedB || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: A, packedB and C must not be null");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: dimensions must be positive");
+    if (kind < 0 || kind > 2 || (kind != 0 && transB)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: kind 0 (fp32), 1 (fp16) or 2 (bf16); transB only for fp32");
+    if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: unknown activation");
+    if (aidn_mi355_packed_b_bytes(kind, K, N, transB) == 0) return fail(c, AIDN_ERR_UNSUPPORTED, "gemm_packed_b: dimensions beyond the packed layout");
+    if (((((uintptr_t)packedB) | ((uintptr_t)C)) & 15u) != 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: packedB and C must be 16-byte aligned");
+    void* ws = nullptr;
+    const size_t need = kind == 0 ? aidn::gemm_f32_packed_workspace_bytes(M, N, K, transB != 0) : aidn::gemm_16_packed_workspace_bytes(M, N, K);
+    if (kind != 0 && need == 0) return fail(c, AIDN_ERR_UNSUPPORTED, "gemm_packed_b: problem beyond the 4 GiB workspace limit");
+    if (need) {
+        if (int st = acquire_ws(c, stream, need, &ws)) return st;       // (a stream under capture must have it reserved: B itself is not at hand)
+    }
+    if (kind == 0) {
+        if ((((uintptr_t)A) & 15u) != 0 && K % 32 == 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: A must be 16-byte aligned");
+        return hip_status(c, aidn::gemm_f32((hipStream_t)stream, (const float*)A, nullptr, (float*)C, M, N, K, 1.0f, 0.0f, transB != 0, 1, 0, 0, 0, 0,
+                                            bias, activation, act_param, ws, (const float*)packedB), "gemm_f32 (packed B)");
+    }
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind - 1, (const uint16_t*)A, nullptr, C, out_is_f32 != 0, M, N, K, 0, ws, bias, activation,
+                                       act_param, (const uint16_t*)packedB), "gemm_16 (packed B)");
+}
+
 AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K)
 { return gemm16_common(ctx, stream, 0, A, B, C, 1, M, N, K); }
 AIDN_API int aidn_mi355_hgemm_f16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K)

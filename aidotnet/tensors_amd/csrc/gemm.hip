@@ -56,6 +56,8 @@ struct GemmArgs {
     int c_cols = 0;
 };
 
+[[maybe_unused]] static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
+
 #if AIDN_GEMM_PART == 0
 hipError_t ensure_dynamic_smem(const void* kernel, int bytes, unsigned long long* done_mask)
 {
@@ -1497,13 +1499,9 @@ static size_t gemm_16_inner_workspace_bytes(int M, int N, int K)
     const int ks = splitk16_ranges(M, N, K, &big);
     return ks ? (size_t)ks * M * N * sizeof(float) : 0;
 }
-static bool pad16_plan(int M, int N, int K, PadPlan* pl)
+// the padded shapes and the workspace layout for them (no judgement on whether padding pays)
+static bool pad16_layout(int M, int N, int K, PadPlan* pl)
 {
-    if (N % 8 == 0 && K % 8 == 0) return false;
-    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;        // launch-bound either way
-    // few rows over a short K: the copy of B would cost more than the product; the general kernel reads such rows in place with
-    // element-aligned 16-byte loads (64 x 50257 x 768: 42 us against 51 us through the copies)
-    if (M <= 512 && K <= 1024) return false;
     const int Np = N >= 512 ? (N + 127) / 128 * 128 : (N + 7) / 8 * 8;
     const int Kp = (K + 63) / 64 * 64;
     auto up = [](size_t b) { return (b + 255) & ~(size_t)255; };
@@ -1516,6 +1514,15 @@ static bool pad16_plan(int M, int N, int K, PadPlan* pl)
     pl->inner_off = off; off += gemm_16_inner_workspace_bytes(M, Np, Kp);
     pl->total = off;
     return off <= ((size_t)4 << 30);
+}
+static bool pad16_plan(int M, int N, int K, PadPlan* pl)
+{
+    if (N % 8 == 0 && K % 8 == 0) return false;
+    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;        // launch-bound either way
+    // few rows over a short K: the copy of B would cost more than the product; the general kernel reads such rows in place with
+    // element-aligned 16-byte loads (64 x 50257 x 768: 42 us against 51 us through the copies)
+    if (M <= 512 && K <= 1024) return false;
+    return pad16_layout(M, N, K, pl);
 }
 
 // dst [rows_dst, cols_dst] (16-byte aligned rows) <- src [rows_src, cols_src] (dense, any alignment), zeros elsewhere; E = element.
@@ -1679,6 +1686,25 @@ size_t gemm_16_workspace_bytes(int M, int N, int K)
     PadPlan pl;
     if (pad16_plan(M, N, K, &pl)) return pl.total;
     return gemm_16_inner_workspace_bytes(M, N, K);
+}
+// Pre-packed B (the caller keeps it): B [K,N] zero-padded to [Kp, Np] -- the copy that an unaligned product otherwise makes on every
+// call, made once.  An aligned weight is packed the same way (its K and N padded to whole tiles).
+size_t gemm_16_packed_b_bytes(int N, int K)
+{
+    PadPlan pl;
+    if (N <= 0 || K <= 0 || !pad16_layout(1, N, K, &pl)) return 0;
+    return (size_t)pl.Kp * pl.Np * 2;
+}
+hipError_t gemm_16_pack_b(hipStream_t stream, const uint16_t* B, int K, int N, void* packed)
+{
+    PadPlan pl;
+    if (!pad16_layout(1, N, K, &pl) || !aligned16(packed)) return hipErrorInvalidValue;
+    return pad_rows(stream, B, packed, K, N, pl.Kp, pl.Np, 2);
+}
+size_t gemm_16_packed_workspace_bytes(int M, int N, int K)
+{
+    PadPlan pl;
+    return pad16_layout(M, N, K, &pl) ? pl.total : 0;
 }
 #endif
 
@@ -1997,11 +2023,8 @@ size_t gemm_smallm_workspace_bytes(int M, int N, int K)
 // in the workspace (K up to a multiple of 32, N up to a multiple of 4) feed the direct-to-LDS kernel, whose element stores put the N
 // real columns straight into the caller's C.  Same sums as the plain product: the padding contributes exact zeros.
 struct Pad32Plan { int Np, Kp; size_t a_off, b_off, total; };
-static bool pad32_plan(int M, int N, int K, int transB, Pad32Plan* pl)
+static bool pad32_layout(int M, int N, int K, int transB, Pad32Plan* pl)
 {
-    if (K % 4 == 0 && (transB || N % 4 == 0)) return false;
-    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;
-    if (M <= 512 && K <= 1024) return false;          // as for 16-bit: the general kernel reads the rows in place
     pl->Kp = (K + 31) / 32 * 32;
     pl->Np = transB ? N : (N + 3) / 4 * 4;
     if (pl->Kp >= (1 << 21) || pl->Np >= (1 << 21)) return false;
@@ -2010,6 +2033,33 @@ static bool pad32_plan(int M, int N, int K, int transB, Pad32Plan* pl)
     pl->b_off = up((size_t)M * pl->Kp * 4);
     pl->total = pl->b_off + up((size_t)(transB ? N : pl->Kp) * (transB ? pl->Kp : pl->Np) * 4);
     return pl->total <= ((size_t)4 << 30);
+}
+static bool pad32_plan(int M, int N, int K, int transB, Pad32Plan* pl)
+{
+    if (K % 4 == 0 && (transB || N % 4 == 0)) return false;
+    if (N < 16 || (double)M * N * K < (double)(1 << 21)) return false;
+    if (M <= 512 && K <= 1024) return false;          // as for 16-bit: the general kernel reads the rows in place
+    return pad32_layout(M, N, K, transB, pl);
+}
+
+// Pre-packed fp32 B (the caller keeps it): [K,N] zero-padded to [Kp, Np], or [N,K] to [N, Kp] -- the GPU form of the reference's
+// cached packed weight operand (SimdGemm.SgemmWithCachedB / PrePackedB): packed once, the product is that of the plain call.
+size_t gemm_f32_packed_b_bytes(int N, int K, int transB)
+{
+    Pad32Plan pl;
+    if (N <= 0 || K <= 0 || !pad32_layout(1, N, K, transB, &pl)) return 0;
+    return (size_t)(transB ? N : pl.Kp) * (transB ? pl.Kp : pl.Np) * 4;
+}
+hipError_t gemm_f32_pack_b(hipStream_t stream, const float* B, int K, int N, int transB, void* packed)
+{
+    Pad32Plan pl;
+    if (!pad32_layout(1, N, K, transB, &pl) || !aligned16(packed)) return hipErrorInvalidValue;
+    return transB ? pad_rows(stream, B, packed, N, K, N, pl.Kp, 4) : pad_rows(stream, B, packed, K, N, pl.Kp, pl.Np, 4);
+}
+size_t gemm_f32_packed_workspace_bytes(int M, int N, int K, int transB)
+{
+    Pad32Plan pl;
+    return pad32_layout(M, N, K, transB, &pl) ? pl.b_off : 0;         // the padded copy of A only
 }
 
 size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB)
@@ -2065,7 +2115,6 @@ static hipError_t launch_gemm(GemmArgs g, int batch, hipStream_t stream)
     return hipGetLastError();
 }
 
-static bool aligned16(const void* p) { return (((uintptr_t)p) & 15u) == 0; }
 
 
 // 128 x 128 or 64 x 64 tile; rel64 = efficiency per flop of the smaller tile relative to the larger one when both load the
@@ -2256,21 +2305,28 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
 #if AIDN_GEMM_PART == 0
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile, const float* bias, int act, float act_param, void* workspace)
+                    int force_tile, const float* bias, int act, float act_param, void* workspace, const float* Bpre)
 {
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
-    if (force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
+    if (!Bpre && force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
         return launch_smallm<false>(g, stream, (float*)workspace);
+    // Bpre: B already packed by gemm_f32_pack_b (B itself is then not read); such a call always takes the padded shapes
     Pad32Plan pl;
-    if (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && (pl.Kp != K || aligned16(A))) {
+    if (Bpre && !(batch == 1 && aligned16(Bpre) && pad32_layout(M, N, K, transB, &pl) && (pl.Kp == K ? aligned16(A) : (workspace && aligned16(workspace)))))
+        return hipErrorInvalidValue;
+    if (Bpre || (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && (pl.Kp != K || aligned16(A)))) {
         unsigned char* w = (unsigned char*)workspace;
         const float* Ap = A;
         if (pl.Kp != K) {
             if (hipError_t e = pad_rows(stream, A, w + pl.a_off, M, K, M, pl.Kp, 4)) return e;
             Ap = (const float*)(w + pl.a_off);
         }
-        if (hipError_t e = transB ? pad_rows(stream, B, w + pl.b_off, N, K, N, pl.Kp, 4) : pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 4)) return e;
-        GemmArgs gp{Ap, w + pl.b_off, C, M, pl.Np, pl.Kp, pl.Kp, transB ? pl.Kp : pl.Np, N, 0, 0, 0, alpha, beta, 0, 0, bias, act, act_param};
+        const void* Bp = Bpre;
+        if (!Bpre) {
+            if (hipError_t e = transB ? pad_rows(stream, B, w + pl.b_off, N, K, N, pl.Kp, 4) : pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 4)) return e;
+            Bp = w + pl.b_off;
+        }
+        GemmArgs gp{Ap, Bp, C, M, pl.Np, pl.Kp, pl.Kp, transB ? pl.Kp : pl.Np, N, 0, 0, 0, alpha, beta, 0, 0, bias, act, act_param};
         if (pl.Np != N) gp.c_cols = N;
         return transB ? dispatch_gemm<float, float, true>(gp, 1, stream, 0) : dispatch_gemm<float, float, false>(gp, 1, stream, 0);
     }
@@ -2331,10 +2387,13 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
 // one 16-bit type per part: T = f16_t in part 1, bf16_t in part 2; out32: C is fp32 (else the same 16-bit type as the inputs)
 template <typename T>
 static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                                int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+                                int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param,
+                                const uint16_t* Bpre = nullptr)
 {
+    // Bpre: B already packed by gemm_16_pack_b (B itself is then not read); such a call always takes the padded shapes
     PadPlan pl;
-    if (force_tile == 0 && workspace && aligned16(C) && aligned16(workspace) && pad16_plan(M, N, K, &pl)) {
+    if (Bpre && !(workspace && aligned16(C) && aligned16(workspace) && aligned16(Bpre) && pad16_layout(M, N, K, &pl))) return hipErrorInvalidValue;
+    if (Bpre || (force_tile == 0 && workspace && aligned16(C) && aligned16(workspace) && pad16_plan(M, N, K, &pl))) {
         unsigned char* w = (unsigned char*)workspace;
         const bool padA = pl.Kp != K, padC = pl.Np != N;
         const uint16_t* Ap = A;
@@ -2342,7 +2401,11 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
             if (hipError_t e = pad_rows(stream, A, w + pl.a_off, M, K, M, pl.Kp, 2)) return e;
             Ap = (const uint16_t*)(w + pl.a_off);
         }
-        if (hipError_t e = pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 2)) return e;
+        const uint16_t* Bp = Bpre;
+        if (!Bpre) {
+            if (hipError_t e = pad_rows(stream, B, w + pl.b_off, K, N, pl.Kp, pl.Np, 2)) return e;
+            Bp = (const uint16_t*)(w + pl.b_off);
+        }
         const float* bp = bias;
         if (bias && padC) {
             if (hipError_t e = pad_rows(stream, bias, w + pl.bias_off, 1, N, 1, pl.Np, 4)) return e;
@@ -2350,9 +2413,9 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
         }
         if (padC && pl.Np % 128 == 0 && pl.Kp < (1 << 21) && pl.Np < (1 << 21)) {
             // the 16 x 16 x 32 kernel stores the N real columns straight into the caller's C
-            GemmArgs gp{Ap, w + pl.b_off, C, M, pl.Np, pl.Kp, pl.Kp, pl.Np, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bp, act, act_param};
+            GemmArgs gp{Ap, Bp, C, M, pl.Np, pl.Kp, pl.Kp, pl.Np, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bp, act, act_param};
             gp.c_cols = N;
-            const int wd = dl16_width(M, pl.Np, pl.Kp, 1);
+            const int wd = aligned16(Ap) ? dl16_width(M, pl.Np, pl.Kp, 1) : 0;
             if (wd == 4) return out32 ? launch_gemm_dl16<T, float, 4>(gp, 1, stream) : launch_gemm_dl16<T, T, 4>(gp, 1, stream);
             if (wd == 3) return out32 ? launch_gemm_dl16<T, float, 3>(gp, 1, stream) : launch_gemm_dl16<T, T, 3>(gp, 1, stream);
             if (wd == 2) return out32 ? launch_gemm_dl16<T, float, 2>(gp, 1, stream) : launch_gemm_dl16<T, T, 2>(gp, 1, stream);
@@ -2360,7 +2423,7 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
             if (wd == 5) return out32 ? launch_gemm_dl16<T, float, 2, true, 2>(gp, 1, stream) : launch_gemm_dl16<T, T, 2, true, 2>(gp, 1, stream);
         }
         void* Cp = padC ? (void*)(w + pl.c_off) : C;
-        if (hipError_t e = gemm_16_typed<T>(stream, Ap, (const uint16_t*)(w + pl.b_off), Cp, out32, M, pl.Np, pl.Kp, 0,
+        if (hipError_t e = gemm_16_typed<T>(stream, Ap, Bp, Cp, out32, M, pl.Np, pl.Kp, 0,
                                             pl.total > pl.inner_off ? (void*)(w + pl.inner_off) : nullptr, bp, act, act_param)) return e;
         return padC ? unpad_rows(stream, Cp, C, M, N, pl.Np, out32 ? 4 : 2) : hipSuccess;
     }
@@ -2400,24 +2463,24 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
 }
 
 hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param);
+                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre);
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param);
+                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre);
 #if AIDN_GEMM_PART == 1
 hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
-{ return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param); }
+                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
+{ return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre); }
 #elif AIDN_GEMM_PART == 2
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
-{ return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param); }
+                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
+{ return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre); }
 #else
 // kind: 0 = fp16, 1 = bf16
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param)
+                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
 {
-    if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param);
-    return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param);
+    if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre);
+    return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre);
 }
 #endif
 

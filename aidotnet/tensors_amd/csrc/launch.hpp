@@ -9,7 +9,13 @@ namespace aidn {
 // act_param, 6 swish) form the fused epilogue C = act(alpha A B + beta C + bias)
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f, void* workspace = nullptr);
+                    int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f, void* workspace = nullptr,
+                    const float* Bpre = nullptr);
+// Bpre: B packed once by gemm_f32_pack_b into gemm_f32_packed_b_bytes(N, K, transB) bytes (B itself is then ignored; one batch); the
+// workspace must then hold gemm_f32_packed_workspace_bytes(M, N, K, transB) bytes
+size_t gemm_f32_packed_b_bytes(int N, int K, int transB);
+size_t gemm_f32_packed_workspace_bytes(int M, int N, int K, int transB);
+hipError_t gemm_f32_pack_b(hipStream_t stream, const float* B, int K, int N, int transB, void* packed);
 // bytes of workspace that let gemm_f32 take its small-M (M <= 8, B [K,N], one batch) or split-K path, and gemm_f32_f16weight its
 // small-M path; 0 = not applicable
 size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB);
@@ -20,9 +26,14 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
                               void* workspace = nullptr);
 // workspace: gemm_16_workspace_bytes(M, N, K) bytes (0 = none needed); without it the skinny-M path is not taken
 size_t gemm_16_workspace_bytes(int M, int N, int K);
+// Bpre: B packed once by gemm_16_pack_b into gemm_16_packed_b_bytes(N, K) bytes (B itself is then ignored); the workspace must then
+// hold gemm_16_packed_workspace_bytes(M, N, K) bytes
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
                    int M, int N, int K, int force_tile, void* workspace, const float* bias = nullptr, int act = 0,
-                   float act_param = 0.0f);
+                   float act_param = 0.0f, const uint16_t* Bpre = nullptr);
+size_t gemm_16_packed_b_bytes(int N, int K);
+size_t gemm_16_packed_workspace_bytes(int M, int N, int K);
+hipError_t gemm_16_pack_b(hipStream_t stream, const uint16_t* B, int K, int N, void* packed);
 
 // kind: 0 f32->f16, 1 f16->f32, 2 f32->bf16, 3 bf16->f32
 hipError_t convert(hipStream_t stream, int kind, const void* in, void* out, long long n);

@@ -115,6 +115,22 @@ AIDN_API int aidn_mi355_bf16gemm_bias_act(void* ctx, void* stream, const uint16_
 AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A, const uint16_t* B_f16, const float* bias, float* C,
                                int M, int N, int K, int activation, float act_param);
 
+/* ---- pre-packed weight operand -----------------------------------------------------------------------
+ * The GPU form of the reference's cached packed B (SimdGemm.SgemmWithCachedB and its PrePackedB cache, Engines/Simd/SimdGemm.cs:327-684,
+ * 1030-1159: a weight matrix is packed once into the layout the kernel wants and re-used by every later product; results are those of
+ * the plain call).  Here the packed layout is the weight zero-padded to whole tiles with 16-byte aligned rows, which is what a product
+ * whose N or K is odd (a vocabulary of 50257 columns) otherwise copies on every call.  kind: 0 fp32 (B [K,N], or [N,K] when transB != 0),
+ * 1 fp16, 2 bf16 (B [K,N], transB must be 0).  The caller owns `packed` (aidn_mi355_packed_b_bytes bytes, 16-byte aligned) and repacks
+ * when the weight changes -- no identity or content check is made here; the reference's cache keys (array identity, version,
+ * FNV-1a of the contents) are host-side bookkeeping that stays with the caller.
+ * aidn_mi355_gemm_packed_b: C[M,N] = act(A[M,K] * B + bias) with B given in packed form; 16-bit kinds store fp32 (out_is_f32 != 0) or
+ * the input type; fp32 ignores out_is_f32.  Same sums as the plain entry points (bit-identical on inputs whose partial sums are exact).
+ * Needs the stream's workspace (a padded copy of A when K is not a whole tile, split-K partials): under capture reserve it first. */
+AIDN_API uint64_t aidn_mi355_packed_b_bytes(int kind, int K, int N, int transB);
+AIDN_API int aidn_mi355_pack_b(void* ctx, void* stream, int kind, const void* B, int K, int N, int transB, void* packed);
+AIDN_API int aidn_mi355_gemm_packed_b(void* ctx, void* stream, int kind, const void* A, const void* packedB, const float* bias, void* C,
+                             int out_is_f32, int M, int N, int K, int transB, int activation, float act_param);
+
 /* ---- 16-bit GEMM, fp32 accumulation ------------------------------------------------------------
  * C[M,N] = A[M,K] * B[K,N].  *_f32out replaces IGpuHalfPrecisionBackend.GemmFp16In32fOut
  * (Engines/Gpu/IGpuHalfPrecisionBackend.cs:39-48; host HipBackend.HalfPrecision.cs:125-150,
