@@ -81,6 +81,39 @@ class Mi355Engine:
             raise ArgumentException("batched TensorMatMul needs equal leading dimensions")
         return self.BatchMatMul(a, b)
 
+    def TensorMatMulCachedB(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+        """a [..., K] times a rank-2 weight b [K, N] that is expected again: b is packed once (backend.PackB) and the packed form
+        is kept, keyed the way SimdGemm.SgemmWithCachedB keys its PrePackedB entries (SimdGemm.cs:327-684: array identity, the
+        array's version and its shape; a changed weight is packed again) -- here the tensor's storage pointer, shape, dtype and
+        torch's in-place version counter.  Values are those of TensorMatMul.  At most ``CACHED_B_CAPACITY`` weights are kept, the
+        least recently used one leaves first (the reference bounds its cache the same way, SimdGemm.cs:1030-1159)."""
+        if a is None or b is None:
+            raise ArgumentNullException("a" if a is None else "b")
+        if b.dim() != 2 or a.dim() < 1:
+            raise ArgumentException("TensorMatMulCachedB needs a rank-2 weight")
+        if a.dtype != b.dtype or a.dtype not in _KIND:
+            raise NotSupportedException("TensorMatMulCachedB: unsupported dtype combination %s x %s" % (a.dtype, b.dtype))
+        if a.shape[-1] != b.shape[0]:
+            raise ArgumentException("inner dimensions do not match: %s x %s" % (tuple(a.shape), tuple(b.shape)))
+        be = self.backend
+        a = a.contiguous(); b = b.contiguous()
+        K, N = b.shape
+        kind = _KIND[a.dtype]
+        cache = self.__dict__.setdefault("_packed_b", {})
+        key = (b.data_ptr(), K, N, b.dtype)
+        hit = cache.pop(key, None)
+        if hit is None or hit[0] != b._version:
+            hit = (b._version, be.PackB(kind, be.WrapTensor(b), K, N))
+        cache[key] = hit                                                        # most recently used last
+        while len(cache) > self.CACHED_B_CAPACITY:
+            cache.pop(next(iter(cache)))
+        M = a.numel() // K
+        out = torch.empty(*a.shape[:-1], N, dtype=a.dtype, device=a.device)
+        be.GemmPackedB(kind, be.WrapTensor(a), hit[1], None, be.WrapTensor(out), M, N, K, outputIsFp32=(a.dtype == torch.float32))
+        return out
+
+    CACHED_B_CAPACITY = 64
+
     def TensorMatMulTransposed(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """a [..., M, K] times the transpose of b stored [..., N, K] -> [..., M, N] (CpuEngine.cs:12337-12452 for the argument rules;
         DirectGpuTensorEngine.cs:19860-19905: rank 2 runs the backend's MatMulTransposed, which reads B in place with no transposed

@@ -94,3 +94,28 @@ def test_packed_b_is_reused_and_argument_errors(be):
     with pytest.raises(Exception):
         be.GemmPackedB("bf16", be.WrapTensor(torch.zeros(4 * K, dtype=torch.bfloat16, device="cuda")), small, None,
                        be.WrapTensor(torch.zeros(4 * N, device="cuda")), 4, N, K)                     # packed buffer too small
+
+
+def test_engine_cached_weight_matmul_repacks_a_changed_weight():
+    from aidotnet.tensors_amd import Mi355Engine
+    eng = Mi355Engine()
+    g = torch.Generator(device="cuda").manual_seed(3)
+    w = (torch.randint(-4, 5, (130, 1001), device="cuda", generator=g).float() / 8).bfloat16()
+    x = (torch.randint(-4, 5, (3, 7, 130), device="cuda", generator=g).float() / 8).bfloat16()
+    first = eng.TensorMatMulCachedB(x, w)
+    assert first.shape == (3, 7, 1001) and first.dtype == torch.bfloat16
+    assert torch.equal(first, eng.TensorMatMul(x, w))                       # the values of the plain product
+    assert len(eng._packed_b) == 1
+    packed_before = next(iter(eng._packed_b.values()))[1]
+    again = eng.TensorMatMulCachedB(x, w)
+    assert torch.equal(again, first) and next(iter(eng._packed_b.values()))[1] is packed_before     # packed once
+    w.mul_(2)                                                               # in place: same storage, new version
+    doubled = eng.TensorMatMulCachedB(x, w)
+    assert torch.equal(doubled.float(), 2 * first.float())
+    assert next(iter(eng._packed_b.values()))[1] is not packed_before
+    xf = x.float(); wf = w.float()
+    assert torch.equal(eng.TensorMatMulCachedB(xf, wf), eng.TensorMatMul(xf, wf))
+    assert len(eng._packed_b) == 2
+    with pytest.raises(Exception):
+        eng.TensorMatMulCachedB(x, w.float())
+    eng.backend.Dispose()
