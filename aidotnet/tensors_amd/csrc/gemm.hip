@@ -1831,7 +1831,7 @@ __global__ __launch_bounds__(256) void gemm_smallm_kernel(const GemmArgs g, floa
                     for (int e = 0; e < 4; e++) v[e] += o[e];
                 }
                 float* dst = ws + ((long long)ks * g.M + m) * g.N + n;
-                if (VEC) *(f32x4*)dst = v;
+                if (VEC && (g.N & 3) == 0) *(f32x4*)dst = v;          // (rows of B may be padded beyond an N that is no multiple of 4)
                 else {
 #pragma unroll
                     for (int e = 0; e < 4; e++) if (e < nvalid) dst[e] = v[e];
@@ -2059,7 +2059,9 @@ hipError_t gemm_f32_pack_b(hipStream_t stream, const float* B, int K, int N, int
 size_t gemm_f32_packed_workspace_bytes(int M, int N, int K, int transB)
 {
     Pad32Plan pl;
-    return pad32_layout(M, N, K, transB, &pl) ? pl.b_off : 0;         // the padded copy of A only
+    if (!pad32_layout(M, N, K, transB, &pl)) return 0;
+    const size_t small = !transB && smallm_applies(M, N, K) ? gemm_smallm_workspace_bytes(M, N, K) : 0;
+    return pl.b_off > small ? pl.b_off : small;                       // the padded copy of A, or the small-M partials
 }
 
 size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB)
@@ -2078,7 +2080,8 @@ static hipError_t launch_smallm(const GemmArgs& g, hipStream_t stream, float* ws
 {
     const int kper = smallm_kper(g.N, g.K);
     const int ks = (g.K + kper - 1) / kper;
-    const bool vec = g.N % 4 == 0 && g.ldb % 4 == 0 && (((uintptr_t)g.B) & (B16 ? 7u : 15u)) == 0;
+    // whole 16-byte loads of B: rows in 16-byte steps that hold every chunk a lane may touch (N a multiple of 4, or rows padded to one)
+    const bool vec = (g.N % 4 == 0 || g.ldb >= (g.N + 3) / 4 * 4) && g.ldb % 4 == 0 && (((uintptr_t)g.B) & (B16 ? 7u : 15u)) == 0;
     const dim3 grid((unsigned)((g.N + 255) / 256), (unsigned)ks);
     const int mr = g.M <= 1 ? 1 : g.M <= 2 ? 2 : g.M <= 4 ? 4 : 8;
 #define AIDN_SMALLM(MR_)                                                                                               \
@@ -2312,6 +2315,11 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
         return launch_smallm<false>(g, stream, (float*)workspace);
     // Bpre: B already packed by gemm_f32_pack_b (B itself is then not read); such a call always takes the padded shapes
     Pad32Plan pl;
+    if (Bpre && !transB && batch == 1 && workspace && smallm_applies(M, N, K) && aligned16(Bpre) && pad32_layout(M, N, K, 0, &pl)) {
+        GemmArgs gs = g;
+        gs.B = Bpre; gs.ldb = pl.Np;                 // the padded rows; only the first K of them are read
+        return launch_smallm<false>(gs, stream, (float*)workspace);
+    }
     if (Bpre && !(batch == 1 && aligned16(Bpre) && pad32_layout(M, N, K, transB, &pl) && (pl.Kp == K ? aligned16(A) : (workspace && aligned16(workspace)))))
         return hipErrorInvalidValue;
     if (Bpre || (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && (pl.Kp != K || aligned16(A)))) {

@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 
 # the reference's own shape, odd and even widths, few and many rows, short and long K, narrow N (padded C), wide N (direct stores)
 SHAPES = [(13, 10, 17), (64, 1001, 300), (300, 301, 299), (1000, 1025, 130), (16, 1024, 512), (700, 4099, 77), (8, 4096, 1030),
-          (2049, 2051, 70), (256, 1152, 1088), (40, 50257, 64)]
+          (2049, 2051, 70), (256, 1152, 1088), (40, 50257, 64), (4, 1001, 300), (1, 50257, 40), (8, 130, 515)]
 
 
 @pytest.fixture(scope="module")
