@@ -232,7 +232,7 @@ def main() -> int:
             return randn(*shape, kind=kind)
         return (2.0 * torch.rand(*shape, device="cuda", generator=g) - 1.0).to(dts[kind])
 
-    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False, extra=False):
+    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False, extra=False, packed=False):
         if not want(name, extra):
             return
         # rotate > 1: cycle through that many distinct weight matrices so the timed loop reads HBM, not the
@@ -243,7 +243,11 @@ def main() -> int:
         c_ = torch.empty(M, N, device="cuda", dtype=torch.float32 if (kind == "f32" or out32) else dts[kind])
         A_, C_ = W(a_), W(c_)
         Bs = [W(x) for x in bs]
-        if kind == "f32":
+        if packed:
+            # the weights packed once, outside the timed region (what a resident model does); the product reads the packed form
+            Bs = [be.PackB(kind, Bx, K, N) for Bx in Bs]
+            fn1 = lambda Bx: be.GemmPackedB(kind, A_, Bx, None, C_, M, N, K, outputIsFp32=(kind == "f32" or out32))
+        elif kind == "f32":
             fn1 = lambda Bx: be.Gemm(A_, Bx, C_, M, N, K)
         elif kind == "f16":
             fn1 = (lambda Bx: be.GemmFp16In32fOut(A_, Bx, C_, M, N, K)) if out32 else (lambda Bx: be.Hgemm(A_, Bx, C_, M, N, K))
@@ -263,7 +267,7 @@ def main() -> int:
             roof["note"] = "%d weight matrices rotated to defeat the last-level cache" % rotate
         else:
             roof = _roof_flops(kind, fl, ms_, TRAFFIC_BYTES.get(name))
-        add(name, kind, "GEMM M=%d N=%d K=%d%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else ""), ms_, roof, st_)
+        add(name, kind, "GEMM M=%d N=%d K=%d%s%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else "", " (pre-packed B)" if packed else ""), ms_, roof, st_)
 
     def attn_case(name, kind, Bn, H, S, D, extra=False):
         if not want(name, extra):
@@ -318,6 +322,9 @@ def main() -> int:
     decode_case("decode_f32_gqa", "f32", 32, 32, 4096, 128, Hkv=8, extra=True)
     gemm_case("gemm_f32_m16", "f32", 16, 4096, 4096, hbm=True, rotate=6, extra=True)
     gemm_case("gemm_f32_m128", "f32", 128, 4096, 4096, extra=True)
+    # an output projection onto a vocabulary of odd width (rows of B off the 16-byte grid), plain and with the weight packed once
+    gemm_case("gemm_bf16_vocab50257", "bf16", 64, 50257, 768, hbm=True, rotate=6, extra=True)
+    gemm_case("gemm_bf16_vocab50257_packed", "bf16", 64, 50257, 768, hbm=True, rotate=6, extra=True, packed=True)
     attn_case("attn_f32_prefill_b32", "f32", 32, 12, 512, 64, extra=True)
     out["others"] = others
 
