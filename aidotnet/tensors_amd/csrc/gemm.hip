@@ -1959,9 +1959,11 @@ __global__ __launch_bounds__(256, NS <= 3 ? 2 : 1) void gemm_skinny32_kernel(con
     // per CU, where a lone wave per SIMD overlaps nothing
     const double eff = tile == 64 ? (wg >= 1024 ? 0.85 : wg >= 512 ? 0.80 : 0.75) : 0.88;
     double tile_us = 2.0 * tile * tile * (double)(K / ks) / (0.614e6 * eff) + 1.5;
-    // measured, not understood: the 128 x 128 instance with edge handling takes 922 us where the plain one takes 721 us on 768
-    // tiles (M = 2945..3071 against 3072, N = K = 4096; one ragged row is enough), 3 % more on 256 tiles (M = 1023) and nothing
-    // extra on 1536 tiles (3000 x 8192 x 8192); the 64 x 64 instance shows no such step
+    // measured: the 128 x 128 instance with edge handling takes 922 us where the plain one takes 721 us on 768 tiles (M = 2945..3071
+    // against 3072, N = K = 4096; one ragged row is enough), 3 % more on 256 tiles (M = 1023) and nothing extra on 1536 tiles.  Two
+    // such workgroups share a CU; 512 tiles take 470 us with either instance, and the 256 tiles of the last round are then spread
+    // one per CU (+250 us) or packed two per CU on half the chip (+450 us) -- the hardware dispatcher's placement, which came out
+    // the second way for the edge instance; the 64 x 64 instance shows no such step
     if (tile == 128 && (M % 128 != 0 || N % 128 != 0)) tile_us *= wg > 512 && wg <= 1024 ? 1.25 : 1.03;
     double t = rounds * tile_us;
     if (ks > 1) t += 3.0 + (double)(ks + 2) * M * N * 4.0 / 3.0e6;
