@@ -95,6 +95,7 @@ SIGNATURES = {
     "aidn_mi355_pack_b": (_i, [_vp, _vp, _i, _vp, _i, _i, _i, _vp]),
     "aidn_mi355_gemm_packed_b": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
     "aidn_mi355_reserve_workspace": (_i, [_vp, _vp, _u64]),
+    "aidn_mi355_release_stream_workspace": (_i, [_vp, _vp]),
     "aidn_mi355_workspace_bytes": (_u64, [_vp, _vp]),
     "aidn_mi355_set_gemm_tile": (_i, [_vp, _i]),
     "aidn_mi355_set_attention_fast_path": (_i, [_vp, _i]),

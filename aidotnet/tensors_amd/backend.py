@@ -88,10 +88,12 @@ class Mi355Backend:
 
     BackendName = "HIP-MI355X"
 
-    def __init__(self, device: int = 0, synchronous: bool = True, validate_block_tables: bool = False):
+    def __init__(self, device: int = 0, synchronous: bool = True, validate_block_tables: Optional[bool] = None):
         # validate_block_tables: read every block table back to the host and check its ids against the pool before a paged
         # call (a device-to-host copy and a stream synchronisation per call; the reference's guard checks capacities only,
-        # GpuKernelGuards.cs:83-100).  Off by default so that paged calls stay launch-only and can be captured into a graph.
+        # GpuKernelGuards.cs:83-100).  The kernels index the pools with the ids unchecked, so a bad id is an out-of-bounds
+        # device read: None (the default) checks whenever the current stream is not being captured into a graph, True always
+        # (a capture then fails on the copy), False never (launch-only calls; the caller vouches for the table).
         self.ValidateBlockTables = validate_block_tables
         self._lib = _lib.load()
         if not torch.cuda.is_available():
@@ -158,6 +160,11 @@ class Mi355Backend:
     def WorkspaceBytes(self) -> int:
         """Current size of the library workspace of the current stream."""
         return int(self._lib.aidn_mi355_workspace_bytes(self._ctx, self._stream()))
+
+    def ReleaseStreamWorkspace(self) -> None:
+        """Waits for the current stream and frees the workspace the library holds for it (for callers that create and destroy
+        streams; graphs captured from the stream must not be replayed afterwards).  No counterpart in the reference."""
+        self._check(self._lib.aidn_mi355_release_stream_workspace(self._ctx, self._stream()))
 
     # buffers -- AllocateBuffer zero-fills (HipBackend.cs:1251-1273)
     def AllocateBuffer(self, data_or_size) -> GpuBuffer:
@@ -430,7 +437,10 @@ class Mi355Backend:
         bt = blockTable.tensor.reshape(-1)[:blocks]
         if bt.dtype != torch.int32:
             raise ArgumentException("%s: blockTable must hold 32-bit block ids." % op)
-        if self.ValidateBlockTables and (int(bt.min()) < 0 or int(bt.max()) >= kcache.SizeInBytes // per_block):
+        validate = self.ValidateBlockTables
+        if validate is None:
+            validate = not torch.cuda.is_current_stream_capturing()
+        if validate and (int(bt.min()) < 0 or int(bt.max()) >= kcache.SizeInBytes // per_block):
             raise ArgumentException("%s: blockTable names a block outside the pool." % op)
         out = self.AllocateBuffer(numQueries * heads * headDim)
         if decode:

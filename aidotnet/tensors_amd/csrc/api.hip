@@ -81,8 +81,16 @@ int acquire_ws(Ctx* c, void* stream, size_t bytes, void** out)
         if (want < 2 * slot.bytes) want = 2 * slot.bytes;           // geometric growth bounds what the retired blocks hold
         want = (want + 255) & ~(size_t)255;
         void* p = nullptr;
-        if (hipMalloc(&p, want) != hipSuccess) {
+        const hipError_t me = hipMalloc(&p, want);
+        if (me != hipSuccess) {
             (void)hipGetLastError();
+            // another stream of the process may be capturing in global mode: allocation is then refused although this stream is not
+            // the one under capture -- the same situation for the caller as a capture of its own stream
+            if (me == hipErrorStreamCaptureUnsupported || me == hipErrorStreamCaptureInvalidated || me == hipErrorStreamCaptureImplicit ||
+                me == hipErrorStreamCaptureWrongThread) {
+                c->last_error = "workspace: allocation refused while a stream capture is in progress; reserve the workspace before the capture";
+                return AIDN_ERR_WORKSPACE;
+            }
             c->last_error = "workspace: hipMalloc failed";
             return AIDN_ERR_OUT_OF_MEMORY;
         }
@@ -197,7 +205,8 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
         else if (st) return st;
     }
     if (!valid_activation(act)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm: unknown activation");
-    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, bias, act, act_param), "gemm_16");
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind, A, B, C, out32, M, N, K, c->force_tile, ws, ws ? need : 0, bias, act, act_param),
+                      "gemm_16");
 }
 
 // [Wq|Wk|Wv] side by side in one [dModel, 3 dModel] matrix (three strided device copies), the weight operand of the fused
@@ -253,7 +262,7 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
     const int M = (int)rows, N3 = 3 * dModel;
     const int tile32 = c->force_tile;
     if (kind == 0) e = aidn::gemm_f32(sm, (const float*)input, (const float*)w3, (float*)qkv, M, N3, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
-    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)w3, qkv, 0, M, N3, dModel, c->force_tile, nullptr);
+    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)input, (const uint16_t*)w3, qkv, 0, M, N3, dModel, c->force_tile, nullptr, 0);
     if (e != hipSuccess) return hip_status(c, e, "mha: QKV projection");
 
     aidn::AttnParams p{};
@@ -269,7 +278,7 @@ int mha_common(void* ctx, void* stream, int kind, const void* input, const void*
     if (e != hipSuccess) return hip_status(c, e, "mha: attention");
 
     if (kind == 0) e = aidn::gemm_f32(sm, (const float*)cc, (const float*)wo, (float*)output, M, dModel, dModel, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile32);
-    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)cc, (const uint16_t*)wo, output, 0, M, dModel, dModel, c->force_tile, nullptr);
+    else e = aidn::gemm_16(sm, kind - 1, (const uint16_t*)cc, (const uint16_t*)wo, output, 0, M, dModel, dModel, c->force_tile, nullptr, 0);
     return hip_status(c, e, "mha: output projection");
 }
 
@@ -301,6 +310,7 @@ int paged_common(void* ctx, void* stream, int kind, const void* q, const void* k
     p.ks[0] = 0; p.ks[1] = head_dim; p.ks[2] = (long long)kv_heads * head_dim;
     p.vs[0] = 0; p.vs[1] = head_dim; p.vs[2] = (long long)kv_heads * head_dim;
     p.block_table = block_table; p.block_size = block_size; p.block_table_stride = 0;
+    p.allow_fast_path = c->attn_fast_path;
     if (decode) {
         int eff = aidn::attn_decode_splits(kind, p, splits);
         size_t need = aidn::attn_decode_workspace_bytes(p, eff);
@@ -308,7 +318,6 @@ int paged_common(void* ctx, void* stream, int kind, const void* q, const void* k
         if (need) { int st = acquire_ws(c, stream, need, &ws); if (st) return st; }
         return hip_status(c, aidn::attn_decode((hipStream_t)stream, kind, p, eff, ws), "paged attn_decode");
     }
-    p.allow_fast_path = c->attn_fast_path;
     return hip_status(c, aidn::attn_fwd((hipStream_t)stream, kind, p), "paged attn_fwd");
 }
 
@@ -420,15 +429,16 @@ AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
 
 // workspace of the fp32 paths that need one: small M (M <= 8, B [K,N]) and split-K partials; mode 0 B [K,N], 1 B [N,K], 2 fp16
 // weights (small M only).  *ws stays null when no such path applies or a tile size is forced
-static int smallm_ws(Ctx* c, void* stream, int M, int N, int K, int transB, void** ws)
+static int smallm_ws(Ctx* c, void* stream, int M, int N, int K, int transB, void** ws, size_t* ws_bytes)
 {
-    *ws = nullptr;
+    *ws = nullptr; *ws_bytes = 0;
     if (c->force_tile != 0) return 0;
     size_t need = transB == 2 ? aidn::gemm_smallm_workspace_bytes(M, N, K) : aidn::gemm_f32_workspace_bytes(M, N, K, transB);
     if (!need) return 0;
     const int st = acquire_ws(c, stream, need, ws);
     // a stream under capture whose workspace would have to grow: the tiled kernel needs none
     if (st == AIDN_ERR_WORKSPACE) { *ws = nullptr; return 0; }
+    if (st == 0) *ws_bytes = need;
     return st;
 }
 
@@ -440,10 +450,10 @@ AIDN_API int aidn_mi355_sgemm(void* ctx, void* stream, const float* A, const flo
     if (!A || !B || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm: dimensions must be positive");
     int tile = c->force_tile;
-    void* ws = nullptr;
-    if (int st = smallm_ws(c, stream, M, N, K, transB != 0, &ws)) return st;
-    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws),
-                      "gemm_f32");
+    void* ws = nullptr; size_t ws_bytes = 0;
+    if (int st = smallm_ws(c, stream, M, N, K, transB != 0, &ws, &ws_bytes)) return st;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, alpha, beta, transB != 0, 1, 0, 0, 0, tile, nullptr, 0, 0.0f, ws,
+                                        nullptr, ws_bytes), "gemm_f32");
 }
 
 AIDN_API int aidn_mi355_sgemm_batched(void* ctx, void* stream, const float* A, const float* B, float* C,
@@ -469,10 +479,10 @@ AIDN_API int aidn_mi355_sgemm_bias_act(void* ctx, void* stream, const float* A, 
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_bias_act: unknown activation");
     int tile = c->force_tile;
-    void* ws = nullptr;
-    if (int st = smallm_ws(c, stream, M, N, K, 0, &ws)) return st;
-    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param, ws),
-                      "gemm_f32 (bias + activation)");
+    void* ws = nullptr; size_t ws_bytes = 0;
+    if (int st = smallm_ws(c, stream, M, N, K, 0, &ws, &ws_bytes)) return st;
+    return hip_status(c, aidn::gemm_f32((hipStream_t)stream, A, B, C, M, N, K, 1.0f, 0.0f, 0, 1, 0, 0, 0, tile, bias, activation, act_param, ws,
+                                        nullptr, ws_bytes), "gemm_f32 (bias + activation)");
 }
 AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A, const uint16_t* B_f16, const float* bias, float* C,
                                int M, int N, int K, int activation, float act_param)
@@ -482,10 +492,10 @@ AIDN_API int aidn_mi355_sgemm_f16weight(void* ctx, void* stream, const float* A,
     if (!A || !B_f16 || !C) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: A, B and C must not be null");
     if (M <= 0 || N <= 0 || K <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: dimensions must be positive");
     if (!valid_activation(activation)) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "sgemm_f16weight: unknown activation");
-    void* ws = nullptr;
-    if (int st = smallm_ws(c, stream, M, N, K, 2, &ws)) return st;
-    return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param, ws),
-                      "gemm_f32_f16weight");
+    void* ws = nullptr; size_t ws_bytes = 0;
+    if (int st = smallm_ws(c, stream, M, N, K, 2, &ws, &ws_bytes)) return st;
+    return hip_status(c, aidn::gemm_f32_f16weight((hipStream_t)stream, A, B_f16, C, M, N, K, c->force_tile, bias, activation, act_param, ws,
+                                                  ws_bytes), "gemm_f32_f16weight");
 }
 AIDN_API int aidn_mi355_hgemm_bias_act(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, const float* bias, void* C,
                               int out_is_f32, int M, int N, int K, int activation, float act_param)
@@ -533,10 +543,10 @@ AIDN_API int aidn_mi355_gemm_packed_b(void* ctx, void* stream, int kind, const v
     if (kind == 0) {
         if ((((uintptr_t)A) & 15u) != 0 && K % 32 == 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_packed_b: A must be 16-byte aligned");
         return hip_status(c, aidn::gemm_f32((hipStream_t)stream, (const float*)A, nullptr, (float*)C, M, N, K, 1.0f, 0.0f, transB != 0, 1, 0, 0, 0, 0,
-                                            bias, activation, act_param, ws, (const float*)packedB), "gemm_f32 (packed B)");
+                                            bias, activation, act_param, ws, (const float*)packedB, ws ? need : 0), "gemm_f32 (packed B)");
     }
-    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind - 1, (const uint16_t*)A, nullptr, C, out_is_f32 != 0, M, N, K, 0, ws, bias, activation,
-                                       act_param, (const uint16_t*)packedB), "gemm_16 (packed B)");
+    return hip_status(c, aidn::gemm_16((hipStream_t)stream, kind - 1, (const uint16_t*)A, nullptr, C, out_is_f32 != 0, M, N, K, 0, ws, ws ? need : 0,
+                                       bias, activation, act_param, (const uint16_t*)packedB), "gemm_16 (packed B)");
 }
 
 AIDN_API int aidn_mi355_hgemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K)
@@ -662,6 +672,29 @@ AIDN_API int aidn_mi355_reserve_workspace(void* ctx, void* stream, uint64_t byte
     if (!c) return AIDN_ERR_INVALID_ARGUMENT;
     void* ws = nullptr;
     return acquire_ws(c, stream, (size_t)bytes, &ws);
+}
+AIDN_API int aidn_mi355_release_stream_workspace(void* ctx, void* stream)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    WsSlot slot;
+    {
+        std::lock_guard<std::mutex> g(c->mu);
+        auto it = c->ws.find(stream);
+        if (it == c->ws.end()) return AIDN_OK;
+        hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing((hipStream_t)stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone) {
+            c->last_error = "release_stream_workspace: the stream is being captured";
+            return AIDN_ERR_WORKSPACE;
+        }
+        slot = it->second;
+        c->ws.erase(it);
+    }
+    // everything the library queued on this stream has to be through with the blocks before they go back
+    if (hipError_t e = hipStreamSynchronize((hipStream_t)stream)) return hip_status(c, e, "release_stream_workspace");
+    for (void* p : slot.retired) (void)hipFree(p);
+    if (slot.cur) (void)hipFree(slot.cur);
+    return AIDN_OK;
 }
 AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream)
 {

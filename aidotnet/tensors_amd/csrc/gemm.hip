@@ -1490,14 +1490,17 @@ struct PadPlan {
 };
 static size_t gemm_16_inner_workspace_bytes(int M, int N, int K)
 {
-    if (skinny_applies(M, N, K)) return (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
+    size_t need = 0;
+    if (skinny_applies(M, N, K)) need = (size_t)skinny_ksplit(N, K) * M * N * sizeof(float);
     if (const int first = msplit16_rows(M, N, K)) {
         const size_t a = gemm_16_inner_workspace_bytes(first, N, K), b = gemm_16_inner_workspace_bytes(M - first, N, K);
-        return a > b ? a : b;
+        if (a > need) need = a;
+        if (b > need) need = b;
     }
     int big;
     const int ks = splitk16_ranges(M, N, K, &big);
-    return ks ? (size_t)ks * M * N * sizeof(float) : 0;
+    const size_t split = ks ? (size_t)ks * M * N * sizeof(float) : 0;
+    return split > need ? split : need;
 }
 // the padded shapes and the workspace layout for them (no judgement on whether padding pays)
 static bool pad16_layout(int M, int N, int K, PadPlan* pl)
@@ -1681,11 +1684,14 @@ hipError_t unpad_rows(hipStream_t stream, const void* src, void* dst, long long 
     return hipGetLastError();
 }
 
+// The largest need over the plans gemm_16 may take for these dimensions (the choice also depends on operand alignment; every
+// plan checks its own need against the bytes it is handed).
 size_t gemm_16_workspace_bytes(int M, int N, int K)
 {
     PadPlan pl;
-    if (pad16_plan(M, N, K, &pl)) return pl.total;
-    return gemm_16_inner_workspace_bytes(M, N, K);
+    const size_t inner = gemm_16_inner_workspace_bytes(M, N, K);
+    if (pad16_plan(M, N, K, &pl) && pl.total > inner) return pl.total;
+    return inner;
 }
 // Pre-packed B (the caller keeps it): B [K,N] zero-padded to [Kp, Np] -- the copy that an unaligned product otherwise makes on every
 // call, made once.  An aligned weight is packed the same way (its K and N padded to whole tiles).
@@ -2066,14 +2072,19 @@ size_t gemm_f32_packed_workspace_bytes(int M, int N, int K, int transB)
     return pl.b_off > small ? pl.b_off : small;                       // the padded copy of A, or the small-M partials
 }
 
+// The largest need over every plan gemm_f32 may take for these dimensions: which one it takes also depends on the alignment of
+// the operands, which the sizing does not see, and every plan checks its own need against the bytes it is handed.
 size_t gemm_f32_workspace_bytes(int M, int N, int K, int transB)
 {
+    size_t need = 0;
+    auto upto = [&](size_t n) { if (n > need) need = n; };
     Pad32Plan pl;
-    if (!(!transB && smallm_applies(M, N, K)) && pad32_plan(M, N, K, transB, &pl)) return pl.total;
-    if (!transB && smallm_applies(M, N, K)) return gemm_smallm_workspace_bytes(M, N, K);
-    if (!transB && skinny32_applies(M, N, K)) return (size_t)skinny32_ksplit(N, K) * M * N * sizeof(float);
+    if (pad32_plan(M, N, K, transB, &pl)) upto(pl.total);
+    if (!transB && smallm_applies(M, N, K)) upto(gemm_smallm_workspace_bytes(M, N, K));
+    if (!transB && skinny32_applies(M, N, K)) upto((size_t)skinny32_ksplit(N, K) * M * N * sizeof(float));
     const int ks = splitk32_ranges(M, N, K);
-    return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
+    if (ks > 1) upto((size_t)ks * M * N * sizeof(float));
+    return need;
 }
 #endif
 
@@ -2310,21 +2321,28 @@ static hipError_t dispatch_gemm(const GemmArgs& g, int batch, hipStream_t stream
 #if AIDN_GEMM_PART == 0
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
-                    int force_tile, const float* bias, int act, float act_param, void* workspace, const float* Bpre)
+                    int force_tile, const float* bias, int act, float act_param, void* workspace, const float* Bpre,
+                    size_t workspace_bytes)
 {
     GemmArgs g{A, B, C, M, N, K, K, transB ? K : N, N, sA, sB, sC, alpha, beta, 0, 0, bias, act, act_param};
-    if (!Bpre && force_tile == 0 && workspace && !transB && batch == 1 && smallm_applies(M, N, K))
+    if (!workspace) workspace_bytes = 0;
+    // every plan below that writes to the workspace first holds its own need against the bytes handed in, and is passed over
+    // (down to the tiled kernels, which need none) when they do not suffice
+    const bool smallm_fits = workspace && smallm_applies(M, N, K) && gemm_smallm_workspace_bytes(M, N, K) <= workspace_bytes;
+    if (!Bpre && force_tile == 0 && smallm_fits && !transB && batch == 1)
         return launch_smallm<false>(g, stream, (float*)workspace);
     // Bpre: B already packed by gemm_f32_pack_b (B itself is then not read); such a call always takes the padded shapes
     Pad32Plan pl;
-    if (Bpre && !transB && batch == 1 && workspace && smallm_applies(M, N, K) && aligned16(Bpre) && pad32_layout(M, N, K, 0, &pl)) {
+    if (Bpre && !transB && batch == 1 && smallm_fits && aligned16(Bpre) && pad32_layout(M, N, K, 0, &pl)) {
         GemmArgs gs = g;
         gs.B = Bpre; gs.ldb = pl.Np;                 // the padded rows; only the first K of them are read
         return launch_smallm<false>(gs, stream, (float*)workspace);
     }
-    if (Bpre && !(batch == 1 && aligned16(Bpre) && pad32_layout(M, N, K, transB, &pl) && (pl.Kp == K ? aligned16(A) : (workspace && aligned16(workspace)))))
+    if (Bpre && !(batch == 1 && aligned16(Bpre) && pad32_layout(M, N, K, transB, &pl) &&
+                  (pl.Kp == K ? aligned16(A) : (workspace && aligned16(workspace) && pl.b_off <= workspace_bytes))))
         return hipErrorInvalidValue;
-    if (Bpre || (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && (pl.Kp != K || aligned16(A)))) {
+    if (Bpre || (force_tile == 0 && workspace && batch == 1 && aligned16(workspace) && pad32_plan(M, N, K, transB, &pl) && pl.total <= workspace_bytes &&
+                 (pl.Kp != K || aligned16(A)))) {
         unsigned char* w = (unsigned char*)workspace;
         const float* Ap = A;
         if (pl.Kp != K) {
@@ -2340,9 +2358,10 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
         if (pl.Np != N) gp.c_cols = N;
         return transB ? dispatch_gemm<float, float, true>(gp, 1, stream, 0) : dispatch_gemm<float, float, false>(gp, 1, stream, 0);
     }
-    if (force_tile == 0 && workspace && !transB && batch == 1 && skinny32_applies(M, N, K) && aligned16(A) && aligned16(B)) {
-        int ks;
-        const int kper = 32 * skinny32_plan(N, K, &ks);
+    int ks32 = 0;
+    const int kper32 = (force_tile == 0 && workspace && !transB && batch == 1 && skinny32_applies(M, N, K)) ? 32 * skinny32_plan(N, K, &ks32) : 0;
+    if (kper32 && aligned16(A) && aligned16(B) && (size_t)ks32 * M * N * sizeof(float) <= workspace_bytes) {
+        const int ks = ks32, kper = kper32;
         constexpr int smem = SKINNY32_STAGES * (32 * 128 + 32 * 512);
         static unsigned long long attr_done = 0;
         if (hipError_t e0 = ensure_dynamic_smem((const void*)gemm_skinny32_kernel<SKINNY32_STAGES>, smem, &attr_done)) return e0;
@@ -2357,7 +2376,7 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
         // few tiles over a long K: the K ranges run as batches into fp32 partials, summed in range order (deterministic)
         // by the pass that also applies alpha, beta, bias and activation
         const int ks = splitk32_ranges(M, N, K);
-        if (ks > 1) {
+        if (ks > 1 && (size_t)ks * M * N * sizeof(float) <= workspace_bytes) {
             GemmArgs gp = g;
             gp.C = workspace; gp.K = K / ks; gp.ldc = N; gp.alpha = 1.0f; gp.beta = 0.0f;
             gp.sA = K / ks; gp.sB = transB ? (long long)(K / ks) : (long long)(K / ks) * N; gp.sC = (long long)M * N;
@@ -2376,10 +2395,11 @@ hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C
 
 // fp32 A [M,K] x fp16 weights B [K,N] -> fp32 C, optional fused epilogue
 hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K,
-                              int force_tile, const float* bias, int act, float act_param, void* workspace)
+                              int force_tile, const float* bias, int act, float act_param, void* workspace, size_t workspace_bytes)
 {
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
-    if (force_tile == 0 && workspace && smallm_applies(M, N, K)) return launch_smallm<true>(g, stream, (float*)workspace);
+    if (force_tile == 0 && workspace && smallm_applies(M, N, K) && gemm_smallm_workspace_bytes(M, N, K) <= workspace_bytes)
+        return launch_smallm<true>(g, stream, (float*)workspace);
     // rows of A in 16-byte steps, rows of the fp16 B in 8-byte steps
     const bool vec = aligned16(A) && K % 4 == 0 && (((uintptr_t)B) & 7u) == 0 && N % 4 == 0;
     auto tiles = [&](int bm, int bn) { return (long long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
@@ -2397,13 +2417,17 @@ hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t
 // one 16-bit type per part: T = f16_t in part 1, bf16_t in part 2; out32: C is fp32 (else the same 16-bit type as the inputs)
 template <typename T>
 static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                                int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param,
-                                const uint16_t* Bpre = nullptr)
+                                int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act,
+                                float act_param, const uint16_t* Bpre = nullptr)
 {
+    // Every plan below that writes to the workspace holds its own need against workspace_bytes first and is passed over when the
+    // bytes do not suffice (the tiled kernels at the end need none).
+    if (!workspace) workspace_bytes = 0;
     // Bpre: B already packed by gemm_16_pack_b (B itself is then not read); such a call always takes the padded shapes
     PadPlan pl;
-    if (Bpre && !(workspace && aligned16(C) && aligned16(workspace) && aligned16(Bpre) && pad16_layout(M, N, K, &pl))) return hipErrorInvalidValue;
-    if (Bpre || (force_tile == 0 && workspace && aligned16(C) && aligned16(workspace) && pad16_plan(M, N, K, &pl))) {
+    if (Bpre && !(workspace && aligned16(C) && aligned16(workspace) && aligned16(Bpre) && pad16_layout(M, N, K, &pl) && pl.total <= workspace_bytes))
+        return hipErrorInvalidValue;
+    if (Bpre || (force_tile == 0 && workspace && aligned16(C) && aligned16(workspace) && pad16_plan(M, N, K, &pl) && pl.total <= workspace_bytes)) {
         unsigned char* w = (unsigned char*)workspace;
         const bool padA = pl.Kp != K, padC = pl.Np != N;
         const uint16_t* Ap = A;
@@ -2434,26 +2458,28 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
         }
         void* Cp = padC ? (void*)(w + pl.c_off) : C;
         if (hipError_t e = gemm_16_typed<T>(stream, Ap, Bp, Cp, out32, M, pl.Np, pl.Kp, 0,
-                                            pl.total > pl.inner_off ? (void*)(w + pl.inner_off) : nullptr, bp, act, act_param)) return e;
+                                            pl.total > pl.inner_off ? (void*)(w + pl.inner_off) : nullptr,
+                                            pl.total > pl.inner_off ? pl.total - pl.inner_off : 0, bp, act, act_param)) return e;
         return padC ? unpad_rows(stream, Cp, C, M, N, pl.Np, out32 ? 4 : 2) : hipSuccess;
     }
     GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, bias, act, act_param};
-    if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B)) {
+    if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B) &&
+        (size_t)skinny_ksplit(N, K) * M * N * sizeof(float) <= workspace_bytes) {
         float* ws = (float*)workspace;
         return out32 ? launch_skinny<T, float>(g, stream, ws) : launch_skinny<T, T>(g, stream, ws);
     }
     if (force_tile == 0 && dl16_applies<float>(g)) {
         if (const int first = msplit16_rows(M, N, K)) {
             // the rows of the whole rounds, then the rest (stream order; the two share the workspace one after the other)
-            if (hipError_t e = gemm_16_typed<T>(stream, A, B, C, out32, first, N, K, 0, workspace, bias, act, act_param)) return e;
+            if (hipError_t e = gemm_16_typed<T>(stream, A, B, C, out32, first, N, K, 0, workspace, workspace_bytes, bias, act, act_param)) return e;
             return gemm_16_typed<T>(stream, A + (size_t)first * K, B, (unsigned char*)C + (size_t)first * N * (out32 ? 4 : 2), out32, M - first, N, K, 0,
-                                    workspace, bias, act, act_param);
+                                    workspace, workspace_bytes, bias, act, act_param);
         }
     }
     if (force_tile == 0 && workspace) {
         int big = 0;
         const int ks = splitk16_ranges(M, N, K, &big);
-        if (ks) {
+        if (ks && (size_t)ks * M * N * sizeof(float) <= workspace_bytes) {
             GemmArgs gp = g;
             gp.C = workspace; gp.K = K / ks; gp.ldc = N;
             gp.sA = K / ks; gp.sB = (long long)(K / ks) * N; gp.sC = (long long)M * N;
@@ -2473,24 +2499,24 @@ static hipError_t gemm_16_typed(hipStream_t stream, const uint16_t* A, const uin
 }
 
 hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre);
+                       int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre);
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre);
+                        int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre);
 #if AIDN_GEMM_PART == 1
 hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                       int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
-{ return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre); }
+                       int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre)
+{ return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre); }
 #elif AIDN_GEMM_PART == 2
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                        int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
-{ return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre); }
+                        int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre)
+{ return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre); }
 #else
 // kind: 0 = fp16, 1 = bf16
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace, const float* bias, int act, float act_param, const uint16_t* Bpre)
+                   int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre)
 {
-    if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre);
-    return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, bias, act, act_param, Bpre);
+    if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre);
+    return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre);
 }
 #endif
 

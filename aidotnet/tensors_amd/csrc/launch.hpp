@@ -10,7 +10,8 @@ namespace aidn {
 hipError_t gemm_f32(hipStream_t stream, const float* A, const float* B, float* C, int M, int N, int K,
                     float alpha, float beta, int transB, int batch, long long sA, long long sB, long long sC,
                     int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f, void* workspace = nullptr,
-                    const float* Bpre = nullptr);
+                    const float* Bpre = nullptr, size_t workspace_bytes = 0);
+// workspace_bytes: size of `workspace`; a plan whose partials or padded copies would not fit is passed over
 // Bpre: B packed once by gemm_f32_pack_b into gemm_f32_packed_b_bytes(N, K, transB) bytes (B itself is then ignored; one batch); the
 // workspace must then hold gemm_f32_packed_workspace_bytes(M, N, K, transB) bytes
 size_t gemm_f32_packed_b_bytes(int N, int K, int transB);
@@ -23,13 +24,13 @@ size_t gemm_smallm_workspace_bytes(int M, int N, int K);
 // weight-only fp16 GEMM: fp32 A [M,K] x fp16 B [K,N] -> fp32 C (the weights are widened exactly, everything else is fp32)
 hipError_t gemm_f32_f16weight(hipStream_t stream, const float* A, const uint16_t* B, float* C, int M, int N, int K,
                               int force_tile, const float* bias = nullptr, int act = 0, float act_param = 0.0f,
-                              void* workspace = nullptr);
+                              void* workspace = nullptr, size_t workspace_bytes = 0);
 // workspace: gemm_16_workspace_bytes(M, N, K) bytes (0 = none needed); without it the skinny-M path is not taken
 size_t gemm_16_workspace_bytes(int M, int N, int K);
 // Bpre: B packed once by gemm_16_pack_b into gemm_16_packed_b_bytes(N, K) bytes (B itself is then ignored); the workspace must then
 // hold gemm_16_packed_workspace_bytes(M, N, K) bytes
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
-                   int M, int N, int K, int force_tile, void* workspace, const float* bias = nullptr, int act = 0,
+                   int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias = nullptr, int act = 0,
                    float act_param = 0.0f, const uint16_t* Bpre = nullptr);
 size_t gemm_16_packed_b_bytes(int N, int K);
 size_t gemm_16_packed_workspace_bytes(int M, int N, int K);

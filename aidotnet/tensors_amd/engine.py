@@ -13,6 +13,8 @@ from __future__ import annotations
 import math
 from typing import Optional, Tuple
 
+import weakref
+
 import torch
 
 from .backend import (ArgumentException, ArgumentNullException, ArgumentOutOfRangeException, Mi355Backend,
@@ -83,10 +85,14 @@ class Mi355Engine:
 
     def TensorMatMulCachedB(self, a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
         """a [..., K] times a rank-2 weight b [K, N] that is expected again: b is packed once (backend.PackB) and the packed form
-        is kept, keyed the way SimdGemm.SgemmWithCachedB keys its PrePackedB entries (SimdGemm.cs:327-684: array identity, the
-        array's version and its shape; a changed weight is packed again) -- here the tensor's storage pointer, shape, dtype and
-        torch's in-place version counter.  Values are those of TensorMatMul.  At most ``CACHED_B_CAPACITY`` weights are kept, the
-        least recently used one leaves first (the reference bounds its cache the same way, SimdGemm.cs:1030-1159)."""
+        is kept, keyed the way SimdGemm.SgemmWithCachedB keys its PrePackedB entries (SimdGemm.cs:292, 327-684: a
+        ConditionalWeakTable on the identity of the weight array, collected with the array, plus the array's version; a changed
+        weight is packed again) -- here the identity of the caller's tensor object, held through a weak reference that is
+        compared on every hit and that drops the entry when the tensor dies, plus torch's in-place version counter.  A device
+        address is never the key: the allocator hands a freed block to the next tensor of the same size.  A weight that is not
+        contiguous (a transposed view) is packed from a temporary copy on every call and not cached.  Values are those of
+        TensorMatMul.  At most ``CACHED_B_CAPACITY`` weights are kept, the least recently used one leaves first (the reference
+        bounds its cache the same way, SimdGemm.cs:1030-1159)."""
         if a is None or b is None:
             raise ArgumentNullException("a" if a is None else "b")
         if b.dim() != 2 or a.dim() < 1:
@@ -96,20 +102,25 @@ class Mi355Engine:
         if a.shape[-1] != b.shape[0]:
             raise ArgumentException("inner dimensions do not match: %s x %s" % (tuple(a.shape), tuple(b.shape)))
         be = self.backend
-        a = a.contiguous(); b = b.contiguous()
+        a = a.contiguous()
         K, N = b.shape
         kind = _KIND[a.dtype]
-        cache = self.__dict__.setdefault("_packed_b", {})
-        key = (b.data_ptr(), K, N, b.dtype)
-        hit = cache.pop(key, None)
-        if hit is None or hit[0] != b._version:
-            hit = (b._version, be.PackB(kind, be.WrapTensor(b), K, N))
-        cache[key] = hit                                                        # most recently used last
-        while len(cache) > self.CACHED_B_CAPACITY:
-            cache.pop(next(iter(cache)))
+        if not b.is_contiguous():
+            packed = be.PackB(kind, be.WrapTensor(b.contiguous()), K, N)      # a temporary copy has no identity to key on
+        else:
+            cache = self.__dict__.setdefault("_packed_b", {})
+            key = id(b)
+            hit = cache.pop(key, None)
+            if hit is None or hit[0]() is not b or hit[1] != b._version or hit[2] != (b.data_ptr(), K, N, b.dtype):
+                owner = weakref.ref(b, lambda _r, c=cache, k=key: c.pop(k, None) if (k in c and c[k][0] is _r) else None)
+                hit = (owner, b._version, (b.data_ptr(), K, N, b.dtype), be.PackB(kind, be.WrapTensor(b), K, N))
+            cache[key] = hit                                                    # most recently used last
+            while len(cache) > self.CACHED_B_CAPACITY:
+                cache.pop(next(iter(cache)))
+            packed = hit[3]
         M = a.numel() // K
         out = torch.empty(*a.shape[:-1], N, dtype=a.dtype, device=a.device)
-        be.GemmPackedB(kind, be.WrapTensor(a), hit[1], None, be.WrapTensor(out), M, N, K, outputIsFp32=(a.dtype == torch.float32))
+        be.GemmPackedB(kind, be.WrapTensor(a), packed, None, be.WrapTensor(out), M, N, K, outputIsFp32=(a.dtype == torch.float32))
         return out
 
     CACHED_B_CAPACITY = 64

@@ -49,7 +49,11 @@ enum {
  * the context has been called on, so calls on different streams never share it; it grows on demand
  * (a block that has been handed to a kernel is never freed before aidn_mi355_destroy, so queued work
  * and captured graphs keep valid addresses) and is released by aidn_mi355_destroy.  Calls on the SAME
- * stream run in order and may share it.  The context may be used from several host threads. */
+ * stream run in order and may share it.  The context may be used from several host threads; every call
+ * must be made with the context's device current on the calling thread (hipSetDevice(device) -- the
+ * library launches on the caller's current device and does not switch it: aidn_mi355_create leaves
+ * `device` current on the thread that called it, other threads set it themselves; the reference's
+ * backend likewise selects its device once, in its constructor, HipBackend.cs:246). */
 AIDN_API int aidn_mi355_create(int device, void** ctx);
 AIDN_API int aidn_mi355_destroy(void* ctx);
 /* Text of the last failure on this context (never NULL; empty when none). */
@@ -65,6 +69,12 @@ AIDN_API int aidn_mi355_sync(void* ctx, void* stream);
  * per call from its buffer pool (HipBackend.cs:12214-12270). */
 AIDN_API int aidn_mi355_reserve_workspace(void* ctx, void* stream, uint64_t bytes);
 AIDN_API uint64_t aidn_mi355_workspace_bytes(void* ctx, void* stream);
+/* Gives back the workspace the context holds for `stream` (waits for the stream first, then frees the current block and every
+ * block retired by growth): for callers that create and destroy streams, since a block is otherwise kept until
+ * aidn_mi355_destroy.  Graphs captured from this stream must not be replayed afterwards (they hold the freed addresses).
+ * AIDN_ERR_WORKSPACE while the stream is being captured.  No counterpart in the reference (its buffers return to a pool per
+ * call, HipBackend.cs:12214-12270). */
+AIDN_API int aidn_mi355_release_stream_workspace(void* ctx, void* stream);
 
 /* ---- fp32 GEMM -------------------------------------------------------------------------------
  * C[M,N] = alpha * A[M,K] * op(B) + beta * C.  transB == 0: B is [K,N]; transB != 0: B is stored

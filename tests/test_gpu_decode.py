@@ -105,9 +105,43 @@ def test_batched_decode_all_types_and_layouts(be, kind, layout, B, H, Hkv, S, D)
         assert mixed_err(out16.float().cpu().numpy(), o64) <= tol
 
 
+def _decode_truth_f64(q, k, v, scale):
+    """float64 softmax(scale q K^T) V and log-sum-exp of EVERY (batch, head) slice on the device, from the same rounded inputs:
+    the arithmetic of oracle.attention_f64 (the callers tie the two together on sampled slices).  q [B,H,1,D]; k, v [B,Hkv,S,D]."""
+    B, H, _, D = q.shape
+    Hkv = k.shape[1]
+    o = torch.empty(B, H, D, dtype=torch.float64, device="cuda")
+    lse = torch.empty(B, H, dtype=torch.float64, device="cuda")
+    for b in range(B):              # one batch entry at a time: the float64 copy of a 2 GiB cache would be 8 GiB
+        k64, v64 = k[b].double(), v[b].double()                                   # [Hkv, S, D]
+        q64 = q[b, :, 0].double().reshape(Hkv, H // Hkv, D)                       # query head h reads K/V head h / (H / Hkv)
+        logits = torch.einsum("ugd,usd->ugs", q64, k64) * scale
+        lse[b] = torch.logsumexp(logits, dim=2).reshape(H)
+        o[b] = torch.einsum("ugs,usd->ugd", torch.softmax(logits, dim=2), v64).reshape(H, D)
+    return o, lse
+
+
+def _check_every_slice(out, lse, q, k, v, scale, samples):
+    o64, lse64 = _decode_truth_f64(q, k, v, scale)
+    err = ((out[:, :, 0].double() - o64).abs() / (1 + o64.abs())).amax(dim=2)     # per (batch, head)
+    worst = int(err.argmax())
+    assert float(err.max()) <= 2e-2, ("slice", worst // err.shape[1], worst % err.shape[1], float(err.max()))
+    # the row sum adds the probabilities as rounded to bf16 (the numbers the P V product uses): up to 2^-9 relative per term
+    lerr = (lse.reshape(lse64.shape).double() - lse64).abs()
+    assert float(lerr.max()) <= 4e-3, ("lse slice", int(lerr.argmax()), float(lerr.max()))
+    G = q.shape[1] // k.shape[1]
+    for (b, h) in samples:          # the device float64 arithmetic against the oracle's
+        qs = q[b:b + 1, h:h + 1].float().cpu().numpy()
+        ks, vs = (t[b:b + 1, h // G:h // G + 1].float().cpu().numpy() for t in (k, v))
+        oo, ll = oracle.attention_f64(qs, ks, vs, scale)
+        assert np.max(np.abs(o64[b, h].cpu().numpy() - oo[0, 0, 0])) <= 1e-9
+        assert abs(float(lse64[b, h]) - float(np.ravel(ll)[0])) <= 1e-9
+        assert mixed_err(out[b, h].cpu().numpy(), oo[0, 0]) <= 2e-2
+
+
 def test_config5_decode_bf16_b32_h32_s4096_d128(be):
-    # B=32, H=32, q_len=1, KV length 4096, d=128, contiguous [32,32,4096,128] bf16 cache.  Sampled (batch, head)
-    # slices against the fp64 oracle; every slice against the prefill kernel run at Sq = 1 on the same cache.
+    # B=32, H=32, q_len=1, KV length 4096, d=128, contiguous [32,32,4096,128] bf16 cache: every one of the 1024 (batch, head)
+    # outputs and log-sum-exps against a float64 softmax of the same bf16 inputs; three slices tie that arithmetic to the oracle.
     B, H, S, D = 32, 32, 4096, 128
     g = torch.Generator(device="cuda"); g.manual_seed(4096)
     q = torch.randn(B, H, 1, D, device="cuda", generator=g).to(torch.bfloat16)
@@ -118,18 +152,31 @@ def test_config5_decode_bf16_b32_h32_s4096_d128(be):
     lse = torch.empty(B, H, 1, device="cuda")
     be.DecodeAttention("bf16", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), B, H, S, D, scale,
                        0, 0, False, be.WrapTensor(lse))
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    _check_every_slice(out, lse, q, k, v, scale, [(0, 0), (13, 7), (31, 31)])
+    # the prefill kernel run at Sq = 1 on the same cache is a second implementation of the same function
     ref = torch.full((B, H, 1, D), float("nan"), device="cuda")
     ref_lse = torch.empty(B, H, 1, device="cuda")
     be.FlashAttentionHalf("bf16", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(ref), be.WrapTensor(ref_lse),
                           B, H, 1, S, D, scale, True, S - 1)
-    assert torch.isfinite(out).all()
     assert mixed_err(out.cpu().numpy(), ref.cpu().numpy()) <= 2e-2
     assert mixed_err(lse.cpu().numpy(), ref_lse.cpu().numpy()) <= 1e-3
-    for (b, h) in [(0, 0), (13, 7), (31, 31)]:
-        qs, ks, vs = (t[b:b + 1, h:h + 1].float().cpu().numpy() for t in (q, k, v))
-        o64, lse64 = oracle.attention_f64(qs, ks, vs, scale)
-        assert mixed_err(out[b, h].cpu().numpy(), o64[0, 0]) <= 2e-2
-        assert mixed_err(lse[b, h].cpu().numpy(), lse64[0, 0]) <= 1e-3
+
+
+def test_grouped_decode_bf16_b32_h32_hkv8_s4096_d128_every_slice(be):
+    # the grouped-query form of the same decode step (8 K/V heads for 32 query heads) at full size, every slice as above
+    B, H, Hkv, S, D = 32, 32, 8, 4096, 128
+    g = torch.Generator(device="cuda"); g.manual_seed(4097)
+    q = torch.randn(B, H, 1, D, device="cuda", generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, S, D, device="cuda", generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, S, D, device="cuda", generator=g).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((B, H, 1, D), float("nan"), device="cuda")
+    lse = torch.empty(B, H, 1, device="cuda")
+    be.DecodeAttention("bf16", be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), B, H, S, D, scale,
+                       Hkv, 0, False, be.WrapTensor(lse))
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    _check_every_slice(out, lse, q, k, v, scale, [(0, 0), (17, 5), (31, 31)])
 
 
 # Grouped-query decode at head dimension 128 in the 16-bit types: the query heads of a K/V head run as the rows of one query tile of

@@ -150,3 +150,46 @@ def test_random_fp16_weight_and_epilogue(be):
         be.GemmBiasActivationInto(be.WrapTensor(dev(a)), be.WrapTensor(dev(b)), be.WrapTensor(dev(bias)), be.WrapTensor(c2), m, n, k, 4)
         truth = np.tanh(a.astype(np.float64) @ b.astype(np.float64) + bias[None, :])
         assert mixed_err(c2.cpu().numpy().reshape(m, n), truth) <= 1e-4, (m, n, k)
+
+
+def _offset_view(x: np.ndarray, elems: int, dtype=None) -> torch.Tensor:
+    """Device copy of x whose first element sits `elems` elements past a 256-byte aligned allocation."""
+    flat = torch.from_numpy(np.ascontiguousarray(x).reshape(-1))
+    if dtype is not None:
+        flat = flat.view(dtype)
+    buf = torch.zeros(flat.numel() + elems, dtype=flat.dtype, device="cuda")
+    buf[elems:] = flat.cuda()
+    return buf[elems:]
+
+
+# The workspace of a GEMM call is sized from the dimensions alone, while the plan that runs also depends on the alignment of the
+# operands: a sub-view pointer passes over the padded-copy / streamed-weight plans and lands on a later one, which must then find
+# its own partials inside the bytes it was handed (or pass as well).  Results against float64, and a guard band behind C.
+@pytest.mark.parametrize("off_a,off_b", [(1, 0), (0, 1), (1, 1), (3, 2)])
+def test_fp32_gemm_with_sub_view_pointers_stays_inside_its_workspace(be, off_a, off_b):
+    be.SetGemmTile(0)
+    rng = np.random.default_rng(7 + off_a * 4 + off_b)
+    for (m, n, k) in [(16, 256, 4096), (24, 1024, 2048), (128, 256, 4096), (8, 512, 1024), (32, 4096, 4096), (100, 130, 4100), (512, 768, 3072)]:
+        a = rng.uniform(-1, 1, (m, k)).astype(np.float32); b = rng.uniform(-1, 1, (k, n)).astype(np.float32)
+        c = torch.full((m * n + 64,), 7.0, device="cuda")
+        be.Gemm(be.WrapTensor(_offset_view(a, off_a)), be.WrapTensor(_offset_view(b, off_b)), be.WrapTensor(c), m, n, k)
+        got = c.cpu().numpy()
+        assert np.all(got[m * n:] == 7.0), (m, n, k)
+        assert mixed_err(got[:m * n].reshape(m, n), a.astype(np.float64) @ b.astype(np.float64)) <= 1e-4, (m, n, k, off_a, off_b)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("off_a,off_b", [(1, 0), (0, 1), (4, 4), (3, 5)])
+def test_16bit_gemm_with_sub_view_pointers_stays_inside_its_workspace(be, kind, off_a, off_b):
+    be.SetGemmTile(0)
+    rng = np.random.default_rng(11 + off_a * 8 + off_b)
+    for (m, n, k) in [(16, 4096, 4096), (32, 1024, 2048), (256, 4096, 4096), (128, 4096, 4096), (1000, 768, 3072), (100, 130, 4100), (300, 1001, 520)]:
+        abits, a = round_to(rng.standard_normal((m, k)).astype(np.float32), kind)
+        bbits, b = round_to((0.05 * rng.standard_normal((k, n))).astype(np.float32), kind)
+        c = torch.full((m * n + 64,), 7.0, device="cuda")
+        A = _offset_view(abits.view(np.int16), off_a, torch.int16).view(TORCH16[kind])
+        B = _offset_view(bbits.view(np.int16), off_b, torch.int16).view(TORCH16[kind])
+        (be.GemmFp16In32fOut if kind == "f16" else be.GemmBf16In32fOut)(be.WrapTensor(A), be.WrapTensor(B), be.WrapTensor(c), m, n, k)
+        got = c.cpu().numpy()
+        assert np.all(got[m * n:] == 7.0), (m, n, k)
+        assert mixed_err(got[:m * n].reshape(m, n), a.astype(np.float64) @ b.astype(np.float64)) <= 1e-4, (kind, m, n, k, off_a, off_b)

@@ -106,13 +106,13 @@ def test_engine_cached_weight_matmul_repacks_a_changed_weight():
     assert first.shape == (3, 7, 1001) and first.dtype == torch.bfloat16
     assert torch.equal(first, eng.TensorMatMul(x, w))                       # the values of the plain product
     assert len(eng._packed_b) == 1
-    packed_before = next(iter(eng._packed_b.values()))[1]
+    packed_before = next(iter(eng._packed_b.values()))[3]
     again = eng.TensorMatMulCachedB(x, w)
-    assert torch.equal(again, first) and next(iter(eng._packed_b.values()))[1] is packed_before     # packed once
+    assert torch.equal(again, first) and next(iter(eng._packed_b.values()))[3] is packed_before     # packed once
     w.mul_(2)                                                               # in place: same storage, new version
     doubled = eng.TensorMatMulCachedB(x, w)
     assert torch.equal(doubled.float(), 2 * first.float())
-    assert next(iter(eng._packed_b.values()))[1] is not packed_before
+    assert next(iter(eng._packed_b.values()))[3] is not packed_before
     xf = x.float(); wf = w.float()
     assert torch.equal(eng.TensorMatMulCachedB(xf, wf), eng.TensorMatMul(xf, wf))
     assert len(eng._packed_b) == 2

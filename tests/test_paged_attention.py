@@ -141,9 +141,6 @@ def test_gpu_paged_guards(be):
     with pytest.raises(ArgumentException):
         be.PagedAttentionDecode(q, pool, W(torch.zeros(5, device="cuda")), bt, 4, 16, 4, 8, 1.0)
     bad = W(torch.tensor([0, 7, 2], dtype=torch.int32, device="cuda"))
-    be.ValidateBlockTables = True           # the content check is opt-in (it costs a device-to-host copy per call)
-    try:
-        with pytest.raises(ArgumentException):
-            be.PagedAttentionDecode(q, pool, pool, bad, 4, 16, 4, 12, 1.0)      # block id outside the pool
-    finally:
-        be.ValidateBlockTables = False
+    assert be.ValidateBlockTables is None   # the content check runs by default whenever the stream is not being captured
+    with pytest.raises(ArgumentException):
+        be.PagedAttentionDecode(q, pool, pool, bad, 4, 16, 4, 12, 1.0)          # block id outside the pool
