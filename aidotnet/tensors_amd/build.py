@@ -16,7 +16,8 @@ LIB_NAME = "libaidotnet_mi355.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 # (source, object name, extra flags): gemm.hip is compiled in three parts so that its template instances build in parallel
 SOURCES = [("gemm.hip", "gemm.o", ["-DAIDN_GEMM_PART=0"]), ("gemm.hip", "gemm_f16.o", ["-DAIDN_GEMM_PART=1"]),
-           ("gemm.hip", "gemm_bf16.o", ["-DAIDN_GEMM_PART=2"]), ("attention.hip", "attention.o", []), ("decode.hip", "decode.o", []),
+           ("gemm.hip", "gemm_bf16.o", ["-DAIDN_GEMM_PART=2"]), ("attention.hip", "attention.o", []), ("attention_x16.hip", "attention_x16.o", []),
+           ("decode.hip", "decode.o", []),
            ("convert.hip", "convert.o", []), ("api.hip", "api.o", [])]
 # -packed-fp32-ops off: packed fp32 VALU forms are kept out of all device code.
 HIPCC_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -65,7 +66,7 @@ def _stale(src: str, obj: str) -> bool:
     return any(os.path.getmtime(d) > os.path.getmtime(obj) for d in deps if os.path.exists(d))
 
 
-def build_library(verbose: bool = False, jobs: int = 7, incremental: bool = False) -> str:
+def build_library(verbose: bool = False, jobs: int = 8, incremental: bool = False) -> str:
     """Compiles every source (always, unless `incremental`: then only those newer than their object file) and links."""
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)

@@ -134,8 +134,9 @@ def _check_every_slice(out, lse, q, k, v, scale, samples):
         qs = q[b:b + 1, h:h + 1].float().cpu().numpy()
         ks, vs = (t[b:b + 1, h // G:h // G + 1].float().cpu().numpy() for t in (k, v))
         oo, ll = oracle.attention_f64(qs, ks, vs, scale)
-        assert np.max(np.abs(o64[b, h].cpu().numpy() - oo[0, 0, 0])) <= 1e-9
-        assert abs(float(lse64[b, h]) - float(np.ravel(ll)[0])) <= 1e-9
+        # (1e-6: the oracle takes the scale as the float the C ABI carries, the device expression as a double)
+        assert np.max(np.abs(o64[b, h].cpu().numpy() - oo[0, 0, 0])) <= 1e-6
+        assert abs(float(lse64[b, h]) - float(np.ravel(ll)[0])) <= 1e-6
         assert mixed_err(out[b, h].cpu().numpy(), oo[0, 0]) <= 2e-2
 
 
