@@ -147,9 +147,9 @@ class Mi355Backend:
         self._check(self._lib.aidn_mi355_set_gemm_tile(self._ctx, tile))
 
     def SetAttentionFastPath(self, enabled) -> None:
-        """Test hook: False routes every attention shape through the general kernel; 2 keeps the fast paths but runs unsplit
-        head-dimension-128 prefill on the 32 x 32 x 16 kernel instead of the 16 x 16 x 32 one."""
-        self._check(self._lib.aidn_mi355_set_attention_fast_path(self._ctx, 2 if enabled == 2 else (1 if enabled else 0)))
+        """Test hook: False routes every attention shape through the general kernel; 2 / 3 keep the fast paths and pin unsplit
+        head-dimension-128 prefill to the phase-structured / the software-pipelined kernel (True: chosen by pass length)."""
+        self._check(self._lib.aidn_mi355_set_attention_fast_path(self._ctx, int(enabled) if enabled in (2, 3) and enabled is not True else (1 if enabled else 0)))
 
     def ReserveWorkspace(self, size_in_bytes: int) -> None:
         """Grow the library workspace of the current stream now, so that later calls on it allocate nothing (needed before a

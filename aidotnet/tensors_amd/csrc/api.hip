@@ -423,7 +423,7 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile)
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled)
 {
     if (!ctx) return AIDN_ERR_INVALID_ARGUMENT;
-    ((Ctx*)ctx)->attn_fast_path = enabled == 2 ? 2 : (enabled != 0);
+    ((Ctx*)ctx)->attn_fast_path = (enabled == 2 || enabled == 3) ? enabled : (enabled != 0);
     return AIDN_OK;
 }
 

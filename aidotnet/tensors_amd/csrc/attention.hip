@@ -1174,10 +1174,20 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
             a.nsplit = ns; a.chunk = chunk; a.part = (float*)p.workspace;
         }
     }
-    if (dl && a.nsplit == 1 && p.allow_fast_path != 2) {
-        // unsplit prefill: the 16 x 16 x 32 kernel (allow_fast_path == 2, a test hook, keeps the 32 x 32 x 16 one below)
-        err = launch_attn_x16(kind, p.out16, a, stream);
-    } else
+    // Unsplit prefill has two kernels.  The software-pipelined one has the faster steady state and the longer way into and out of
+    // a pass, so it takes the shapes whose passes are long: at least 48 units of 32 keys per pass on average (measured: 1025
+    // against 975 TFLOP/s at 64 units, 373 against 452 at 10).  allow_fast_path 2 / 3 (test hooks) pin the choice.
+    bool pipelined = false;
+    if (dl && a.nsplit == 1 && (p.ks[2] * 2) % 256 == 0) {
+        long long keys = p.Sk;          // keys a query sees, averaged over the queries
+        if (p.causal) {
+            auto clampk = [&](long long x) { return x < 0 ? 0LL : (x > p.Sk ? (long long)p.Sk : x); };
+            keys = (clampk((long long)p.qoff + 1) + clampk((long long)p.qoff + p.Sq)) / 2;
+        }
+        pipelined = p.allow_fast_path == 3 || (p.allow_fast_path == 1 && keys >= 48 * 32);
+    }
+    if (pipelined) err = launch_attn_prefill(kind, p.out16, a, stream);
+    else
     if (dl) {
         if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t>(a, stream) : launch_attn_dl<f16_t, float>(a, stream);
         else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t>(a, stream) : launch_attn_dl<bf16_t, float>(a, stream);

@@ -119,7 +119,7 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
 }
 
 
-// 16-bit, head dimension 128, plain / causal attention on v_mfma_f32_16x16x32 (attention_x16.hip); kind: 1 fp16, 2 bf16
-hipError_t launch_attn_x16(int kind, int out16, AttnArgs a, hipStream_t stream);
+// 16-bit, head dimension 128, plain / causal attention in the software-pipelined form (attention_prefill.hip); kind: 1 fp16, 2 bf16
+hipError_t launch_attn_prefill(int kind, int out16, AttnArgs a, hipStream_t stream);
 
 }  // namespace aidn

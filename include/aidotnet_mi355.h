@@ -331,10 +331,10 @@ AIDN_API int aidn_mi355_mha_fwd_packed_bf16(void* ctx, void* stream, const uint1
  * reference. */
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
 /* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast
- * paths are then not taken), so the parity suite can hold the kernels against each other; enabled == 2
- * keeps the fast paths but runs unsplit head-dim-128 prefill on the 32 x 32 x 16 kernel instead of the
- * 16 x 16 x 32 one (each of the three is checked against the others).  Per context.  No counterpart in
- * the reference. */
+ * paths are then not taken), so the parity suite can hold the kernels against each other; unsplit
+ * head-dim-128 prefill has two kernels, chosen by the length of a pass: enabled == 2 pins the phase-structured
+ * one, enabled == 3 the software-pipelined one (each of the three is checked against the others).  Per context.
+ * No counterpart in the reference. */
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled);
 
 #ifdef __cplusplus

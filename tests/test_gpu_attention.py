@@ -363,7 +363,9 @@ def test_fast_path_d128_matches_oracle_and_general_kernel(be, kind, B, H, Hkv, S
     args = (be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)))
     outs = {}
     try:
-        for fast in (True, False):
+        # 2 / 3: the phase-structured / the software-pipelined prefill kernel (key ranges side by side where the shape asks for
+        # them in both); False: the general kernel
+        for fast in (2, 3, False):
             be.SetAttentionFastPath(fast)
             out = torch.full((B, H, Sq, D), float("nan"), device="cuda")
             lse = torch.full((B, H, Sq), float("nan"), device="cuda")
@@ -371,12 +373,13 @@ def test_fast_path_d128_matches_oracle_and_general_kernel(be, kind, B, H, Hkv, S
             outs[fast] = (out.cpu().numpy(), lse.cpu().numpy())
             assert mixed_err(outs[fast][0], o64) <= HALF_TOL
             assert mixed_err(outs[fast][1], lse64) <= 1e-3
-        # the two kernels agree far inside the 16-bit tolerance (both round P to 16 bits, at different scalings)
-        assert mixed_err(outs[True][0], outs[False][0]) <= 1e-2
-        be.SetAttentionFastPath(True)
-        out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
-        be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
-        assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
+        # the kernels agree far inside the 16-bit tolerance (all round P to 16 bits, at different scalings)
+        assert mixed_err(outs[2][0], outs[False][0]) <= 1e-2 and mixed_err(outs[3][0], outs[False][0]) <= 1e-2
+        for fast in (2, 3):
+            be.SetAttentionFastPath(fast)
+            out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
+            assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
     finally:
         be.SetAttentionFastPath(True)
 
@@ -392,13 +395,60 @@ def test_fast_path_all_masked_rows_and_large_logits(be):
         (qb, qw), (kb, kw), (vb, vw) = round_to(q, "bf16"), round_to(k, "bf16"), round_to(v, "bf16")
         o64, lse64 = oracle.attention_f64(qw, kw, vw, 0.5, True, -3)
         dt = torch.bfloat16
-        out = torch.full((B, H, S, D), float("nan"), device="cuda"); lse = torch.full((B, H, S), float("nan"), device="cuda")
-        be.FlashAttentionHalf("bf16", be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)),
-                              be.WrapTensor(out), be.WrapTensor(lse), B, H, S, S, D, 0.5, True, -3)
-        o = out.cpu().numpy(); l = lse.cpu().numpy()
-        assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
-        assert mixed_err(o, o64) <= HALF_TOL
-        assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
+        try:
+            for fast in (2, 3):         # (the pipelined kernel meets logits it cannot hold against a standing reference: its safe form)
+                be.SetAttentionFastPath(fast)
+                out = torch.full((B, H, S, D), float("nan"), device="cuda"); lse = torch.full((B, H, S), float("nan"), device="cuda")
+                be.FlashAttentionHalf("bf16", be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)),
+                                      be.WrapTensor(out), be.WrapTensor(lse), B, H, S, S, D, 0.5, True, -3)
+                o = out.cpu().numpy(); l = lse.cpu().numpy()
+                assert np.all(o[:, :, :3] == 0) and np.all(np.isneginf(l[:, :, :3]))
+                assert mixed_err(o, o64) <= HALF_TOL
+                assert mixed_err(l[:, :, 3:], lse64[:, :, 3:]) <= 1e-3
+        finally:
+            be.SetAttentionFastPath(True)
+
+
+LONG_PASS_CASES = [
+    # B, H, Hkv, Sq, Sk, causal, offset, q scale: passes long enough that every part of the pipelined kernel runs (the assembly loop
+    # through several rounds of both LDS stages, tile loads that end before the pass does, paired causal query tiles)
+    (1, 4, 4, 2048, 2048, True, 0, 1.0),
+    (1, 2, 1, 1024, 2048 + 37, False, 0, 1.0),      # partial last tile behind a long run
+    (1, 4, 2, 512, 4096, True, 3584, 1.0),          # chunked prefill against a long cache, GQA
+    (2, 2, 2, 1280, 1280, True, 0, 1.0),            # ten query tiles: paired
+    (1, 3, 3, 1152, 1152, True, 0, 1.0),            # nine query tiles: not paired
+    (1, 2, 2, 1024, 1024, True, 0, 40.0),           # logits far beyond what a standing reference holds: the safe form
+    (1, 2, 2, 700, 1900, False, 0, 25.0),
+]
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset,qscale", LONG_PASS_CASES)
+def test_pipelined_prefill_long_passes(be, kind, B, H, Hkv, Sq, Sk, causal, offset, qscale):
+    D = 128
+    rng = np.random.default_rng(5 * B + 3 * H + 7 * Sq + 11 * Sk + len(kind))
+    q, k, v = qscale * _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+    scale = 1.0 / math.sqrt(D)
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale, causal, offset)
+    dt = TORCH16[kind]
+    args = (be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)))
+    outs = {}
+    try:
+        for fast in (3, 2):
+            be.SetAttentionFastPath(fast)
+            out = torch.full((B, H, Sq, D), float("nan"), device="cuda")
+            lse = torch.full((B, H, Sq), float("nan"), device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out), be.WrapTensor(lse), B, H, Sq, Sk, D, scale, causal, offset, Hkv)
+            outs[fast] = (out.cpu().numpy(), lse.cpu().numpy())
+            assert mixed_err(outs[fast][0], o64) <= HALF_TOL
+            assert mixed_err(outs[fast][1], lse64) <= 1e-3
+            out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
+            assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
+        assert mixed_err(outs[3][0], outs[2][0]) <= 1e-2
+    finally:
+        be.SetAttentionFastPath(True)
 
 
 # --------------------------------------------------------------- fp32 head-dim-64 direct-to-LDS form of the general kernel
