@@ -1174,17 +1174,13 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
             a.nsplit = ns; a.chunk = chunk; a.part = (float*)p.workspace;
         }
     }
-    // Unsplit prefill has two kernels.  The software-pipelined one has the faster steady state and the longer way into and out of
-    // a pass, so it takes the shapes whose passes are long: at least 48 units of 32 keys per pass on average (measured: 1025
-    // against 975 TFLOP/s at 64 units, 373 against 452 at 10).  allow_fast_path 2 / 3 (test hooks) pin the choice.
+    // Unsplit prefill has two kernels.  The software-pipelined one is the faster (894 against 840 TFLOP/s on causal B4 H32 S2048 fp16,
+    // 1035 against 983 without the mask, 312 against 292 at S 128) except where a sequence ends inside a 64-key tile and the passes
+    // are short: the partial tile is then a larger share of a pass, and the pipelined kernel walks it in plain steps (509 against
+    // 530 at S 1100).  allow_fast_path 2 / 3 (test hooks) pin the choice.
     bool pipelined = false;
-    if (dl && a.nsplit == 1 && (p.ks[2] * 2) % 256 == 0) {
-        long long keys = p.Sk;          // keys a query sees, averaged over the queries
-        if (p.causal) {
-            auto clampk = [&](long long x) { return x < 0 ? 0LL : (x > p.Sk ? (long long)p.Sk : x); };
-            keys = (clampk((long long)p.qoff + 1) + clampk((long long)p.qoff + p.Sq)) / 2;
-        }
-        pipelined = p.allow_fast_path == 3 || (p.allow_fast_path == 1 && keys >= 48 * 32);
+    if (dl && a.nsplit == 1 && p.ks[2] == 128 && p.vs[2] == 128) {      // (its tile loads count on K and V rows 256 bytes apart)
+        pipelined = p.allow_fast_path == 3 || (p.allow_fast_path == 1 && (p.Sk % 64 == 0 || p.Sk >= 2048));
     }
     if (pipelined) err = launch_attn_prefill(kind, p.out16, a, stream);
     else

@@ -7,6 +7,17 @@
 
 namespace aidn {
 
+// Division of a 31-bit unsigned number by a divisor fixed at launch: q = (mulhi(x, m) + x) >> s with s = ceil(log2 d),
+// m = floor(2^32 (2^s - d) / d) + 1 (two scalar instructions and a shift where the compiler's general sequence takes about 25).
+struct FastDiv { uint32_t m, s; };
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    uint32_t s = 0;
+    while ((1ull << s) < d) s++;
+    return FastDiv{(uint32_t)((((1ull << s) - d) << 32) / d + 1), s};
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t x, FastDiv f) { return (__umulhi(x, f.m) + x) >> f.s; }
+
 struct AttnArgs {
     const void* q; const void* k; const void* v; void* o;
     float* lse; const float* bias; const float* mask;
@@ -15,6 +26,8 @@ struct AttnArgs {
     long long bias_bs;
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
+    int nvb;       // pipelined prefill kernel: virtual blocks (the grid's workgroups take them in turn)
+    FastDiv dH, dgroup, dunits, dqtiles;      // pipelined prefill kernel: H, H / Hkv, qtiles / 2, qtiles as divisors
     int hgroup;    // general kernel, causal: > 0 heads per group of the workgroup order of a large grid; < 0 the placement of a small one
     // fast kernel, grouped decode: the workgroup's key range is split `split` of nsplit (chunk keys each) and, when part is not
     // null, it stores its unnormalised partial (m, l, O[128]) at part + ((b H_q + head) nsplit + split) * 130 for the merge pass

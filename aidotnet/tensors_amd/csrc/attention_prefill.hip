@@ -32,35 +32,34 @@
 namespace aidn {
 
 #define PREFILL_HEAD_GROUP 4
-#ifndef PREFILL_RING
-#define PREFILL_RING 4
-#endif
 
 template <typename T, typename OutT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 {
     typedef uint16_t raw_t;
-    constexpr int BC = 64, BR = 128, R = PREFILL_RING;
+    constexpr int BC = 64, BR = 128;
     constexpr int KBYTES = BC * 256, VBYTES = BC * 256;
     constexpr float BIG = 1.152921504606847e18f;       // 2^60: a unit's probability sum beyond it means exp2 left the range
-    static_assert(16 % R == 0 && R >= 2, "the fragment ring is indexed i % R over the 16 MFMAs of an iteration");
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int l32 = lane & 31, h = lane >> 5;
-    int bh, qt;
-    {
-        int nblk = gridDim.x, pid = blockIdx.x;
+    // The grid is at most two workgroups per CU; a workgroup takes the virtual blocks blockIdx.x, blockIdx.x + gridDim.x, ... one
+    // after the other (so that the loads that open a pass can be issued while the pass before it is still storing), and, with
+    // paired causal query tiles, two passes per virtual block.  Item k of this workgroup -> (batch * head, query tile):
+    const int npass = a.paired ? 2 : 1;
+    auto decode = [&](int k, int& bh, int& qt) {
+        int nblk = a.nvb, pid = blockIdx.x + (k >> (npass - 1)) * gridDim.x;
         int per = nblk >> 3, rem = nblk & 7;
         int xcd = pid & 7, idx = pid >> 3;
         int logical = (xcd < rem ? xcd * (per + 1) : rem * (per + 1) + (xcd - rem) * per) + idx;
-        bh = logical / a.qtiles;
+        bh = (int)fastdiv((uint32_t)logical, a.dqtiles);
         qt = a.qtiles - 1 - (logical - bh * a.qtiles);
         if (a.paired) {
             // XCD-contiguous heads, qtiles / 2 workgroups per head: first the late (heavy) tile of the pair, then the early one
             const int units = a.qtiles >> 1;
-            bh = logical / units;
+            bh = (int)fastdiv((uint32_t)logical, a.dunits);
             qt = a.qtiles - 1 - (logical - bh * units);
         } else if (a.causal) {
             // heads in groups of PREFILL_HEAD_GROUP (their K and V are what an XCD's L2 holds); a group's query tiles heaviest first
@@ -75,7 +74,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             qt = a.qtiles - 1 - in / cur;
             bh = (whole ? xcd * heads : 0) + first + in % cur;
         }
-    }
+        if (npass == 2 && (k & 1)) qt = a.qtiles - 1 - qt;
+    };
+    const int nitems = (int)blockIdx.x < a.nvb ? ((a.nvb - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) * npass : 0;
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
@@ -93,25 +94,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     const uint32_t k_lane_off = (uint32_t)(ld_key * k_row_bytes) + ((ld_pos ^ ld_key) << 4);
     const uint32_t v_lane_off = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (ld_key << 2)) << 4);
 
-    const int npass = a.paired ? 2 : 1;
-    for (int pass = 0; pass < npass; pass++) {
-#ifdef PREFILL_DBG
-    unsigned long long stamp[8];
-#define STAMP(i) stamp[i] = __builtin_amdgcn_s_memtime()
-    STAMP(0);
-#else
-#define STAMP(i)
-#endif
-    if (pass == 1) qt = a.qtiles - 1 - qt;
-    const int b = bh / a.H, hd = bh - b * a.H;
-    const int kvh = hd / (a.H / a.Hkv);
-    const int q0 = qt * BR;
-    const int qi = q0 + wave * 32 + l32;
-    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
-    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
-    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
-
-    auto issue_k = [&](int tile) {
+    // tiles of the workgroup whose first query row is q0
+    auto tiles_of = [&](int q0) -> int {
+        int nt = (Sk + BC - 1) / BC;
+        if (a.causal) {
+            long long lastkey = (long long)q0 + BR - 1 + qoff;
+            if (lastkey < 0) nt = 0;
+            else { long long c = lastkey / BC + 1; if (c < nt) nt = (int)c; }
+        }
+        return nt;
+    };
+    auto issue_k = [&](const uint16_t* K, int tile) {
         const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * 4096;
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)K + (long long)(tile * BC + 16 * wave_s) * k_row_bytes;
@@ -129,7 +122,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             }
         }
     };
-    auto issue_v = [&](int tile) {
+    auto issue_v = [&](const uint16_t* V, int tile) {
         const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * 4096;
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
@@ -146,22 +139,56 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             }
         }
     };
-
-    // Q fragments (B operand of S^T = K Q^T): lane (l32, h) holds row l32, elements 16 s + 8 h .. + 7
-    u32x4 qf[8];
+    // What opens a pass and can be asked for while the pass before it is still storing: the Q fragments (B operand of
+    // S^T = K Q^T: lane (l32, h) holds row l32, elements 16 s + 8 h .. + 7) and the K tiles 0 and 1, which land in the K half of the
+    // tile memory (the stores stage through the V half).
+    typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+    u32x16 qlo, qhi;                        // k-steps 0..3 and 4..7 (held the way the assembly loop takes them)
+    auto qfrag = [&](int s) -> u32x4 {
+        return s < 4 ? u32x4{qlo[4 * s], qlo[4 * s + 1], qlo[4 * s + 2], qlo[4 * s + 3]}
+                     : u32x4{qhi[4 * s - 16], qhi[4 * s - 15], qhi[4 * s - 14], qhi[4 * s - 13]};
+    };
+    auto open_pass = [&](int bh, int qt) {
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int b = (int)fastdiv((uint32_t)bh, a.dH), hd = bh - b * a.H;
+        const int kvh = (int)fastdiv((uint32_t)hd, a.dgroup);
+        const int qrow = qt * BR + wave_s * 32 + (ln & 31);
+        const uint16_t* Q = (const uint16_t*)a.q + b * a.qs[0] + hd * a.qs[1] + (long long)qrow * a.qs[2] + (ln >> 5) * 8;
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        u32x4 z = {0u, 0u, 0u, 0u};
-        qf[s] = (qi < a.Sq) ? *(const u32x4*)(Q + (long long)qi * a.qs[2] + (2 * s + h) * 8) : z;
-    }
+        for (int s = 0; s < 8; s++) {
+            u32x4 z = {0u, 0u, 0u, 0u};
+            const u32x4 x = (qrow < a.Sq) ? *(const u32x4*)(Q + 16 * s) : z;
+#pragma unroll
+            for (int e = 0; e < 4; e++) { if (s < 4) qlo[4 * s + e] = x[e]; else qhi[4 * s - 16 + e] = x[e]; }
+        }
+        const uint16_t* K = (const uint16_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+        const int nt = tiles_of(qt * BR);
+        if (nt > 0) issue_k(K, 0);
+        if (nt > 1) issue_k(K, 1);
+    };
+
+    int bh = 0, qt = 0;
+    if (nitems > 0) { decode(0, bh, qt); open_pass(bh, qt); }
+    for (int item = 0; item < nitems; item++) {
+    const int pass = item & 1;
+#ifdef PREFILL_DBG
+    unsigned long long stamp[12];
+#define STAMP(i) stamp[i] = __builtin_amdgcn_s_memtime()
+    STAMP(0);
+#else
+#define STAMP(i)
+#endif
+    const int b = (int)fastdiv((uint32_t)bh, a.dH), hd = bh - b * a.H;
+    const int kvh = (int)fastdiv((uint32_t)hd, a.dgroup);
+    const int q0 = qt * BR;
+    const int qi = q0 + wave * 32 + l32;
+    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
+    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
 
     // tiles of the workgroup, units (32 keys) of this wave
-    int ntiles = (Sk + BC - 1) / BC;
-    if (a.causal) {
-        long long lastkey = (long long)q0 + BR - 1 + qoff;
-        if (lastkey < 0) ntiles = 0;
-        else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
-    }
+    const int ntiles = tiles_of(q0);
     const int wq_min = q0 + wave_s * 32, wq_max = wq_min + 31;
     auto key_limit = [&](int q) -> int {        // last key query q may see (sequence end and causal diagonal in one bound)
         long long lim = Sk - 1;
@@ -224,7 +251,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     u32x4 pf[2];                   // [16-key half]: packed probabilities of one unit, the B operand of the P V step
     float m_ref = -INFINITY;       // reference point of the exponent (log2 domain); the same in lanes l and l ^ 32
     float l_run = 0.0f;
-    u32x4 fr[R];                   // fragment ring of the interleaved block, carried from block to block
 
     // ---- plain (not interleaved) forms of the three steps of a unit
     auto qk_plain = [&]() {                                    // S of the unit the K addresses point to
@@ -232,15 +258,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            Mma32<T>::run(sacc, k_frag(s), qf[s]);
-            if (s & 1) __builtin_amdgcn_sched_barrier(0);
+            Mma32<T>::run(sacc, k_frag(s), qfrag(s));
+            if (s == 3) __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto pv_plain = [&]() {                                    // O += V^T P^T, unit the V addresses point to
 #pragma unroll
         for (int s = 0; s < 8; s++) {
             Mma32<T>::run(oacc[s & 3], v_frag(s), pf[s >> 2]);
-            if (s & 1) __builtin_amdgcn_sched_barrier(0);
+            if (s == 3) __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto mask_unit = [&](int u) {
@@ -251,13 +277,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     };
     // Probabilities of unit u with the row maxima formed first (the safe form, also the wave's first unit in the fast form): the
     // reference of a row is raised when the row's maximum lies more than 8 above it (always on first use).  Adds the row sums to l.
-    auto softmax_exact = [&](int u, bool apply_mask) {
+    auto softmax_exact = [&](int u, bool apply_mask, bool first) {
         if (apply_mask) mask_unit(u);
         float m = -INFINITY;
 #pragma unroll
         for (int r = 0; r < 16; r++) m = fmaxf(m, sacc[r]);
         const float mloc = max_with_partner32(m) * sl2;            // scale > 0: max commutes with the scaling
-        if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
+        if (first) {
+            m_ref = mloc < INFINITY ? mloc : -INFINITY;            // nothing accumulated yet: no O or l to move
+        } else if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
             const float m_new = (mloc > m_ref + 8.0f && mloc < INFINITY) ? mloc : m_ref;
             const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
             m_ref = m_new;
@@ -283,81 +311,68 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     // the tiles they replace went out of use at the barrier just passed), after an even unit the barrier that publishes K(t+1), V(t)
     auto unit_loads = [&](int u) {
         const int tl = u >> 1;
-        if (tl + 2 < ntiles) issue_k(tl + 2);
-        if (tl + 1 < ntiles) issue_v(tl + 1);
+        if (tl + 2 < ntiles) issue_k(K, tl + 2);
+        if (tl + 1 < ntiles) issue_v(V, tl + 1);
     };
     auto tile_barrier = [&]() {
         __builtin_amdgcn_s_waitcnt(0);      // this wave's loads have landed, its fragment reads are in registers ...
         __syncthreads();                    // ... everyone's
     };
 
-    // ---- the interleaved block of unit u (sacc holds S(u), pf holds P(u-1), the V addresses point at unit u-1, the K addresses at
-    // unit u+1, the ring holds the first R-1 fragments): the matrix pipe runs P(u-1) V, then S(u+1); beside the first the vector
-    // pipe turns the logits of unit u into exponentials in place (FMA + exp2 against the standing reference, two logits per MFMA);
-    // between the two it packs them into the P buffer, which the P V step has finished reading, and sums them; S(u+1) then lands
-    // in the registers the logits have left.  Once the block's last fragment read is issued the addresses move on, an even unit
-    // passes the tile barrier, and the reads that follow fetch the first fragments of the next block.  An odd unit issues the tile
-    // loads (dma) one per MFMA.  Returns the unit's row sums.
-    auto full_block = [&](int u, bool dma) -> float {
-        // fragment stream of the block: V^T fragments 0 .. 7, then K fragments 0 .. 7
-        auto frag = [&](int j) -> u32x4 { return j < 8 ? v_frag(j) : k_frag(j - 8); };
-        const int tile_k = (u >> 1) + 2, tile_v = (u >> 1) + 1;
-        const unsigned char* ksrc = (const unsigned char*)K + (long long)(tile_k * BC + 16 * wave_s) * k_row_bytes;
-        const unsigned char* vsrc = (const unsigned char*)V + (long long)(tile_v * BC + 16 * wave_s) * v_row_bytes;
-        const uint32_t kdst = lds0 + (tile_k & 1) * KBYTES + wave_s * 4096;
-        const uint32_t vdst = lds0 + 2 * KBYTES + (tile_v & 1) * VBYTES + wave_s * 4096;
-        const float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
-        float ps = 0.0f;
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            if (i == 16 - (R - 1)) {
-                // every fragment of this block is requested: on to the next units
-                next_k_unit();
-                next_v_unit();
-                if (!(u & 1)) tile_barrier();
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            // the fragment R - 1 MFMAs ahead; past the end of this block it is one of the first of the next block
-            fr[(i + R - 1) % R] = frag((i + R - 1) % 16);
-            if (i < 8) {
-                Mma32<T>::run(oacc[i & 3], fr[i % R], pf[i >> 2]);
-                float e0 = __builtin_amdgcn_exp2f(fmaf(sacc[2 * i], sl2, -m_use));
-                float e1 = __builtin_amdgcn_exp2f(fmaf(sacc[2 * i + 1], sl2, -m_use));
-                asm volatile("" : "+v"(e0), "+v"(e1));
-                sacc[2 * i] = e0;
-                sacc[2 * i + 1] = e1;
-                if (dma) {
-                    if (i < 4) attn_dma16_base(ksrc + 4 * i * k_row_bytes, k_lane_off ^ (uint32_t)(i << 6), kdst + i * 1024);
-                    else attn_dma16_base(vsrc + 4 * (i - 4) * v_row_bytes, v_lane_off, vdst + (i - 4) * 1024);
-                }
-            } else {
-                const int s = i - 8;
-                if (s == 0) {
-                    // every P V MFMA has been issued: P(u) takes the buffer, then S(u+1) the registers of the exponentials
-#pragma unroll
-                    for (int pi = 0; pi < 8; pi++) {
-                        uint32_t pk = pack2_p<T>(sacc[2 * pi], sacc[2 * pi + 1]);
-                        ps = add_pair<T>(pk, ps);
-                        pf[pi >> 2][pi & 3] = pk;
-                    }
-                    asm volatile("" : "+v"(ps));
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
-                }
-                Mma32<T>::run(sacc, fr[i % R], qf[s]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        }
-        return ps;
-    };
-
     // The workgroup's loads: K(0), V(0), K(1) up front; before every odd unit K(t+2) and V(t+1), after every even unit the tile
     // barrier.  Fast form: unit 0 is done in plain steps (its row maxima set the reference of every row), units 1 .. take the
     // interleaved block, which forms the probabilities against that standing reference.  Should a probability leave the range of
     // exp2 (seen in the row sums at the end), the pass is run again in the safe form, which forms the row maxima of every unit.
-    uint32_t* const redo_flag = (uint32_t*)smem;       // one word per wave, in the tile memory once the tiles are done with
+    // Runs of whole unmasked units go through the assembly form of the block (attention_prefill_loop.inc: the same steps, every
+    // LDS offset an immediate, no instruction that is not needed).  run_units(u, n, loads): units u .. u + n - 1 with sacc, pf,
+    // the addresses and l as the C++ block would find and leave them; the first k_loads / v_loads odd units of the run issue the
+    // loads of K(t+2) / V(t+1), which have to be whole tiles.
+    auto run_units = [&](int u, int n, int k_loads, int v_loads, bool masked_last) {
+        typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
+        // read addresses of unit 0 (the K addresses stand at unit u + 1, the V addresses at unit u - 1)
+        const uint32_t koff = (uint32_t)((u + 1) & 3) << 13, voff = (uint32_t)((u - 1) & 3) << 13;
+        const u32x4 kad0 = {k_ad[0] ^ koff, k_ad[1] ^ koff, k_ad[2] ^ koff, k_ad[3] ^ koff};
+        const u32x4 kad1 = {kad0[0] ^ 128u, kad0[1] ^ 128u, kad0[2] ^ 128u, kad0[3] ^ 128u};
+        const u32x4 vad = {v_ad[0] ^ voff, v_ad[1] ^ voff, v_ad[2] ^ voff, v_ad[3] ^ voff};
+        const u32x4 klo = {k_lane_off, k_lane_off ^ 64u, k_lane_off ^ 128u, k_lane_off ^ 192u};
+        const uint32_t vlo = v_lane_off;
+        const float negm = (m_ref == -INFINITY) ? -0.0f : -m_ref;
+        float ps = 0.0f;
+        const int tl = u >> 1;
+        unsigned long long kptr = (unsigned long long)(uintptr_t)((const unsigned char*)K + (long long)((tl + 2) * BC + 16 * wave_s) * k_row_bytes);
+        unsigned long long vptr = (unsigned long long)(uintptr_t)((const unsigned char*)V + (long long)((tl + 1) * BC + 16 * wave_s) * v_row_bytes);
+        const unsigned long long ktile = (unsigned long long)(BC * k_row_bytes), vtile = (unsigned long long)(BC * v_row_bytes);
+        const u32x8 sc = {(uint32_t)(4 * k_row_bytes), (uint32_t)(4 * v_row_bytes), (uint32_t)ktile, (uint32_t)(ktile >> 32),
+                          (uint32_t)vtile, (uint32_t)(vtile >> 32), lds0 + wave_s * 4096u, lds0 + 2 * KBYTES + wave_s * 4096u};
+        const float sl2s = sl2;
+        int count = __builtin_amdgcn_readfirstlane(n);
+        int kleft = __builtin_amdgcn_readfirstlane(k_loads), vleft = __builtin_amdgcn_readfirstlane(v_loads);
+        const int phase = __builtin_amdgcn_readfirstlane((u - 1) & 3);
+        // (with masked_last the run is n whole units and then unit u + n, masked first; n >= 1)
+        int mask_follows = __builtin_amdgcn_readfirstlane(masked_last ? 1 : 0);
+        const int mask_rel = klim - 32 * (u + n);
+        const float ninf = -INFINITY;
+        if (masked_last) n++;
+        u32x4 p0 = pf[0], p1 = pf[1];
+#define PREFILL_LOOP_OPERANDS \
+            : "+{v[0:15]}"(oacc[0]), "+{v[16:31]}"(oacc[1]), "+{v[32:47]}"(oacc[2]), "+{v[48:63]}"(oacc[3]), "+{v[64:79]}"(sacc), \
+              "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v170}"(ps), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft), "+{s59}"(mask_follows) \
+            : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad0), "{v[156:159]}"(kad1), "{v[160:163]}"(vad), \
+              "{v[164:167]}"(klo), "{v168}"(vlo), "{v169}"(negm), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), "{v171}"(mask_rel), "{v174}"(ninf) \
+            : "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", \
+              "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \
+              "v150", "v151", "v172", "v173", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", \
+              "v187", "v188", "v189", "v190", "v191", "s54", "s55", "scc", "vcc", "memory"
+        if constexpr (std::is_same<T, f16_t>::value) asm volatile(PREFILL_LOOP_F16 PREFILL_LOOP_OPERANDS);
+        else asm volatile(PREFILL_LOOP_BF16 PREFILL_LOOP_OPERANDS);
+#undef PREFILL_LOOP_OPERANDS
+        pf[0] = p0; pf[1] = p1;
+        l_run += ps;
+        for (int i = 0; i < (n & 3); i++) { next_k_unit(); next_v_unit(); }
+        k_unit += n & ~3; v_unit += n & ~3;
+    };
+    // one word per wave behind the tile memory, a set of four per (pass, attempt) parity so that no set is cleared or reused early
+    uint32_t* const redo_flag = (uint32_t*)(smem + 2 * KBYTES + 4 * 32 * 272) + 4 * (pass & 1);
     const int nunits = 2 * ntiles;
     for (int attempt = 0; attempt < 2; attempt++) {
     const bool safe = attempt == 1;
@@ -368,176 +383,124 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #pragma unroll
     for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
     pf[0] = u32x4{0u, 0u, 0u, 0u}; pf[1] = u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int i = 0; i < R; i++) fr[i] = u32x4{0u, 0u, 0u, 0u};
     m_ref = -INFINITY; l_run = 0.0f;
     while (k_unit & 3) next_k_unit();           // (a second attempt starts from unit 0 again)
     while (v_unit & 3) next_v_unit();
     k_unit = 0; v_unit = 0;
-    if (ntiles > 0) { issue_k(0); issue_v(0); }
-    if (ntiles > 1) issue_k(1);
-    tile_barrier();
+    if (!safe) {
+        // Q, K(0) and K(1) are on their way (open_pass); V(0) is asked for now and waited for only after S(0), P(0) and S(1): the
+        // wait below leaves this wave's last four loads, which are those of V(0), outstanding (loads complete in issue order)
+        if (ntiles > 0) { issue_v(V, 0); asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); }
+        else __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    } else {
+        if (ntiles > 0) { issue_k(K, 0); issue_v(V, 0); }
+        if (ntiles > 1) issue_k(K, 1);
+        tile_barrier();
+    }
     STAMP(1);
     if (nu > 0) qk_plain();                     // S(0)
-    next_k_unit();
-    if (!safe) {
-        if (nu > 0) softmax_exact(0, 0 > ufull);                // P(0); sets the reference of every row
-        if (nu > 1) qk_plain();                                 // S(1)
-        next_k_unit();                                          // K addresses at unit 2, V addresses at unit 0: block 1 may start
-        if (nunits > 1) {
-            __syncthreads();                                    // everyone is done with the first half of K(0), which K(2) replaces
-            if (1 < nu) {
-#pragma unroll
-                for (int j = 0; j < R - 1; j++) fr[j] = v_frag(j);
-            }
-        }
-        // Runs of whole unmasked units go through the assembly form of the block (attention_prefill_loop.inc: the same steps, every
-        // LDS offset an immediate, no instruction that is not needed).  run_units(u, n, loads): units u .. u + n - 1 with sacc, pf,
-        // the addresses and l as the C++ block would find and leave them; the first k_loads / v_loads odd units of the run issue the
-        // loads of K(t+2) / V(t+1), which have to be whole tiles.
-        auto run_units = [&](int u, int n, int k_loads, int v_loads) {
-            typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-            typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
-            u32x16 qlo, qhi;
-#pragma unroll
-            for (int s4 = 0; s4 < 4; s4++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) { qlo[4 * s4 + e] = qf[s4][e]; qhi[4 * s4 + e] = qf[4 + s4][e]; }
-            // read addresses of unit 0 (the K addresses stand at unit u + 1, the V addresses at unit u - 1)
-            const uint32_t koff = (uint32_t)((u + 1) & 3) << 13, voff = (uint32_t)((u - 1) & 3) << 13;
-            const u32x4 kad0 = {k_ad[0] ^ koff, k_ad[1] ^ koff, k_ad[2] ^ koff, k_ad[3] ^ koff};
-            const u32x4 kad1 = {kad0[0] ^ 128u, kad0[1] ^ 128u, kad0[2] ^ 128u, kad0[3] ^ 128u};
-            const u32x4 vad = {v_ad[0] ^ voff, v_ad[1] ^ voff, v_ad[2] ^ voff, v_ad[3] ^ voff};
-            const u32x4 klo = {k_lane_off, k_lane_off ^ 64u, k_lane_off ^ 128u, k_lane_off ^ 192u};
-            const uint32_t vlo = v_lane_off;
-            const float negm = (m_ref == -INFINITY) ? -0.0f : -m_ref;
-            float ps = 0.0f;
-            const int tl = u >> 1;
-            unsigned long long kptr = (unsigned long long)(uintptr_t)((const unsigned char*)K + (long long)((tl + 2) * BC + 16 * wave_s) * k_row_bytes);
-            unsigned long long vptr = (unsigned long long)(uintptr_t)((const unsigned char*)V + (long long)((tl + 1) * BC + 16 * wave_s) * v_row_bytes);
-            const unsigned long long ktile = (unsigned long long)(BC * k_row_bytes), vtile = (unsigned long long)(BC * v_row_bytes);
-            const u32x8 sc = {(uint32_t)(4 * k_row_bytes), (uint32_t)(4 * v_row_bytes), (uint32_t)ktile, (uint32_t)(ktile >> 32),
-                              (uint32_t)vtile, (uint32_t)(vtile >> 32), lds0 + wave_s * 4096u, lds0 + 2 * KBYTES + wave_s * 4096u};
-            const float sl2s = sl2;
-            int count = __builtin_amdgcn_readfirstlane(n);
-            int kleft = __builtin_amdgcn_readfirstlane(k_loads), vleft = __builtin_amdgcn_readfirstlane(v_loads);
-            const int phase = __builtin_amdgcn_readfirstlane((u - 1) & 3);
-            u32x4 p0 = pf[0], p1 = pf[1];
-#define PREFILL_LOOP_OPERANDS \
-                : "+{v[0:15]}"(oacc[0]), "+{v[16:31]}"(oacc[1]), "+{v[32:47]}"(oacc[2]), "+{v[48:63]}"(oacc[3]), "+{v[64:79]}"(sacc), \
-                  "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v170}"(ps), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft) \
-                : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad0), "{v[156:159]}"(kad1), "{v[160:163]}"(vad), \
-                  "{v[164:167]}"(klo), "{v168}"(vlo), "{v169}"(negm), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase) \
-                : "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", \
-                  "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \
-                  "v150", "v151", "v172", "v173", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", \
-                  "v187", "v188", "v189", "v190", "v191", "s54", "s55", "scc", "vcc", "memory"
-            if constexpr (std::is_same<T, f16_t>::value) asm volatile(PREFILL_LOOP_F16 PREFILL_LOOP_OPERANDS);
-            else asm volatile(PREFILL_LOOP_BF16 PREFILL_LOOP_OPERANDS);
-#undef PREFILL_LOOP_OPERANDS
-            pf[0] = p0; pf[1] = p1;
-            l_run += ps;
-            for (int i = 0; i < (n & 3); i++) { next_k_unit(); next_v_unit(); }
-            k_unit += n & ~3; v_unit += n & ~3;
-        };
-        int u_first = 1;
-        STAMP(2);
-        {
-            // one run: units 1 .. u_last, whole, unmasked, with a successor; it ends ahead of the odd unit that would have to load a
-            // partial tile (the last tile of a sequence that is not a multiple of 64 keys long)
+    next_k_unit();                              // K addresses at unit 1, V addresses at unit 0
+    int u = 0;
+    while (u < nunits) {
+        if (!safe && u == 1) {
+            // one run of the assembly loop: units 1 .. u_last, whole, unmasked, with a successor; it ends ahead of the odd unit
+            // that would have to load a partial tile (the last tile of a sequence that is not a multiple of 64 keys long)
             const int whole = min(ntiles, Sk / BC);                 // the workgroup's tiles 0 .. whole - 1 are whole tiles
             int u_last = min(ufull, nu - 1);
             if (whole < ntiles) u_last = min(u_last, 2 * (whole - 2));      // unit 2 (whole - 2) + 1 loads tile `whole` as its K tile
             if (u_last >= 1) {
+                // the unit on the causal diagonal goes with the run when it is the wave's last unit and no partial tile is about
+                const bool with_diagonal = u_last == ufull && ufull + 2 == nu && whole == ntiles;
                 // odd unit 2 t + 1 loads K(t + 2) for t <= whole - 3 and V(t + 1) for t <= whole - 2
-                run_units(1, u_last, max(0, whole - 2), max(0, whole - 1));
-                u_first = u_last + 1;
-                if (u_first < nu) {
-#pragma unroll
-                    for (int j = 0; j < R - 1; j++) fr[j] = v_frag(j);
-                }
+                STAMP(2);
+                run_units(1, u_last, max(0, whole - 2), max(0, whole - 1), with_diagonal);
+                STAMP(3);
+                u = u_last + 1 + (with_diagonal ? 1 : 0);
+                continue;
             }
         }
-        STAMP(3);
-        for (int u = u_first; u < nunits; u++) {
-            const int tl = u >> 1;
-            const bool fast_loads = (u & 1) && tl + 2 < ntiles && (tl + 2) * BC + BC <= Sk && (tl + 1) * BC + BC <= Sk;
-            if ((u & 1) && !fast_loads) unit_loads(u);
-            if (u < nu) {
-                if (u > ufull) mask_unit(u);
-                l_run += full_block(u, fast_loads);
-            } else {
-                if (u == nu) pv_plain();
-                next_k_unit();
-                next_v_unit();
-                if ((u & 1) && fast_loads) unit_loads(u);
-                if (!(u & 1)) tile_barrier();
-            }
+        // the steps of unit u one after the other, row maxima formed first: P(u-1) V, P(u), S(u+1)
+        if (u & 1) unit_loads(u);
+        if (u >= 1) {
+            if (u - 1 < nu) pv_plain();
+            next_v_unit();
         }
-        if (nunits == nu && nunits > 0) pv_plain();             // P V of the workgroup's last unit
-        STAMP(4);
+        if (u < nu) softmax_exact(u, u > ufull, u == 0);
+        if (u + 1 < nu) qk_plain();
+        next_k_unit();
+        if (!(u & 1)) tile_barrier();
+        u++;
+    }
+    if (nunits - 1 < nu && nunits > 0) pv_plain();              // P V of the workgroup's last unit
+    STAMP(4);
+    if (!safe) {
         const bool left_range = __builtin_amdgcn_ballot_w64(!(l_run < 1.2676506e30f)) != 0ull;
-        __syncthreads();                        // every wave is past its last fragment read
         if (lane == 0) redo_flag[wave] = left_range ? 1u : 0u;
-        __syncthreads();
-        const bool redo = (redo_flag[0] | redo_flag[1] | redo_flag[2] | redo_flag[3]) != 0u;
-#ifdef PREFILL_NO_REDO
-        break;
-#endif
-        if (!redo) break;
-        __syncthreads();                        // everyone has read the flags before the next attempt's loads land on them
+        __syncthreads();                        // the flags are written, and every wave is past its last fragment read
+        const u32x4 fl = *(const u32x4*)redo_flag;
+        if (__builtin_amdgcn_readfirstlane((fl[0] | fl[1] | fl[2] | fl[3])) == 0u) break;
     } else {
-        // K addresses at unit 1, V addresses at unit 0
-        for (int u = 0; u < nunits; u++) {
-            if (u & 1) unit_loads(u);
-            if (u >= 1) {
-                if (u - 1 < nu) pv_plain();
-                next_v_unit();
-            }
-            if (u < nu) softmax_exact(u, u > ufull);
-            if (u + 1 < nu) qk_plain();
-            next_k_unit();
-            if (!(u & 1)) tile_barrier();
-        }
-        if (nunits - 1 < nu && nunits > 0) pv_plain();
+        __syncthreads();                        // every wave is past its last fragment read
     }
     }   // attempt
 
-    // ---- epilogue: normalise, store
+    // ---- the next pass is opened (every wave is past its last fragment read, see the end of the attempts)
     STAMP(5);
+    int bh_next = 0, qt_next = 0;
+    if (item + 1 < nitems) { decode(item + 1, bh_next, qt_next); open_pass(bh_next, qt_next); }
+    STAMP(8);
+    // ---- epilogue: normalise, store
     const float l_tot = sum_with_partner32(l_run);
     const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
     if (Elem<OutT>::BYTES == 4 && a.vec_out) {
         // fp32 O through LDS: the lane holds 16-byte pieces of ONE row (64 rows per store instruction, each a partial line); staged
-        // per wave as [32 rows][512 B] (chunk c of row r at position c ^ r, conflict-free both ways) and written back as whole
-        // 512-byte rows with non-temporal stores (O is written once and would otherwise displace K and V tiles that other
-        // workgroups re-read).  The tile memory is free only when every wave is past its last fragment read: barrier first.
-        __syncthreads();
-        unsigned char* stg = smem + wave_s * 16384;
-        int lnw = lane;
-        asm volatile("" : "+v"(lnw));
-        const int l32w = lnw & 31, hw = lnw >> 5;
+        // per wave, one half of the head dimension at a time, as [32 rows][256 B + 16] (the pad keeps neighbouring rows on different
+        // banks, and leaves every LDS address a lane constant plus an immediate) in the V half of the tile memory (the K half is
+        // receiving the next pass's tiles) and written back as 256-byte row halves, whole lines, with non-temporal stores (O is
+        // written once and would otherwise displace K and V tiles that other workgroups re-read).
+        constexpr int SROW = 272;
+        unsigned char* stg = smem + 2 * KBYTES + wave_s * (32 * SROW);
 #pragma unroll
         for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int c = 8 * i + 2 * g + hw;
-                *(f32x4*)(stg + l32w * 512 + ((c ^ l32w) << 4)) =
-                    f32x4{oacc[i][4 * g + 0] * inv, oacc[i][4 * g + 1] * inv, oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv};
-            }
+            for (int r = 0; r < 16; r++) oacc[i][r] *= inv;
         if (a.lse && h == 0 && qi < a.Sq)
             a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
-        // (row and chunk from an opaque copy of the lane index: the store addresses are then formed here, not ahead of the loops)
-        int lne = lane;
-        asm volatile("" : "+v"(lne));
-        const int c = lne & 31;
+        // (lane constants from an opaque copy of the lane index: they are then formed here, not ahead of the loops)
+        int lnw = lane;
+        asm volatile("" : "+v"(lnw));
+        unsigned char* wr = stg + (lnw & 31) * SROW + (lnw >> 5) * 16;                  // chunk 8 (i % 2) + 2 g + h of row l32
+        const unsigned char* rd = stg + (lnw >> 4) * SROW + (lnw & 15) * 16;           // chunk lane % 16 of row 4 q + lane / 16
+        // the wave's 32 output rows: a uniform base, a 32-bit lane offset (the launcher checks that 32 rows span less than 4 GB)
+        unsigned char* obase = (unsigned char*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)(q0 + wave_s * 32) * a.os[2]);
+        const uint32_t row_bytes = (uint32_t)a.os[2] * 4u;
+        const uint32_t lane_off = (uint32_t)(lnw >> 4) * row_bytes + (uint32_t)(lnw & 15) * 16u;
+        const int rows_left = a.Sq - (q0 + wave_s * 32);                                // rows of the wave inside the sequence
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-            const int r = 2 * q + (lne >> 5);
-            const int row = q0 + wave_s * 32 + r;
-            const f32x4 v = *(const f32x4*)(stg + r * 512 + ((c ^ r) << 4));
-            f32x4* dst = (f32x4*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)row * a.os[2] + c * 4);
-            if (row < a.Sq) __builtin_nontemporal_store(v, dst);
+        for (int half = 0; half < 2; half++) {
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    *(f32x4*)(wr + (8 * i + 2 * g) * 16) = f32x4{oacc[2 * half + i][4 * g + 0], oacc[2 * half + i][4 * g + 1],
+                                                                 oacc[2 * half + i][4 * g + 2], oacc[2 * half + i][4 * g + 3]};
+            f32x4 piece[8];
+#pragma unroll
+            for (int q = 0; q < 8; q++) piece[q] = *(const f32x4*)(rd + 4 * q * SROW);
+            if (rows_left >= 32) {
+#pragma unroll
+                for (int q = 0; q < 8; q++)
+                    __builtin_nontemporal_store(piece[q], (f32x4*)(obase + (size_t)(4 * q) * row_bytes + 256 * half + lane_off));
+            } else {
+#pragma unroll
+                for (int q = 0; q < 8; q++)
+                    if (4 * q + (lnw >> 4) < rows_left)
+                        __builtin_nontemporal_store(piece[q], (f32x4*)(obase + (size_t)(4 * q) * row_bytes + 256 * half + lane_off));
+            }
+#ifdef PREFILL_DBG
+            if (half == 0) STAMP(9);
+#endif
         }
     } else if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
@@ -570,33 +533,50 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         float dv = (float)(stamp[0] & 0xFFFFFFull);
 #pragma unroll
         for (int i = 1; i < 8; i++) if (lane == i) dv = (float)(long long)(stamp[i] - stamp[i - 1]);
-        if (a.lse && lane < 8) a.lse[(long long)bh * a.Sq + q0 + wave_s * 32 + lane] = dv;
+        if (lane == 8) dv = (float)(long long)(stamp[8] - stamp[5]);
+        if (lane == 9) dv = (float)(long long)(stamp[9] - stamp[8]);
+        if (lane == 10) dv = (float)(long long)(stamp[6] - stamp[9]);
+        if (a.lse && lane < 11) a.lse[(long long)bh * a.Sq + q0 + wave_s * 32 + lane] = dv;
     }
 #endif
-    if (npass > 1) __syncthreads();      // the next pass's loads must not overtake this pass's last LDS reads
-    }   // pass
+    if (item + 1 < nitems) {
+        __syncthreads();                 // the next pass's V(0) must not land on rows that are still being staged
+        bh = bh_next; qt = qt_next;
+    }
+    }   // item
 }
 
 template <typename T, typename OutT>
 static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
 {
     auto kern = attn_prefill_kernel<T, OutT>;
-    constexpr int smem = 2 * (64 * 256 + 64 * 256);
+    constexpr int smem = 2 * 64 * 256 + 4 * 32 * 272 + 64;     // K tiles, two stages; V tiles, two stages, or the padded rows of O on their way out; the redo flags
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
+    if (a.os[2] * 4 * 32 >= 0xFFFFFFFFLL || a.os[2] < 0) return hipErrorInvalidValue;     // the lane offsets of the O stores are 32 bits
     // causal self-attention with an even number of query tiles: tile i and tile qtiles-1-i in one workgroup (equal work everywhere)
     a.paired = (a.causal && a.qoff == 0 && a.Sq == a.Sk && a.qtiles >= 2 && a.qtiles % 2 == 0) ? 1 : 0;
     const long long nblk = (long long)(a.paired ? a.qtiles / 2 : a.qtiles) * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL || nblk <= 0) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblk), dim3(256), smem, stream, a);
+    // two workgroups fit a CU (LDS): that many run at once, each taking its virtual blocks in turn (a multiple of the eight
+    // XCDs, which the block order counts on)
+    int dev = 0, cus = 0;
+    if (hipError_t e = hipGetDevice(&dev)) return e;
+    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+    const long long resident = (long long)(2 * cus) / 8 * 8;
+    a.nvb = (int)nblk;
+    a.dH = make_fastdiv((uint32_t)a.H); a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));
+    a.dunits = make_fastdiv((uint32_t)(a.qtiles / 2 > 0 ? a.qtiles / 2 : 1)); a.dqtiles = make_fastdiv((uint32_t)a.qtiles);
+    const unsigned grid = (unsigned)((resident >= 8 && nblk > resident) ? resident : nblk);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, a);
     return hipGetLastError();
 }
 
 hipError_t launch_attn_prefill(int kind, int out16, AttnArgs a, hipStream_t stream)
 {
     if (a.D != 128 || a.nsplit > 1 || a.part || a.stream || a.bt || !(a.scale > 0.0f)) return hipErrorInvalidValue;
-    if ((a.ks[2] * 2) % 256 != 0) return hipErrorInvalidValue;      // the lane offsets of the K wave-loads are formed by XOR
+    if (a.ks[2] != 128 || a.vs[2] != 128) return hipErrorInvalidValue;     // the tile loads count on K and V rows 256 bytes apart
     if (kind == 1) return out16 ? launch_prefill<f16_t, f16_t>(a, stream) : launch_prefill<f16_t, float>(a, stream);
     if (kind == 2) return out16 ? launch_prefill<bf16_t, bf16_t>(a, stream) : launch_prefill<bf16_t, float>(a, stream);
     return hipErrorInvalidValue;
