@@ -1179,7 +1179,7 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
     // are short: the partial tile is then a larger share of a pass, and the pipelined kernel walks it in plain steps (509 against
     // 530 at S 1100).  allow_fast_path 2 / 3 (test hooks) pin the choice.
     bool pipelined = false;
-    if (dl && a.nsplit == 1 && p.ks[2] == 128 && p.vs[2] == 128) {      // (its tile loads count on K and V rows 256 bytes apart)
+    if (dl && a.nsplit == 1 && attn_prefill_applies(a)) {      // (dense arrays: its tile loads count on rows 256 bytes apart)
         pipelined = p.allow_fast_path == 3 || (p.allow_fast_path == 1 && (p.Sk % 64 == 0 || p.Sk >= 2048));
     }
     if (pipelined) err = launch_attn_prefill(kind, p.out16, a, stream);

@@ -27,7 +27,7 @@ struct AttnArgs {
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
     int nvb;       // pipelined prefill kernel: virtual blocks (the grid's workgroups take them in turn)
-    FastDiv dH, dgroup, dunits, dqtiles;      // pipelined prefill kernel: H, H / Hkv, qtiles / 2, qtiles as divisors
+    FastDiv dgroup, dunits, dqtiles;      // pipelined prefill kernel: H / Hkv, qtiles / 2, qtiles as divisors
     int hgroup;    // general kernel, causal: > 0 heads per group of the workgroup order of a large grid; < 0 the placement of a small one
     // fast kernel, grouped decode: the workgroup's key range is split `split` of nsplit (chunk keys each) and, when part is not
     // null, it stores its unnormalised partial (m, l, O[128]) at part + ((b H_q + head) nsplit + split) * 130 for the merge pass
@@ -133,6 +133,7 @@ template <> __device__ __forceinline__ uint32_t pack2_p<bf16_t>(float a, float b
 
 
 // 16-bit, head dimension 128, plain / causal attention in the software-pipelined form (attention_prefill.hip); kind: 1 fp16, 2 bf16
+bool attn_prefill_applies(const AttnArgs& a);
 hipError_t launch_attn_prefill(int kind, int out16, AttnArgs a, hipStream_t stream);
 
 }  // namespace aidn

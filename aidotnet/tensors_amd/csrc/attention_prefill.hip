@@ -82,15 +82,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
     const float sl2 = a.scale * LOG2E;
     const int Sk = a.Sk;
-    const long long qoff = a.qoff;
+    const int qoff = a.qoff;                    // (the launcher keeps |qoff|, Sq and Sk below 2^30: row and key sums stay 32-bit)
 
     // Direct-to-LDS loads.  This wave's share of a tile: K wave-loads 4 w .. 4 w + 3 and the same of V, each 4 keys x 256 B; lane ->
     // (key = 4 * load + lane / 16, chunk position lane % 16).  LDS layout [key][256 B]: 16-byte chunk c of key k sits at position
     // c ^ (k & 15) in a K tile (b128 fragment reads) and at c ^ ((k & 3) << 2) in a V tile (transposing reads).
     const int ld_key = lane >> 4, ld_pos = lane & 15;
-    const long long k_row_bytes = a.ks[2] * 2, v_row_bytes = a.vs[2] * 2;
-    // (wave-load i of K differs from load 0 by the swizzle bits 4 i of the chunk position: an XOR with i << 6 when the row pitch
-    // is a multiple of 256 bytes, which the launcher checks)
+    // Q, K, V and O are dense [batch, head, row, 128] arrays (the launcher checks): row r of (batch, head) pair j is row
+    // j * rows + r of the array, 256 bytes a row in the 16-bit types.
+    constexpr int k_row_bytes = 256, v_row_bytes = 256;
+    // (wave-load i of K differs from load 0 by the swizzle bits 4 i of the chunk position: an XOR with i << 6)
     const uint32_t k_lane_off = (uint32_t)(ld_key * k_row_bytes) + ((ld_pos ^ ld_key) << 4);
     const uint32_t v_lane_off = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (ld_key << 2)) << 4);
 
@@ -98,9 +99,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     auto tiles_of = [&](int q0) -> int {
         int nt = (Sk + BC - 1) / BC;
         if (a.causal) {
-            long long lastkey = (long long)q0 + BR - 1 + qoff;
+            const int lastkey = q0 + BR - 1 + qoff;
             if (lastkey < 0) nt = 0;
-            else { long long c = lastkey / BC + 1; if (c < nt) nt = (int)c; }
+            else { const int c = lastkey / BC + 1; if (c < nt) nt = c; }
         }
         return nt;
     };
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             for (int i = 0; i < 4; i++) {
                 const int key = 4 * (wave_s * 4 + i) + (ln >> 4);       // key inside the tile
                 const int gkey = min(tile * BC + key, Sk - 1);          // rows past the end are clamped loads, masked later
-                attn_dma16(K + (long long)gkey * a.ks[2] + ((ln & 15) ^ (key & 15)) * 8, dst + i * 1024);
+                attn_dma16(K + (long long)gkey * 128 + ((ln & 15) ^ (key & 15)) * 8, dst + i * 1024);
             }
         }
     };
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             for (int i = 0; i < 4; i++) {
                 const int key = 4 * (wave_s * 4 + i) + (ln >> 4);
                 const int gkey = min(tile * BC + key, Sk - 1);
-                attn_dma16(V + (long long)gkey * a.vs[2] + ((ln & 15) ^ ((key & 3) << 2)) * 8, dst + i * 1024);
+                attn_dma16(V + (long long)gkey * 128 + ((ln & 15) ^ ((key & 3) << 2)) * 8, dst + i * 1024);
             }
         }
     };
@@ -151,18 +152,17 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     auto open_pass = [&](int bh, int qt) {
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        const int b = (int)fastdiv((uint32_t)bh, a.dH), hd = bh - b * a.H;
-        const int kvh = (int)fastdiv((uint32_t)hd, a.dgroup);
-        const int qrow = qt * BR + wave_s * 32 + (ln & 31);
-        const uint16_t* Q = (const uint16_t*)a.q + b * a.qs[0] + hd * a.qs[1] + (long long)qrow * a.qs[2] + (ln >> 5) * 8;
+        // (a lane whose row lies past the end of the sequence takes the last row: what it computes is never stored)
+        const int qrow = min(qt * BR + wave_s * 32 + (ln & 31), a.Sq - 1);
+        const uint16_t* Q = (const uint16_t*)a.q + ((long long)(bh * a.Sq) << 7) + qrow * 128 + (ln >> 5) * 8;
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            u32x4 z = {0u, 0u, 0u, 0u};
-            const u32x4 x = (qrow < a.Sq) ? *(const u32x4*)(Q + 16 * s) : z;
+            const u32x4 x = *(const u32x4*)(Q + 16 * s);
 #pragma unroll
             for (int e = 0; e < 4; e++) { if (s < 4) qlo[4 * s + e] = x[e]; else qhi[4 * s - 16 + e] = x[e]; }
         }
-        const uint16_t* K = (const uint16_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
+        // (H = Hkv * group: K/V head b Hkv + head / group is (b H + head) / group)
+        const uint16_t* K = (const uint16_t*)a.k + ((long long)((int)fastdiv((uint32_t)bh, a.dgroup) * Sk) << 7);
         const int nt = tiles_of(qt * BR);
         if (nt > 0) issue_k(K, 0);
         if (nt > 1) issue_k(K, 1);
@@ -179,21 +179,19 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #else
 #define STAMP(i)
 #endif
-    const int b = (int)fastdiv((uint32_t)bh, a.dH), hd = bh - b * a.H;
-    const int kvh = (int)fastdiv((uint32_t)hd, a.dgroup);
     const int q0 = qt * BR;
     const int qi = q0 + wave * 32 + l32;
-    const raw_t* __restrict__ Q = (const raw_t*)a.q + b * a.qs[0] + hd * a.qs[1];
-    const raw_t* __restrict__ K = (const raw_t*)a.k + b * a.ks[0] + kvh * a.ks[1];
-    const raw_t* __restrict__ V = (const raw_t*)a.v + b * a.vs[0] + kvh * a.vs[1];
+    const long long kv_first = (long long)((int)fastdiv((uint32_t)bh, a.dgroup) * Sk) << 7;      // first element of the head's K and V
+    const raw_t* __restrict__ K = (const raw_t*)a.k + kv_first;
+    const raw_t* __restrict__ V = (const raw_t*)a.v + kv_first;
 
     // tiles of the workgroup, units (32 keys) of this wave
     const int ntiles = tiles_of(q0);
     const int wq_min = q0 + wave_s * 32, wq_max = wq_min + 31;
     auto key_limit = [&](int q) -> int {        // last key query q may see (sequence end and causal diagonal in one bound)
-        long long lim = Sk - 1;
-        if (a.causal) { long long c = (long long)q + qoff; if (c < lim) lim = c; }
-        return (int)(lim < -1 ? -1 : lim);
+        int lim = Sk - 1;
+        if (a.causal) { const int c = q + qoff; if (c < lim) lim = c; }
+        return lim < -1 ? -1 : lim;
     };
     int nu = 0;
     if (wq_min < a.Sq) nu = (key_limit(wq_max) + 1 + 31) / 32;
@@ -201,7 +199,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     nu = __builtin_amdgcn_readfirstlane(nu);
     // a unit all of whose keys every row of the wave sees needs no mask: units 0 .. ufull
     const int ufull = __builtin_amdgcn_readfirstlane((key_limit(wq_min) + 1) / 32 - 1);
-    const int usteady = min(nu - 2, ufull);          // units 1 .. usteady take the interleaved block
     const int klim = key_limit(qi) - 4 * h;          // element r of unit u is masked when 32 u + 8 (r / 4) + r % 4 > klim
 
     // LDS read addresses (per lane).  The two stages of the K tiles are 32 KB of four 32-key units, unit index j at offset
@@ -277,7 +274,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     };
     // Probabilities of unit u with the row maxima formed first (the safe form, also the wave's first unit in the fast form): the
     // reference of a row is raised when the row's maximum lies more than 8 above it (always on first use).  Adds the row sums to l.
-    auto softmax_exact = [&](int u, bool apply_mask, bool first) {
+    auto softmax_exact = [&](int u, bool apply_mask, const bool first) {
         if (apply_mask) mask_unit(u);
         float m = -INFINITY;
 #pragma unroll
@@ -285,7 +282,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         const float mloc = max_with_partner32(m) * sl2;            // scale > 0: max commutes with the scaling
         if (first) {
             m_ref = mloc < INFINITY ? mloc : -INFINITY;            // nothing accumulated yet: no O or l to move
-        } else if (__builtin_amdgcn_ballot_w64(mloc > m_ref + 8.0f) != 0ull) {
+        } else {
+            // (the accumulators are scaled whether a reference moves or not, by 1 if not: a branch around the scaling costs more,
+            // in copies of all 64 of them, than the scaling)
             const float m_new = (mloc > m_ref + 8.0f && mloc < INFINITY) ? mloc : m_ref;
             const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
             m_ref = m_new;
@@ -401,7 +400,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     STAMP(1);
     if (nu > 0) qk_plain();                     // S(0)
     next_k_unit();                              // K addresses at unit 1, V addresses at unit 0
-    int u = 0;
+    // unit 0 (nothing accumulated yet): P(0), S(1), the tile barrier of an even unit
+    if (nu > 0) softmax_exact(0, 0 > ufull, true);
+    if (nu > 1) qk_plain();
+    next_k_unit();
+    tile_barrier();
+    int u = 1;
     while (u < nunits) {
         if (!safe && u == 1) {
             // one run of the assembly loop: units 1 .. u_last, whole, unmasked, with a successor; it ends ahead of the odd unit
@@ -422,17 +426,15 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         }
         // the steps of unit u one after the other, row maxima formed first: P(u-1) V, P(u), S(u+1)
         if (u & 1) unit_loads(u);
-        if (u >= 1) {
-            if (u - 1 < nu) pv_plain();
-            next_v_unit();
-        }
-        if (u < nu) softmax_exact(u, u > ufull, u == 0);
+        if (u - 1 < nu) pv_plain();
+        next_v_unit();
+        if (u < nu) softmax_exact(u, u > ufull, false);
         if (u + 1 < nu) qk_plain();
         next_k_unit();
         if (!(u & 1)) tile_barrier();
         u++;
     }
-    if (nunits - 1 < nu && nunits > 0) pv_plain();              // P V of the workgroup's last unit
+    if (nunits - 1 < nu && nunits > 0) pv_plain();       // P V of the workgroup's last unit
     STAMP(4);
     if (!safe) {
         const bool left_range = __builtin_amdgcn_ballot_w64(!(l_run < 1.2676506e30f)) != 0ull;
@@ -473,8 +475,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         unsigned char* wr = stg + (lnw & 31) * SROW + (lnw >> 5) * 16;                  // chunk 8 (i % 2) + 2 g + h of row l32
         const unsigned char* rd = stg + (lnw >> 4) * SROW + (lnw & 15) * 16;           // chunk lane % 16 of row 4 q + lane / 16
         // the wave's 32 output rows: a uniform base, a 32-bit lane offset (the launcher checks that 32 rows span less than 4 GB)
-        unsigned char* obase = (unsigned char*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)(q0 + wave_s * 32) * a.os[2]);
-        const uint32_t row_bytes = (uint32_t)a.os[2] * 4u;
+        unsigned char* obase = (unsigned char*)((float*)a.o + ((long long)(bh * a.Sq + q0 + wave_s * 32) << 7));
+        constexpr uint32_t row_bytes = 512u;
         const uint32_t lane_off = (uint32_t)(lnw >> 4) * row_bytes + (uint32_t)(lnw & 15) * 16u;
         const int rows_left = a.Sq - (q0 + wave_s * 32);                                // rows of the wave inside the sequence
 #pragma unroll
@@ -504,7 +506,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         }
     } else if (qi < a.Sq) {
         typedef typename Raw2<OutT>::type out_t;
-        out_t* __restrict__ O = (out_t*)a.o + b * a.os[0] + hd * a.os[1] + (long long)qi * a.os[2];
+        out_t* __restrict__ O = (out_t*)a.o + ((long long)(bh * a.Sq + qi) << 7);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
 #pragma unroll
@@ -554,7 +556,6 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
-    if (a.os[2] * 4 * 32 >= 0xFFFFFFFFLL || a.os[2] < 0) return hipErrorInvalidValue;     // the lane offsets of the O stores are 32 bits
     // causal self-attention with an even number of query tiles: tile i and tile qtiles-1-i in one workgroup (equal work everywhere)
     a.paired = (a.causal && a.qoff == 0 && a.Sq == a.Sk && a.qtiles >= 2 && a.qtiles % 2 == 0) ? 1 : 0;
     const long long nblk = (long long)(a.paired ? a.qtiles / 2 : a.qtiles) * a.B * a.H;
@@ -566,17 +567,31 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
     if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
     const long long resident = (long long)(2 * cus) / 8 * 8;
     a.nvb = (int)nblk;
-    a.dH = make_fastdiv((uint32_t)a.H); a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));
+    a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));
     a.dunits = make_fastdiv((uint32_t)(a.qtiles / 2 > 0 ? a.qtiles / 2 : 1)); a.dqtiles = make_fastdiv((uint32_t)a.qtiles);
     const unsigned grid = (unsigned)((resident >= 8 && nblk > resident) ? resident : nblk);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, a);
     return hipGetLastError();
 }
 
+// The kernel takes dense [batch, head, row, 128] arrays (rows 256 bytes apart: its tile loads and its addresses count on that) whose
+// row and key counts leave 32-bit index arithmetic room.
+bool attn_prefill_applies(const AttnArgs& a)
+{
+    auto dense = [&](const long long* st, long long heads, long long rows) {
+        return st[2] == 128 && (heads == 1 || st[1] == rows * 128) && (a.B == 1 || st[0] == heads * rows * 128);
+    };
+    if (a.D != 128 || a.nsplit > 1 || a.part || a.stream || a.bt || !(a.scale > 0.0f)) return false;
+    if (a.Hkv <= 0 || a.H % a.Hkv != 0) return false;
+    if (!dense(a.qs, a.H, a.Sq) || !dense(a.os, a.H, a.Sq) || !dense(a.ks, a.Hkv, a.Sk) || !dense(a.vs, a.Hkv, a.Sk)) return false;
+    const long long lim = 1LL << 30;
+    if (a.Sq >= lim || a.Sk >= lim || a.qoff >= lim || a.qoff <= -lim) return false;
+    return (long long)a.B * a.H * a.Sq < (1LL << 31) - 256 && (long long)a.B * a.Hkv * a.Sk < (1LL << 31) - 256;
+}
+
 hipError_t launch_attn_prefill(int kind, int out16, AttnArgs a, hipStream_t stream)
 {
-    if (a.D != 128 || a.nsplit > 1 || a.part || a.stream || a.bt || !(a.scale > 0.0f)) return hipErrorInvalidValue;
-    if (a.ks[2] != 128 || a.vs[2] != 128) return hipErrorInvalidValue;     // the tile loads count on K and V rows 256 bytes apart
+    if (!attn_prefill_applies(a)) return hipErrorInvalidValue;
     if (kind == 1) return out16 ? launch_prefill<f16_t, f16_t>(a, stream) : launch_prefill<f16_t, float>(a, stream);
     if (kind == 2) return out16 ? launch_prefill<bf16_t, bf16_t>(a, stream) : launch_prefill<bf16_t, float>(a, stream);
     return hipErrorInvalidValue;
