@@ -67,6 +67,69 @@ def _sclk_mhz():
     return None
 
 
+def _power_uw():
+    """Board power the driver reports right now (microwatts), and the cap, or (None, None): hwmon power1_average where the driver has
+    it, else power1_input."""
+    import glob
+    for d in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+        for name in ("power1_average", "power1_input"):
+            try:
+                val = int(open(os.path.join(d, name)).read())
+            except (OSError, ValueError):
+                continue
+            try:
+                cap = int(open(os.path.join(d, "power1_cap")).read())
+            except (OSError, ValueError):
+                cap = None
+            return val, cap
+    return None, None
+
+
+def _load_trace(torch, fn, steps, min_ms=80.0):
+    """Board power and engine clock sampled WHILE the workload runs: a third pass (it never touches the timed figures) that keeps
+    `steps`-long batches of the step queued for at least `min_ms` while a thread reads the driver's files every millisecond or so.
+    Returns {"power_w": {...}, "sclk_mhz": {...}} or None where the driver offers neither file."""
+    import threading
+    if _power_uw()[0] is None and _sclk_mhz() is None:
+        return None
+    stop = threading.Event()
+    pw, ck = [], []
+
+    def sample():
+        while not stop.is_set():
+            p, _ = _power_uw()
+            c = _sclk_mhz()
+            if p is not None:
+                pw.append(p / 1e6)
+            if c is not None:
+                ck.append(c)
+            time.sleep(0.001)
+
+    th = threading.Thread(target=sample, daemon=True)
+    t0 = time.perf_counter()
+    n = 0
+    for _ in range(steps):          # the queue is filled before the first sample is taken
+        fn()
+    th.start()
+    while (time.perf_counter() - t0) * 1e3 < min_ms:
+        for _ in range(steps):
+            fn()
+        n += steps
+        # (no synchronisation between the batches beyond what keeps the queue bounded: the device stays busy throughout)
+        if n % (8 * steps) == 0:
+            torch.cuda.synchronize()
+    stop.set()
+    th.join()
+    torch.cuda.synchronize()
+    out = {}
+    if pw:
+        out["power_w"] = {"mean": round(sum(pw) / len(pw), 1), "max": round(max(pw), 1), "samples": len(pw),
+                          "cap": None if _power_uw()[1] is None else round(_power_uw()[1] / 1e6, 1)}
+    if ck:
+        out["sclk_mhz"] = {"mean": round(sum(ck) / len(ck), 1), "min": min(ck), "max": max(ck), "samples": len(ck)}
+    return out or None
+
+
 def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
     """`warmup` untimed steps, continued until `min_warm_ms` of wall time has passed (a launch sequence needs some tens of
     milliseconds of its own load before the clock management of the device settles), then exactly `steps` timed steps.
@@ -106,6 +169,9 @@ def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
     stats = {"median_ms": round(per[len(per) // 2], 5), "p95_ms": round(per[min(len(per) - 1, int(math.ceil(0.95 * len(per))) - 1)], 5),
              "min_ms": round(per[0], 5), "max_ms": round(per[-1], 5), "sclk_mhz_before_after": [clk0, clk1], "sclk_mhz_while_queued": clk_load,
              "note": "single steps timed in a second pass with one event pair each (includes the events' own cost)"}
+    trace = _load_trace(torch, fn, steps)
+    if trace:
+        stats["under_load"] = trace        # board power (W) and engine clock (MHz) sampled in a third pass with the step kept queued
     return ms, wall_ms, stats
 
 
