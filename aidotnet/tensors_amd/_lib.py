@@ -76,6 +76,8 @@ SIGNATURES = {
     "aidn_mi355_hgemm_f16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_f32out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "aidn_mi355_bf16gemm_bf16out": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    "aidn_mi355_hgemm_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i, _i]),
+    "aidn_mi355_bf16gemm_rope": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp, _vp, _i, _i, _i, _i]),
     "aidn_mi355_convert_f32_to_f16": (_i, [_vp, _vp, _vp, _vp, _i64]),
     "aidn_mi355_convert_f16_to_f32": (_i, [_vp, _vp, _vp, _vp, _i64]),
     "aidn_mi355_convert_f32_to_bf16": (_i, [_vp, _vp, _vp, _vp, _i64]),

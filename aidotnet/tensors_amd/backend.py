@@ -607,6 +607,35 @@ class Mi355Backend:
     def GemmBf16In32fOut(self, aBf16: GpuBuffer, bBf16: GpuBuffer, cFp32: GpuBuffer, m: int, n: int, k: int) -> None:
         self._gemm16(self._lib.aidn_mi355_bf16gemm_f32out, aBf16, bBf16, cFp32, m, n, k, 4, "GemmBf16In32fOut")
 
+    def GemmRope(self, kind: str, a: GpuBuffer, b: GpuBuffer, c: GpuBuffer, m: int, n: int, k: int, cos: GpuBuffer, sin: GpuBuffer,
+                 headDim: int, ropeCols: int, seqLen: int, startPosition: int) -> None:
+        """C[m,n] = A * B in fp16 / bf16 (fp32 accumulation), then RopeInterleaved over the first ropeCols columns of C (heads of
+        headDim side by side; row r at position startPosition + r % seqLen) in the same call: a projection of a decode step
+        (SimdGemm.NParallelSmallM.cs:95-109) and its rotation (IDirectGpuBackend.cs:1427-1446) with one launch fewer.  Same values
+        as Hgemm / Bf16Gemm followed by RopeInterleaved.  No single member of the reference does both."""
+        fn = {"f16": self._lib.aidn_mi355_hgemm_rope, "bf16": self._lib.aidn_mi355_bf16gemm_rope}.get(kind)
+        if fn is None:
+            raise NotSupportedException("GemmRope: kind must be 'f16' or 'bf16'")
+        if m <= 0 or n <= 0 or k <= 0:
+            raise ArgumentOutOfRangeException("GemmRope: M, N, K must all be > 0 (got M=%d, N=%d, K=%d)." % (m, n, k))
+        if headDim <= 0 or seqLen <= 0:
+            raise ArgumentOutOfRangeException("RoPE dimensions must be positive.")
+        if headDim & 1:
+            raise ArgumentException("RoPE requires an even head dimension.")
+        if startPosition < 0:
+            raise ArgumentOutOfRangeException("startPosition")
+        if ropeCols < 0 or ropeCols > n or ropeCols % headDim != 0 or n & 1:
+            raise ArgumentException("GemmRope: ropeCols must be a multiple of headDim within n, and n even.")
+        for buf, nm in ((a, "a"), (b, "b"), (c, "c"), (cos, "cos"), (sin, "sin")):
+            self._need(buf, nm)
+        self._capacity(a, m * k * 2, "a", "GemmRope"); self._capacity(b, k * n * 2, "b", "GemmRope"); self._capacity(c, m * n * 2, "c", "GemmRope")
+        need = (startPosition + min(seqLen, m)) * (headDim // 2) * 4
+        if cos.SizeInBytes < need or sin.SizeInBytes < need:
+            raise ArgumentException("RoPE cos/sin caches are shorter than startPosition + seqLen positions.")
+        self._check(fn(self._ctx, self._stream(), a.Handle, b.Handle, c.Handle, m, n, k, cos.Handle, sin.Handle, headDim, ropeCols, seqLen,
+                       startPosition))
+        self._done()
+
     # ------------------------------------------------------------------ conversions
     def _convert(self, fn, inp, out, size, in_bytes, out_bytes, op):
         self._need(inp, "input"); self._need(out, "output")

@@ -209,6 +209,28 @@ int gemm16_common(void* ctx, void* stream, int kind, const uint16_t* A, const ui
                       "gemm_16");
 }
 
+int gemm16_rope_common(void* ctx, void* stream, int kind, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                       const float* cosc, const float* sinc, int head_dim, int rope_cols, int seq_len, int start_position)
+{
+    Ctx* c = (Ctx*)ctx;
+    if (!c) return AIDN_ERR_INVALID_ARGUMENT;
+    if (!A || !B || !C || !cosc || !sinc) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_rope: buffers must not be null");
+    if (M <= 0 || N <= 0 || K <= 0 || head_dim <= 0 || seq_len <= 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_rope: dimensions must be positive");
+    if (head_dim & 1) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_rope: head dimension must be even");
+    if (rope_cols < 0 || rope_cols > N || rope_cols % head_dim != 0 || (N & 1))
+        return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_rope: rope_cols must be a multiple of head_dim within N, and N even");
+    if (start_position < 0) return fail(c, AIDN_ERR_INVALID_ARGUMENT, "gemm_rope: start position must not be negative");
+    void* ws = nullptr;
+    size_t need = c->force_tile == 0 ? aidn::gemm_16_workspace_bytes(M, N, K) : 0;
+    if (need) {
+        int st = acquire_ws(c, stream, need, &ws);
+        if (st == AIDN_ERR_WORKSPACE) ws = nullptr;      // under capture and not reserved: the tiled kernel and a second launch for the rotation
+        else if (st) return st;
+    }
+    const aidn::RopeEpilogue rope{cosc, sinc, head_dim, rope_cols, seq_len, start_position};
+    return hip_status(c, aidn::gemm_16_rope((hipStream_t)stream, kind, A, B, C, M, N, K, c->force_tile, ws, ws ? need : 0, rope), "gemm_16_rope");
+}
+
 // [Wq|Wk|Wv] side by side in one [dModel, 3 dModel] matrix (three strided device copies), the weight operand of the fused
 // QKV projection.
 hipError_t gather_qkv(hipStream_t sm, const void* wq, const void* wk, const void* wv, void* packed, int dModel, size_t es)
@@ -557,6 +579,13 @@ AIDN_API int aidn_mi355_bf16gemm_f32out(void* ctx, void* stream, const uint16_t*
 { return gemm16_common(ctx, stream, 1, A, B, C, 1, M, N, K); }
 AIDN_API int aidn_mi355_bf16gemm_bf16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K)
 { return gemm16_common(ctx, stream, 1, A, B, C, 0, M, N, K); }
+
+AIDN_API int aidn_mi355_hgemm_rope(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                                   const float* cos_cache, const float* sin_cache, int head_dim, int rope_cols, int seq_len, int start_position)
+{ return gemm16_rope_common(ctx, stream, 0, A, B, C, M, N, K, cos_cache, sin_cache, head_dim, rope_cols, seq_len, start_position); }
+AIDN_API int aidn_mi355_bf16gemm_rope(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                                      const float* cos_cache, const float* sin_cache, int head_dim, int rope_cols, int seq_len, int start_position)
+{ return gemm16_rope_common(ctx, stream, 1, A, B, C, M, N, K, cos_cache, sin_cache, head_dim, rope_cols, seq_len, start_position); }
 
 AIDN_API int aidn_mi355_convert_f32_to_f16(void* ctx, void* stream, const float* in, uint16_t* out, int64_t n)
 { return convert_common(ctx, stream, 0, in, out, n); }

@@ -157,4 +157,17 @@ __device__ __forceinline__ void half_swap(float v, float& lo_half, float& hi_hal
 __device__ __forceinline__ float max_with_partner32(float v) { float a, b; half_swap(v, a, b); return fmaxf(a, b); }
 __device__ __forceinline__ float sum_with_partner32(float v) { float a, b; half_swap(v, a, b); return a + b; }
 
+// One interleaved rotary pair: (xe, xo) -> (xe c - xo s, xe s + xo c).  One definition for the stand-alone kernels and for the
+// GEMM pass that rotates while it sums, so that both round alike (HipAttentionKernels.cs:958-989 is the reference form).
+__device__ __forceinline__ void rope_rotate(float xe, float xo, float c, float s, float& re, float& ro)
+{
+    // (spelled out as one product and one fused multiply-add each, so that every kernel that calls this rounds the same way
+    // whatever the compiler would contract around it)
+    re = __builtin_fmaf(xe, c, -(xo * s));
+    ro = __builtin_fmaf(xe, s, xo * c);
+    // (the fp32 results are made opaque: a caller that narrows them to fp16 would otherwise be compiled to the mixed-precision
+    // multiply-add that rounds the exact sum to fp16 once, one caller and not the other, and the two would differ at near-ties)
+    asm("" : "+v"(re), "+v"(ro));
+}
+
 }  // namespace aidn

@@ -93,7 +93,8 @@ __global__ __launch_bounds__(256) void rope_interleaved_kernel(const void* __res
             uint32_t v = ((const uint32_t*)in)[g];
             xe = Elem<T>::widen(v & 0xFFFFu); xo = Elem<T>::widen(v >> 16);
         }
-        const float re = xe * c - xo * sn, ro = xe * sn + xo * c;
+        float re, ro;
+        rope_rotate(xe, xo, c, sn, re, ro);
         if constexpr (Elem<T>::BYTES == 4) ((u32x2*)out)[g] = u32x2{as_u32(re), as_u32(ro)};
         else ((uint32_t*)out)[g] = Elem<T>::narrow(re) | (Elem<T>::narrow(ro) << 16);
     }
@@ -123,19 +124,55 @@ __global__ __launch_bounds__(256) void rope_interleaved_vec_kernel(const void* i
 #pragma unroll
             for (int p = 0; p < 2; p++) {
                 const float xe = as_f32(v[2 * p]), xo = as_f32(v[2 * p + 1]), cc = as_f32(c[p]), ss = as_f32(sn[p]);
-                o[2 * p] = as_u32(xe * cc - xo * ss);
-                o[2 * p + 1] = as_u32(xe * ss + xo * cc);
+                float re, ro;
+                rope_rotate(xe, xo, cc, ss, re, ro);
+                o[2 * p] = as_u32(re);
+                o[2 * p + 1] = as_u32(ro);
             }
         } else {
             const u32x4 c = *(const u32x4*)(cosc + pos * half + i), sn = *(const u32x4*)(sinc + pos * half + i);
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 const float xe = Elem<T>::widen(v[p] & 0xFFFFu), xo = Elem<T>::widen(v[p] >> 16), cc = as_f32(c[p]), ss = as_f32(sn[p]);
-                o[p] = Elem<T>::narrow(xe * cc - xo * ss) | (Elem<T>::narrow(xe * ss + xo * cc) << 16);
+                float re, ro;
+                rope_rotate(xe, xo, cc, ss, re, ro);
+                o[p] = Elem<T>::narrow(re) | (Elem<T>::narrow(ro) << 16);
             }
         }
         ((u32x4*)out)[g] = o;
     }
+}
+
+// The same rotation over the first `cols` columns of every row of a dense 16-bit [M, N] matrix, in place (the columns are heads of
+// headDim elements side by side: what a projection GEMM writes); row m takes the angle of position startPosition + m % seqLen.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_cols_kernel(uint16_t* __restrict__ C, const float* __restrict__ cosc, const float* __restrict__ sinc,
+                                                        int M, int N, int cols, int headDim, int seqLen, int startPosition)
+{
+    const int half = headDim >> 1, pairs = cols >> 1;
+    const long long total = (long long)M * pairs;
+    for (long long g = (long long)blockIdx.x * blockDim.x + threadIdx.x; g < total; g += (long long)gridDim.x * blockDim.x) {
+        const int m = (int)(g / pairs), col = 2 * (int)(g - (long long)m * pairs);
+        const int i = (col % headDim) >> 1;
+        const long long pos = startPosition + m % seqLen;
+        uint32_t* p = (uint32_t*)(C + (long long)m * N + col);
+        const uint32_t v = *p;
+        float re, ro;
+        rope_rotate(Elem<T>::widen(v & 0xFFFFu), Elem<T>::widen(v >> 16), cosc[pos * half + i], sinc[pos * half + i], re, ro);
+        *p = Elem<T>::narrow(re) | (Elem<T>::narrow(ro) << 16);
+    }
+}
+
+hipError_t rope_cols16(hipStream_t stream, int kind, uint16_t* C, const float* cosc, const float* sinc, int M, int N, int cols, int headDim,
+                       int seqLen, int startPosition)
+{
+    const long long total = (long long)M * (cols / 2);
+    if (total <= 0) return hipSuccess;
+    const unsigned grid = (unsigned)((total + 255) / 256 > 256 * 32 ? 256 * 32 : (total + 255) / 256);
+    if (kind == 1) hipLaunchKernelGGL(rope_cols_kernel<f16_t>, dim3(grid), dim3(256), 0, stream, C, cosc, sinc, M, N, cols, headDim, seqLen, startPosition);
+    else if (kind == 2) hipLaunchKernelGGL(rope_cols_kernel<bf16_t>, dim3(grid), dim3(256), 0, stream, C, cosc, sinc, M, N, cols, headDim, seqLen, startPosition);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 // kind: 0 fp32, 1 fp16, 2 bf16

@@ -1377,6 +1377,33 @@ __global__ __launch_bounds__(256) void skinny_reduce_kernel(const float* __restr
     }
 }
 
+// The summing pass with the rotary embedding on top: one thread per column pair (2 j, 2 j + 1) of a row sums both columns in split
+// order, rotates the pair when it lies in the first rope.cols columns, and stores both with one rounding.
+template <typename OutT>
+__global__ __launch_bounds__(256) void skinny_reduce_rope_kernel(const float* __restrict__ ws, uint16_t* __restrict__ C, int M, int N, int ksplit,
+                                                                  const RopeEpilogue rope)
+{
+    typedef float f32x2a __attribute__((ext_vector_type(2)));
+    const long long total = (long long)M * N, pairs = total >> 1;
+    const int half = rope.head_dim >> 1, row_pairs = N >> 1;
+    for (long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += (long long)gridDim.x * blockDim.x) {
+        float s0 = 0.0f, s1 = 0.0f;
+        for (int k = 0; k < ksplit; k++) {
+            const f32x2a t = *(const f32x2a*)(ws + (long long)k * total + 2 * p);
+            s0 += t[0]; s1 += t[1];
+        }
+        const int m = (int)(p / row_pairs), col = 2 * (int)(p - (long long)m * row_pairs);
+        if (col < rope.cols) {
+            const int i = (col % rope.head_dim) >> 1;
+            const long long pos = rope.start_position + m % rope.seq_len;
+            // (the pair is rounded to the output type before it is rotated: what a product followed by the rotation kernel computes)
+            const float xe = Elem<OutT>::widen(Elem<OutT>::narrow(s0)), xo = Elem<OutT>::widen(Elem<OutT>::narrow(s1));
+            rope_rotate(xe, xo, rope.cosc[pos * half + i], rope.sinc[pos * half + i], s0, s1);
+        }
+        ((uint32_t*)C)[p] = Elem<OutT>::narrow(s0) | (Elem<OutT>::narrow(s1) << 16);
+    }
+}
+
 static bool skinny_applies(int M, int N, int K) { return M <= 32 && N % 128 == 0 && K % 64 == 0 && N >= 128; }
 
 // How evenly `tiles` workgroups load the 256 CUs: a CU works through its tiles at about the same rate whether it holds one or
@@ -1715,7 +1742,7 @@ size_t gemm_16_packed_workspace_bytes(int M, int N, int K)
 #endif
 
 template <typename T, typename OutT>
-static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws)
+static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws, const RopeEpilogue* rope = nullptr)
 {
     int ks;
     // more than 64 column slabs over a K of at most 4096 (16 x 28672 x 8192 went 77 -> 88 us): the three-stage form, two workgroups per CU (a workgroup's first memory round trip and its last
@@ -1738,6 +1765,13 @@ static hipError_t launch_skinny(const GemmArgs& g, hipStream_t stream, float* ws
     if (e != hipSuccess) return e;
     long long total = (long long)g.M * g.N;
     unsigned grid = (unsigned)((total + 255) / 256);
+    if constexpr (!std::is_same<OutT, float>::value) {
+        if (rope) {
+            grid = (unsigned)((total / 2 + 255) / 256);
+            hipLaunchKernelGGL((skinny_reduce_rope_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, (uint16_t*)g.C, g.M, g.N, ks, *rope);
+            return hipGetLastError();
+        }
+    }
     hipLaunchKernelGGL((skinny_reduce_kernel<OutT>), dim3(grid), dim3(256), 0, stream, ws, g.C, g.M, g.N, ks, g.bias, g.act, g.act_param,
                        1.0f, 0.0f);
     return hipGetLastError();
@@ -2502,14 +2536,40 @@ hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B,
                        int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre);
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
                         int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre);
+hipError_t gemm_16_rope_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                            void* workspace, size_t workspace_bytes, const RopeEpilogue& rope);
+hipError_t gemm_16_rope_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                             void* workspace, size_t workspace_bytes, const RopeEpilogue& rope);
+// C = A B, then interleaved RoPE over the leading columns of C (launch.hpp)
+template <typename T>
+static hipError_t gemm_16_rope_typed(hipStream_t stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                                     void* workspace, size_t workspace_bytes, const RopeEpilogue& rope)
+{
+    if (!workspace) workspace_bytes = 0;
+    // the plan of gemm_16_typed that sums K ranges in a pass of its own takes the rotation into that pass
+    if (force_tile == 0 && workspace && skinny_applies(M, N, K) && aligned16(A) && aligned16(B) &&
+        (size_t)skinny_ksplit(N, K) * M * N * sizeof(float) <= workspace_bytes) {
+        GemmArgs g{A, B, C, M, N, K, K, N, N, 0, 0, 0, 1.0f, 0.0f, 0, 0, nullptr, 0, 0.0f};
+        return launch_skinny<T, T>(g, stream, (float*)workspace, &rope);
+    }
+    if (hipError_t e = gemm_16_typed<T>(stream, A, B, C, 0, M, N, K, force_tile, workspace, workspace_bytes, nullptr, 0, 0.0f)) return e;
+    return rope_cols16(stream, std::is_same<T, f16_t>::value ? 1 : 2, C, rope.cosc, rope.sinc, M, N, rope.cols, rope.head_dim, rope.seq_len, rope.start_position);
+}
+
 #if AIDN_GEMM_PART == 1
 hipError_t gemm_16_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
                        int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre)
 { return gemm_16_typed<f16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre); }
+hipError_t gemm_16_rope_f16(hipStream_t stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                            void* workspace, size_t workspace_bytes, const RopeEpilogue& rope)
+{ return gemm_16_rope_typed<f16_t>(stream, A, B, C, M, N, K, force_tile, workspace, workspace_bytes, rope); }
 #elif AIDN_GEMM_PART == 2
 hipError_t gemm_16_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, void* C, int out32,
                         int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias, int act, float act_param, const uint16_t* Bpre)
 { return gemm_16_typed<bf16_t>(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre); }
+hipError_t gemm_16_rope_bf16(hipStream_t stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                             void* workspace, size_t workspace_bytes, const RopeEpilogue& rope)
+{ return gemm_16_rope_typed<bf16_t>(stream, A, B, C, M, N, K, force_tile, workspace, workspace_bytes, rope); }
 #else
 // kind: 0 = fp16, 1 = bf16
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
@@ -2517,6 +2577,12 @@ hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16
 {
     if (kind == 0) return gemm_16_f16(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre);
     return gemm_16_bf16(stream, A, B, C, out32, M, N, K, force_tile, workspace, workspace_bytes, bias, act, act_param, Bpre);
+}
+hipError_t gemm_16_rope(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                        void* workspace, size_t workspace_bytes, const RopeEpilogue& rope)
+{
+    if (kind == 0) return gemm_16_rope_f16(stream, A, B, C, M, N, K, force_tile, workspace, workspace_bytes, rope);
+    return gemm_16_rope_bf16(stream, A, B, C, M, N, K, force_tile, workspace, workspace_bytes, rope);
 }
 #endif
 

@@ -32,6 +32,14 @@ size_t gemm_16_workspace_bytes(int M, int N, int K);
 hipError_t gemm_16(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, void* C, int out32,
                    int M, int N, int K, int force_tile, void* workspace, size_t workspace_bytes, const float* bias = nullptr, int act = 0,
                    float act_param = 0.0f, const uint16_t* Bpre = nullptr);
+// C = A B followed by interleaved RoPE over the first rope.cols columns of C (heads of rope.head_dim elements side by side; row m at
+// position rope.start_position + m % rope.seq_len); C has the inputs' type.  Where the product has a summing pass of its own (few
+// rows: K ranges side by side) the rotation rides on that pass, otherwise it is a second launch over C.
+struct RopeEpilogue { const float* cosc; const float* sinc; int head_dim, cols, seq_len, start_position; };
+hipError_t gemm_16_rope(hipStream_t stream, int kind, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K, int force_tile,
+                        void* workspace, size_t workspace_bytes, const RopeEpilogue& rope);
+hipError_t rope_cols16(hipStream_t stream, int kind, uint16_t* C, const float* cosc, const float* sinc, int M, int N, int cols, int headDim,
+                       int seqLen, int startPosition);
 size_t gemm_16_packed_b_bytes(int N, int K);
 size_t gemm_16_packed_workspace_bytes(int M, int N, int K);
 hipError_t gemm_16_pack_b(hipStream_t stream, const uint16_t* B, int K, int N, void* packed);

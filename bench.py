@@ -298,7 +298,7 @@ def main() -> int:
             return randn(*shape, kind=kind)
         return (2.0 * torch.rand(*shape, device="cuda", generator=g) - 1.0).to(dts[kind])
 
-    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False, extra=False, packed=False):
+    def gemm_case(name, kind, M, N, K, out32=False, hbm=False, rotate=1, wstd=0.02, uniform_inputs=False, extra=False, packed=False, rope=None):
         if not want(name, extra):
             return
         # rotate > 1: cycle through that many distinct weight matrices so the timed loop reads HBM, not the
@@ -319,6 +319,13 @@ def main() -> int:
             fn1 = (lambda Bx: be.GemmFp16In32fOut(A_, Bx, C_, M, N, K)) if out32 else (lambda Bx: be.Hgemm(A_, Bx, C_, M, N, K))
         else:
             fn1 = (lambda Bx: be.GemmBf16In32fOut(A_, Bx, C_, M, N, K)) if out32 else (lambda Bx: be.Bf16Gemm(A_, Bx, C_, M, N, K))
+        if rope is not None:
+            # rope = (head_dim, rotated columns, position): the product with the interleaved rotary embedding in its summing pass
+            hd, rcols, pos = rope
+            half = hd // 2
+            ang = torch.arange(pos + 1, device="cuda", dtype=torch.float32)[:, None] * (10000.0 ** (-torch.arange(half, device="cuda") * 2.0 / hd))[None, :]
+            cs_, sn_ = W(torch.cos(ang).contiguous()), W(torch.sin(ang).contiguous())
+            fn1 = lambda Bx: be.GemmRope(kind, A_, Bx, C_, M, N, K, cs_, sn_, hd, rcols, 1, pos)
         it = [0]
 
         def fn():
@@ -333,7 +340,9 @@ def main() -> int:
             roof["note"] = "%d weight matrices rotated to defeat the last-level cache" % rotate
         else:
             roof = _roof_flops(kind, fl, ms_, TRAFFIC_BYTES.get(name))
-        add(name, kind, "GEMM M=%d N=%d K=%d%s%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else "", " (pre-packed B)" if packed else ""), ms_, roof, st_)
+        add(name, kind, "GEMM M=%d N=%d K=%d%s%s%s" % (M, N, K, " fp32 out" if out32 and kind != "f32" else "", " (pre-packed B)" if packed else "",
+                                                      " + interleaved RoPE over the first %d columns (head dim %d) in the same call" % (rope[1], rope[0]) if rope else ""),
+            ms_, roof, st_)
 
     def attn_case(name, kind, Bn, H, S, D, extra=False):
         if not want(name, extra):
@@ -382,6 +391,9 @@ def main() -> int:
     attn_case("attn_bf16_prefill", "bf16", 4, 32, 2048, 128)
     decode_case("decode_bf16", "bf16", 32, 32, 4096, 128)
     gemm_case("gemm_bf16_decode_proj", "bf16", 32, 4096, 4096, hbm=True, rotate=12)
+    # the decode step's concatenated [Wq|Wk|Wv] projection (SimdGemm.SgemmConcatenatedProjections), plain and with Q and K rotated in the same call
+    gemm_case("gemm_bf16_decode_qkv", "bf16", 32, 12288, 4096, hbm=True, rotate=4)
+    gemm_case("gemm_bf16_decode_qkv_rope", "bf16", 32, 12288, 4096, hbm=True, rotate=4, rope=(128, 8192, 4095))
     # shapes beside the listed configurations (run with --only NAME[,NAME...]): grouped-query decode, fp32 products with few rows,
     # a causal fp32 attention grid of several rounds
     decode_case("decode_bf16_gqa", "bf16", 32, 32, 4096, 128, Hkv=8, rotate=2, extra=True)

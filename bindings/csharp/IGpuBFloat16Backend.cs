@@ -19,6 +19,12 @@ namespace AiDotNet.Tensors.Engines.Gpu
         /// <summary>Mixed-precision product: A, B bf16, accumulator and C fp32 (the bf16 counterpart of GemmFp16In32fOut).</summary>
         void GemmBf16In32fOut(IGpuBuffer aBf16, IGpuBuffer bBf16, IGpuBuffer cFp32, int m, int n, int k);
 
+        /// <summary>C = A · B in fp16 or bf16 (fp32 accumulation, C in the inputs' type), then RopeInterleaved over the first
+        /// <paramref name="ropeCols"/> columns of C (heads of <paramref name="headDim"/> side by side; row r at position
+        /// startPosition + r % seqLen): a decode-step projection and its rotation in one call.</summary>
+        void GemmRopeReducedPrecision(GpuScalarType inputType, IGpuBuffer a, IGpuBuffer b, IGpuBuffer c, int m, int n, int k,
+            IGpuBuffer cos, IGpuBuffer sin, int headDim, int ropeCols, int seqLen, int startPosition);
+
         /// <summary>fp32 -> bf16 storage conversion, round-to-nearest-even, NaN keeps a quiet bit (BFloat16.FromFloat).</summary>
         void ConvertToBf16(IGpuBuffer inputFp32, IGpuBuffer outputBf16, int size);
 

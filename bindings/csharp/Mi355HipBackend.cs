@@ -159,6 +159,25 @@ namespace AiDotNet.Tensors.Engines.DirectGpu.HIP
             Sync(nameof(GemmBf16In32fOut));
         }
 
+        public void GemmRopeReducedPrecision(GpuScalarType inputType, IGpuBuffer a, IGpuBuffer b, IGpuBuffer c, int m, int n, int k,
+            IGpuBuffer cos, IGpuBuffer sin, int headDim, int ropeCols, int seqLen, int startPosition)
+        {
+            Positive(m, n, k, nameof(GemmRopeReducedPrecision));
+            if (headDim <= 0 || seqLen <= 0) throw new ArgumentOutOfRangeException(nameof(headDim), "RoPE dimensions must be positive.");
+            if ((headDim & 1) != 0) throw new ArgumentException("headDim must be even.", nameof(headDim));
+            if (startPosition < 0) throw new ArgumentOutOfRangeException(nameof(startPosition));
+            if (ropeCols < 0 || ropeCols > n || ropeCols % headDim != 0 || (n & 1) != 0)
+                throw new ArgumentException("ropeCols must be a multiple of headDim within n, and n even.", nameof(ropeCols));
+            int status = inputType switch
+            {
+                GpuScalarType.Float16 => Mi355Native.aidn_mi355_hgemm_rope(_ctx, _stream, a.Handle, b.Handle, c.Handle, m, n, k, cos.Handle, sin.Handle, headDim, ropeCols, seqLen, startPosition),
+                GpuScalarType.BFloat16 => Mi355Native.aidn_mi355_bf16gemm_rope(_ctx, _stream, a.Handle, b.Handle, c.Handle, m, n, k, cos.Handle, sin.Handle, headDim, ropeCols, seqLen, startPosition),
+                _ => throw new NotSupportedException($"{nameof(GemmRopeReducedPrecision)}: input type must be Float16 or BFloat16 (got {inputType})."),
+            };
+            Mi355Native.Check(_ctx, status, nameof(GemmRopeReducedPrecision));
+            Sync(nameof(GemmRopeReducedPrecision));
+        }
+
         public void ConvertToBf16(IGpuBuffer inputFp32, IGpuBuffer outputBf16, int size)
         {
             if (size <= 0) throw new ArgumentOutOfRangeException(nameof(size));

@@ -77,6 +77,12 @@ namespace AiDotNet.Tensors.Engines.DirectGpu.HIP
         [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_bf16gemm_f32out(IntPtr ctx, IntPtr stream, IntPtr a, IntPtr b, IntPtr c, int m, int n, int k);
         [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_bf16gemm_bf16out(IntPtr ctx, IntPtr stream, IntPtr a, IntPtr b, IntPtr c, int m, int n, int k);
 
+        // ---- projection + rotary embedding in one call
+        [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_hgemm_rope(IntPtr ctx, IntPtr stream, IntPtr a, IntPtr b, IntPtr c, int m, int n, int k,
+            IntPtr cosCache, IntPtr sinCache, int headDim, int ropeCols, int seqLen, int startPosition);
+        [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_bf16gemm_rope(IntPtr ctx, IntPtr stream, IntPtr a, IntPtr b, IntPtr c, int m, int n, int k,
+            IntPtr cosCache, IntPtr sinCache, int headDim, int ropeCols, int seqLen, int startPosition);
+
         // ---- storage conversions
         [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_convert_f32_to_f16(IntPtr ctx, IntPtr stream, IntPtr input, IntPtr output, long n);
         [DllImport(Lib, CallingConvention = CC)] internal static extern int aidn_mi355_convert_f16_to_f32(IntPtr ctx, IntPtr stream, IntPtr input, IntPtr output, long n);

@@ -157,6 +157,22 @@ AIDN_API int aidn_mi355_hgemm_f16out(void* ctx, void* stream, const uint16_t* A,
 AIDN_API int aidn_mi355_bf16gemm_f32out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, float* C, int M, int N, int K);
 AIDN_API int aidn_mi355_bf16gemm_bf16out(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K);
 
+/* ---- projection + rotary embedding in one call ---------------------------------------------------------
+ * C[M,N] = A[M,K] * B[K,N] (fp32 accumulation, C rounded to the inputs' type), then the interleaved rotary embedding of
+ * aidn_mi355_rope_interleaved_* over the first rope_cols columns of C: those columns are heads of head_dim elements side by
+ * side (the Q and K parts of a concatenated [Wq|Wk|Wv] projection; rope_cols = N rotates everything, a multiple of head_dim), the
+ * pair (2i, 2i+1) of a head in row m turns by the angle of position start_position + m % seq_len (rows are [leading, seq_len]:
+ * M = batch and seq_len = 1 in a decode step).  The result is what the product followed by the rotation kernel gives, rounding
+ * included.  Where the product has a summing pass of its own (few rows: the weight is streamed once in K ranges side by side,
+ * the decode-step shapes) the rotation rides on that pass and no separate launch is made; other shapes run the rotation as a
+ * second launch over C.  The decode step the reference composes from SimdGemm.SgemmConcatenatedProjections
+ * (Engines/Simd/SimdGemm.NParallelSmallM.cs:95-109) and RopeInterleaved (IDirectGpuBackend.cs:1427-1446); no single member of the
+ * reference does both. */
+AIDN_API int aidn_mi355_hgemm_rope(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                          const float* cos_cache, const float* sin_cache, int head_dim, int rope_cols, int seq_len, int start_position);
+AIDN_API int aidn_mi355_bf16gemm_rope(void* ctx, void* stream, const uint16_t* A, const uint16_t* B, uint16_t* C, int M, int N, int K,
+                             const float* cos_cache, const float* sin_cache, int head_dim, int rope_cols, int seq_len, int start_position);
+
 /* ---- storage conversions ------------------------------------------------------------------------
  * Replace IDirectGpuBackend.ConvertToFp16 / ConvertToFp32 (IDirectGpuBackend.cs:1876-1911; host
  * HipBackend.cs:11942-11981).  n = element count.  Narrowing is round-to-nearest-even; the bf16

@@ -1,5 +1,6 @@
-"""The entry points are launch-only once the workspace of the stream is sized: a decode step (three skinny projections, RoPE,
-decode attention, output projection) is captured into a HIP graph and replayed; every replay must equal the eager result.
+"""The entry points are launch-only once the workspace of the stream is sized: a decode step (query projection with the rotary
+embedding in its summing pass, decode attention, output projection) is captured into a HIP graph and replayed; every replay must
+equal the eager result, and the eager result must equal the step with projection and rotation as separate calls.
 Between replays the program does its own eager work and synchronises, and the inputs change, so stale-node effects show."""
 import math
 
@@ -27,14 +28,21 @@ def test_decode_step_under_hip_graph_matches_eager():
     att = torch.empty(B, H * D, device="cuda", dtype=torch.bfloat16)
     y = torch.empty(B, dM, device="cuda", dtype=torch.bfloat16)
 
-    def step():
-        be.Bf16Gemm(W(x), W(wq), W(q), B, H * D, dM)                                        # query projection (skinny, split-K)
-        be.RopeInterleaved(W(q), W(cos), W(sin), W(q), B * H, D, 1, S - 1, "bf16")          # rotate at position S-1, in place
+    def step(fused=True):
+        if fused:
+            # query projection (skinny, split-K) rotated at position S-1 in its summing pass: two launches instead of three
+            be.GemmRope("bf16", W(x), W(wq), W(q), B, H * D, dM, W(cos), W(sin), D, H * D, 1, S - 1)
+        else:
+            be.Bf16Gemm(W(x), W(wq), W(q), B, H * D, dM)
+            be.RopeInterleaved(W(q), W(cos), W(sin), W(q), B * H, D, 1, S - 1, "bf16")
         be.DecodeAttention("bf16", W(q), W(kc), W(vc), W(att), B, H, S, D, 1 / math.sqrt(D), Hkv, 0, True)
         be.Bf16Gemm(W(att), W(wo), W(y), B, dM, H * D)                                      # output projection
 
+    step(False); torch.cuda.synchronize()
+    unfused = y.clone(); q_unfused = q.clone()
     step(); torch.cuda.synchronize()                      # an eager run: sizes the workspace of the stream it ran on
     eager = y.clone()
+    assert torch.equal(q, q_unfused) and torch.equal(eager, unfused)      # same values, rounding included
     need = be.WorkspaceBytes()
     assert need > 0
 
