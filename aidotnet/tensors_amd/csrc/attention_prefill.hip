@@ -32,6 +32,9 @@
 namespace aidn {
 
 #define PREFILL_HEAD_GROUP 4
+#ifndef PREFILL_EXTRA_LDS
+#define PREFILL_EXTRA_LDS 0      // (timing experiments: more than 12 KB extra leaves one workgroup per CU)
+#endif
 
 template <typename T, typename OutT>
 __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
@@ -552,7 +555,7 @@ template <typename T, typename OutT>
 static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
 {
     auto kern = attn_prefill_kernel<T, OutT>;
-    constexpr int smem = 2 * 64 * 256 + 4 * 32 * 272 + 64;     // K tiles, two stages; V tiles, two stages, or the padded rows of O on their way out; the redo flags
+    constexpr int smem = 2 * 64 * 256 + 4 * 32 * 272 + 64 + PREFILL_EXTRA_LDS;     // K tiles, two stages; V tiles, two stages, or the padded rows of O on their way out; the redo flags
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
@@ -562,9 +565,14 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
     if (nblk > 0x7FFFFFFFLL || nblk <= 0) return hipErrorInvalidValue;
     // two workgroups fit a CU (LDS): that many run at once, each taking its virtual blocks in turn (a multiple of the eight
     // XCDs, which the block order counts on)
-    int dev = 0, cus = 0;
+    int dev = 0;
     if (hipError_t e = hipGetDevice(&dev)) return e;
-    if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+    static int cu_count[64] = {0};          // per device, asked once (benign if two threads ask at the same time: same value)
+    int cus = dev >= 0 && dev < 64 ? cu_count[dev] : 0;
+    if (cus == 0) {
+        if (hipError_t e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev)) return e;
+        if (dev >= 0 && dev < 64) cu_count[dev] = cus;
+    }
     const long long resident = (long long)(2 * cus) / 8 * 8;
     a.nvb = (int)nblk;
     a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));

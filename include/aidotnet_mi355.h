@@ -348,8 +348,9 @@ AIDN_API int aidn_mi355_mha_fwd_packed_bf16(void* ctx, void* stream, const uint1
 AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
 /* enabled == 0 routes every attention shape through the general kernel (the head-dim-128 16-bit fast
  * paths are then not taken), so the parity suite can hold the kernels against each other; unsplit
- * head-dim-128 prefill has two kernels, chosen by the length of a pass: enabled == 2 pins the phase-structured
- * one, enabled == 3 the software-pipelined one (each of the three is checked against the others).  Per context.
+ * head-dim-128 prefill on dense 16-bit arrays has two kernels (the software-pipelined one is the default, the
+ * phase-structured one takes the other layouts): enabled == 2 pins the phase-structured one, enabled == 3 the
+ * software-pipelined one wherever it applies (each of the three is checked against the others).  Per context.
  * No counterpart in the reference. */
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled);
 
