@@ -1132,10 +1132,13 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
         unsigned char* stg = smem + (HALF ? 0 : ((KT - 1) & 1) * STAGE) + wave * 8192;
         constexpr int ROWB = WTN * OB;                // bytes of one staged row
         constexpr int CPR = ROWB / 16;                // 16-byte chunks per staged row
-        constexpr int FIT = 8192 / (16 * ROWB);       // 16-row blocks that fit the wave's 8 KiB
+        constexpr bool POW2 = (CPR & (CPR - 1)) == 0; // the XOR swizzle of the staged rows needs a power-of-two chunk count
+        // (rows of another width, the 96 columns a wave holds of a 192-wide tile, are staged 16 bytes apart from whole rows instead: the
+        // pad moves neighbouring rows onto different banks, where unpadded rows cost a fifth of the LDS cycles of that tile in conflicts)
+        constexpr int PITCH = POW2 ? ROWB : ROWB + 16;
+        constexpr int FIT = 8192 / (16 * PITCH);      // 16-row blocks that fit the wave's 8 KiB
         constexpr int IPR0 = FIT >= 8 ? 8 : FIT >= 4 ? 4 : FIT >= 2 ? 2 : 1;
         constexpr int IPR = IPR0 < TI ? IPR0 : TI;    // blocks per round (divides TI)
-        constexpr bool POW2 = (CPR & (CPR - 1)) == 0; // the XOR swizzle of the staged rows needs a power-of-two chunk count
         const int sw = POW2 ? ((l16 >> 1) & (CPR - 1) & 7) : 0;
         const bool fused = g.bias != nullptr || g.act != 0;
         f32x4 bias4[TJ];
@@ -1162,10 +1165,10 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                         const uint32_t w0 = Elem<OutT>::narrow(v[0]) | (Elem<OutT>::narrow(v[1]) << 16);
                         const uint32_t w1 = Elem<OutT>::narrow(v[2]) | (Elem<OutT>::narrow(v[3]) << 16);
                         const int chunk = 2 * j + (g4 >> 1);
-                        *(u32x2*)(stg + row * ROWB + ((chunk ^ sw) << 4) + (g4 & 1) * 8) = u32x2{w0, w1};
+                        *(u32x2*)(stg + row * PITCH + ((chunk ^ sw) << 4) + (g4 & 1) * 8) = u32x2{w0, w1};
                     } else {
                         const int chunk = 4 * j + g4;
-                        *(u32x4*)(stg + row * ROWB + ((chunk ^ sw) << 4)) = u32x4{as_u32(v[0]), as_u32(v[1]), as_u32(v[2]), as_u32(v[3])};
+                        *(u32x4*)(stg + row * PITCH + ((chunk ^ sw) << 4)) = u32x4{as_u32(v[0]), as_u32(v[1]), as_u32(v[2]), as_u32(v[3])};
                     }
                 }
             }
@@ -1177,7 +1180,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
                     const int u = q * 64 + lane;
                     const int row = u / CPR, c = u % CPR;
-                    const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
+                    const u32x4 v = *(const u32x4*)(stg + row * PITCH + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
                     u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
                     if constexpr (NTS) __builtin_nontemporal_store(v, dst);
                     else *dst = v;
@@ -1189,7 +1192,7 @@ __global__ __launch_bounds__(512, 1) void gemm_dl16_kernel(const GemmArgs g)
                 for (int q = 0; q < IPR * 16 * CPR / 64; q++) {
                     const int u = q * 64 + lane;
                     const int row = u / CPR, c = u % CPR;
-                    const u32x4 v = *(const u32x4*)(stg + row * ROWB + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
+                    const u32x4 v = *(const u32x4*)(stg + row * PITCH + ((c ^ (POW2 ? ((row >> 1) & (CPR - 1) & 7) : 0)) << 4));
                     u32x4* dst = (u32x4*)(Cw + (long long)(ip * 16 + row) * g.ldc * OB + c * 16);
                     if (m0 + wm * WTM + ip * 16 + row >= g.M) continue;
                     if (g.c_cols > 0) {
