@@ -1,27 +1,21 @@
-// Fused attention forward for the 16-bit types at head dimension 128 (plain or causal, aligned contiguous K/V), software-pipelined:
-// the prefill form of FlashAttentionV2 / ScaledDotProductAttention behind the reference's backend slot
-// (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/HipBackend.cs:6118-6302; value semantics
+// The software-pipelined prefill kernel of attention_prefill.hip on v_mfma_f32_16x16x32 (same workgroup, tile loads, LDS layouts,
+// standing exponent reference with a safe second form, resident workgroups that take their passes in turn): fused attention forward
+// for the 16-bit types at head dimension 128 on dense arrays, behind the reference's FlashAttentionV2 / ScaledDotProductAttention
+// slot (src/AiDotNet.Tensors/Engines/DirectGpu/HIP/HipBackend.cs:6118-6302; value semantics
 // src/AiDotNet.Tensors/Engines/CpuEngine.cs:29146-29288, update order Engines/Simd/FusedAttention.cs:159-286).
 //
-// Workgroup: 128 query rows of one (batch, head), four waves of 32 rows; K and V stream through LDS as 64-key tiles (direct
-// global -> LDS loads, two stages each, one barrier per tile) and are consumed in units of 32 keys.  Formulation and LDS layouts
-// are those of attn_fwd_dl_kernel (attention.hip): S^T = K Q^T and O^T += V^T P^T on v_mfma_f32_32x32x16, lane (l32, h) holds
-// query l32 and keys 8 (r / 4) + 4 h + r % 4 of a unit, P^T in accumulator order is the B operand of the P V step.
+// Why a second instruction shape: the kernel runs at the board's power limit (1.33-1.37 kW of 1.4 kW at 1.76-1.83 GHz), where what
+// counts is the energy a flop takes, and the 16 x 16 x 32 shape moves half the accumulator registers per flop of the 32 x 32 x 16
+// one (the same loop with every MFMA replaced by two of this shape on the same operand registers ran 6-7 % faster).
 //
-// What differs is the order of the work.
-//   * Unit u's exponentials run beside the matrix work of its neighbours: one iteration issues P(u-1) V and S(u+1) = K(u+1) Q^T
-//     as one stream of 16 MFMAs (alternating, so the dependent S chain is spaced) with exp2 / convert / row sum of unit u spread
-//     one logit pair per two MFMAs.  Matrix and vector instructions of an iteration are independent of each other.  (With this
-//     instruction shape a vector instruction issued behind an MFMA costs the matrix pipe nothing up to about three per MFMA;
-//     measured on the part: 16.8 cycles per 16 cycles of matrix work with one exp2, one plain vector instruction and one 16-byte
-//     LDS read per MFMA, against 22 with v_mfma_f32_16x16x32, whose issue leaves no such room.)
-//   * No running-maximum pass: the reference m of a row only has to keep exp2 in range, it need not be the maximum
-//     (LSE = m + log2(l) holds for any m; O = acc / l does not depend on it).  It is set from the row maximum of the wave's first
-//     unit and then stands; a unit's probabilities are formed against it at once and the unit's sum tells whether one of them
-//     left the range.  Only then, and in the units at the two ends of a wave's key range (first unit, masked units), the row
-//     maxima are formed and O, l and m moved.  Per logit that leaves one FMA, one v_exp_f32, half a packed convert, half a v_dot2.
-//   * LDS fragment reads run RING - 1 MFMAs ahead of their use through a register ring that is carried from the second half of
-//     a tile into the first half of the next.
+// A wave's 32 queries are two blocks of 16 (qb), a unit's 32 keys two blocks of 16 (kb), the head dimension eight blocks of 16
+// (db).  Lane (c, g) = (lane % 16, lane / 16):
+//   S^T block (kb, qb) = K_kb Q_qb^T: the lane holds query c of the block and keys 4 g + r, r = 0..3 (accumulator layout);
+//   P^T of a query block as the B operand of P V: the lane's k-positions 8 g + e, e = 4 kb + r, ARE its eight probabilities
+//     in accumulator order (key 16 kb + 4 g + r), so P goes from the exponentials to the operand by packed converts alone,
+//     and the V^T fragment presents the keys in that order (two transposing reads: keys 4 g .. + 3 and 16 + 4 g .. + 3);
+//   O^T block (db, qb) += V^T_db P^T_qb: the lane holds query c and head-dim 16 db + 4 g + r.
+// Every fragment read from LDS (a K block of one 32-wide k-step, a V^T d-block) feeds two MFMAs, one per query block.
 #include "attention_common.hpp"
 #ifdef PREFILL_LOOP_FILE
 #include PREFILL_LOOP_FILE
@@ -47,7 +41,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int l32 = lane & 31, h = lane >> 5;
+    const int c16 = lane & 15, g4 = lane >> 4;
     // The grid is at most two workgroups per CU; a workgroup takes the virtual blocks blockIdx.x, blockIdx.x + gridDim.x, ... one
     // after the other (so that the loads that open a pass can be issued while the pass before it is still storing), and, with
     // paired causal query tiles, two passes per virtual block.  Item k of this workgroup -> (batch * head, query tile):
@@ -144,25 +138,29 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         }
     };
     // What opens a pass and can be asked for while the pass before it is still storing: the Q fragments (B operand of
-    // S^T = K Q^T: lane (l32, h) holds row l32, elements 16 s + 8 h .. + 7) and the K tiles 0 and 1, which land in the K half of the
+    // S^T = K Q^T) and the K tiles 0 and 1, which land in the K half of the
     // tile memory (the stores stage through the V half).
     typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-    u32x16 qlo, qhi;                        // k-steps 0..3 and 4..7 (held the way the assembly loop takes them)
-    auto qfrag = [&](int s) -> u32x4 {
-        return s < 4 ? u32x4{qlo[4 * s], qlo[4 * s + 1], qlo[4 * s + 2], qlo[4 * s + 3]}
-                     : u32x4{qhi[4 * s - 16], qhi[4 * s - 15], qhi[4 * s - 14], qhi[4 * s - 13]};
+    u32x16 qlo, qhi;                        // query block 0 and 1, four k-steps each (held the way the assembly loop takes them)
+    auto qfrag = [&](int qb, int ks) -> u32x4 {
+        return qb == 0 ? u32x4{qlo[4 * ks], qlo[4 * ks + 1], qlo[4 * ks + 2], qlo[4 * ks + 3]}
+                       : u32x4{qhi[4 * ks], qhi[4 * ks + 1], qhi[4 * ks + 2], qhi[4 * ks + 3]};
     };
+    // (B operand of S^T = K Q^T: lane (c, g) holds query c of the block, elements 32 ks + 8 g .. + 7)
     auto open_pass = [&](int bh, int qt) {
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        // (a lane whose row lies past the end of the sequence takes the last row: what it computes is never stored)
-        const int qrow = min(qt * BR + wave_s * 32 + (ln & 31), a.Sq - 1);
-        const uint16_t* Q = (const uint16_t*)a.q + ((long long)(bh * a.Sq) << 7) + qrow * 128 + (ln >> 5) * 8;
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            const u32x4 x = *(const u32x4*)(Q + 16 * s);
+        for (int qb = 0; qb < 2; qb++) {
+            // (a lane whose row lies past the end of the sequence takes the last row: what it computes is never stored)
+            const int qrow = min(qt * BR + wave_s * 32 + 16 * qb + (ln & 15), a.Sq - 1);
+            const uint16_t* Q = (const uint16_t*)a.q + ((long long)(bh * a.Sq) << 7) + qrow * 128 + (ln >> 4) * 8;
 #pragma unroll
-            for (int e = 0; e < 4; e++) { if (s < 4) qlo[4 * s + e] = x[e]; else qhi[4 * s - 16 + e] = x[e]; }
+            for (int ks = 0; ks < 4; ks++) {
+                const u32x4 x = *(const u32x4*)(Q + 32 * ks);
+#pragma unroll
+                for (int e = 0; e < 4; e++) { if (qb == 0) qlo[4 * ks + e] = x[e]; else qhi[4 * ks + e] = x[e]; }
+            }
         }
         // (H = Hkv * group: K/V head b Hkv + head / group is (b H + head) / group)
         const uint16_t* K = (const uint16_t*)a.k + ((long long)((int)fastdiv((uint32_t)bh, a.dgroup) * Sk) << 7);
@@ -183,7 +181,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #define STAMP(i)
 #endif
     const int q0 = qt * BR;
-    const int qi = q0 + wave * 32 + l32;
+    const int qi[2] = {q0 + wave * 32 + c16, q0 + wave * 32 + 16 + c16};
     const long long kv_first = (long long)((int)fastdiv((uint32_t)bh, a.dgroup) * Sk) << 7;      // first element of the head's K and V
     const raw_t* __restrict__ K = (const raw_t*)a.k + kv_first;
     const raw_t* __restrict__ V = (const raw_t*)a.v + kv_first;
@@ -202,27 +200,28 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     nu = __builtin_amdgcn_readfirstlane(nu);
     // a unit all of whose keys every row of the wave sees needs no mask: units 0 .. ufull
     const int ufull = __builtin_amdgcn_readfirstlane((key_limit(wq_min) + 1) / 32 - 1);
-    const int klim = key_limit(qi) - 4 * h;          // element r of unit u is masked when 32 u + 8 (r / 4) + r % 4 > klim
+    // element r of S^T block (kb, qb) in unit u is masked when 32 u + 16 kb + r > klim[qb]
+    const int klim[2] = {key_limit(qi[0]) - 4 * g4, key_limit(qi[1]) - 4 * g4};
 
     // LDS read addresses (per lane).  The two stages of the K tiles are 32 KB of four 32-key units, unit index j at offset
     // (j % 4) * 8 KB, and so are the V tiles: the K and the V addresses each point at one unit and move to the next one by an
     // XOR (8 KB when leaving an even unit, 24 KB when leaving an odd one).
-    //   K fragment (k-step s of the unit): key l32, chunk (2 s + h) ^ (key & 15); the upper four k-steps by an XOR of bit 7
-    //   V^T fragment (s = 4 * (16-key half) + head-dim block): two transposing reads 8 keys apart; in a 16-lane group lane j
-    //   addresses key 4 h + j / 4 and the 8 bytes at head-dim 4 (j % 4) of its 16-wide block
+    //   K fragment (block kb, k-step ks): key 16 kb + c, chunk (4 ks + g) ^ c; the k-steps differ by an XOR of bits 6-7, kb by 4 KB
+    //   V^T fragment of d-block db: two transposing reads 16 keys apart; in the 16-lane group g lane c addresses key 4 g + c / 4 and
+    //   the 8 bytes at head-dim 4 (c % 4) of the block; d-block pairs differ by an XOR of bits 6-7, the odd block by 32 bytes
     uint32_t k_ad[4], v_ad[4];
     int k_unit = 0, v_unit = 0;
     {
         // (from an opaque copy of the lane index, so that these are formed here, per pass, rather than kept across the passes)
         int ln = lane;
         asm volatile("" : "+v"(ln));
-        const int jl = ln & 15, l32p = ln & 31, hp = ln >> 5;
-        const uint32_t k_lane = l32p * 256 + ((hp ^ (l32p & 15)) << 4);
-        const uint32_t v_lane = (4 * hp + (jl >> 2)) * 256 + ((16 * ((ln >> 4) & 1) + 4 * (jl & 3)) >> 3) * 16 + (jl & 1) * 8 + ((jl >> 2) << 6);
+        const int cp = ln & 15, gp = ln >> 4;
+        const uint32_t k_lane = cp * 256 + ((gp ^ cp) << 4);
+        const uint32_t v_lane = (4 * gp + (cp >> 2)) * 256 + ((((cp & 3) >> 1) ^ (((cp >> 2) & 3) << 2)) << 4) + (cp & 1) * 8;
 #pragma unroll
-        for (int s = 0; s < 4; s++) k_ad[s] = (lds0 + k_lane) ^ (uint32_t)(s << 5);
+        for (int ks = 0; ks < 4; ks++) k_ad[ks] = (lds0 + k_lane) ^ (uint32_t)(ks << 6);
 #pragma unroll
-        for (int i = 0; i < 4; i++) v_ad[i] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(i << 6);
+        for (int j = 0; j < 4; j++) v_ad[j] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(j << 6);
     }
     auto next_k_unit = [&]() {
         const uint32_t x = (k_unit & 1) ? 24576u : 8192u;
@@ -236,78 +235,105 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         for (int i = 0; i < 4; i++) v_ad[i] ^= x;
         v_unit++;
     };
-    auto k_frag = [&](int s) -> u32x4 {
-        return *(const __attribute__((address_space(3))) u32x4*)(s < 4 ? k_ad[s] : (k_ad[s - 4] ^ 128u));
+    auto k_frag = [&](int kb, int ks) -> u32x4 {
+        return *(const __attribute__((address_space(3))) u32x4*)(k_ad[ks] + kb * 4096);
     };
-    auto v_frag = [&](int s) -> u32x4 {
-        const uint32_t ad = v_ad[s & 3] + 16 * (s >> 2) * 256;
+    auto v_frag = [&](int db) -> u32x4 {
+        const uint32_t ad = v_ad[db >> 1] + (db & 1) * 32;
         u32x2 w0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)ad));
-        u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 8 * 256)));
+        u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 16 * 256)));
         return u32x4{w0[0], w0[1], w1[0], w1[1]};
     };
+    auto mma16 = [&](f32x4 acc, const u32x4& x, const u32x4& y) -> f32x4 {
+        if constexpr (std::is_same<T, f16_t>::value)
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, x), __builtin_bit_cast(f16x8, y), acc, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, x), __builtin_bit_cast(bf16x8, y), acc, 0, 0, 0);
+    };
 
+    // (sixteen-register groups, the way the assembly loop takes them: O block (db, qb) is elements 4 ((2 db + qb) % 4) .. + 3 of
+    // oacc[db / 2], logit block (kb, qb) elements 4 (2 kb + qb) .. + 3 of sacc)
     f32x16 oacc[4];
-    f32x16 sacc;                   // logits of one unit (S^T accumulator layout), then its exponentials in place
-    u32x4 pf[2];                   // [16-key half]: packed probabilities of one unit, the B operand of the P V step
-    float m_ref = -INFINITY;       // reference point of the exponent (log2 domain); the same in lanes l and l ^ 32
-    float l_run = 0.0f;
+    f32x16 sacc;                   // logits of one unit, then its exponentials in place
+    u32x4 pf[2];                   // [query block]: packed probabilities of one unit, the B operand of the P V step
+    float m_ref[2] = {-INFINITY, -INFINITY};   // per query block: reference point of the exponent (log2 domain); the same in the four lanes of a query
+    float l_run[2] = {0.0f, 0.0f};
+    auto get4 = [&](const f32x16& v, int at) -> f32x4 { return f32x4{v[4 * at], v[4 * at + 1], v[4 * at + 2], v[4 * at + 3]}; };
+    auto put4 = [&](f32x16& v, int at, const f32x4& x) { v[4 * at] = x[0]; v[4 * at + 1] = x[1]; v[4 * at + 2] = x[2]; v[4 * at + 3] = x[3]; };
+    // a value of the four lanes (g = 0..3) that share a query: maximum / sum over them
+    auto max_over_g = [&](float v) -> float { v = fmaxf(v, __shfl_xor(v, 16, 64)); return max_with_partner32(v); };
+    auto sum_over_g = [&](float v) -> float { v += __shfl_xor(v, 16, 64); return sum_with_partner32(v); };
 
     // ---- plain (not interleaved) forms of the three steps of a unit
     auto qk_plain = [&]() {                                    // S of the unit the K addresses point to
 #pragma unroll
         for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            Mma32<T>::run(sacc, k_frag(s), qfrag(s));
-            if (s == 3) __builtin_amdgcn_sched_barrier(0);
+        for (int ks = 0; ks < 4; ks++) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const u32x4 kf = k_frag(kb, ks);
+#pragma unroll
+                for (int qb = 0; qb < 2; qb++) put4(sacc, 2 * kb + qb, mma16(get4(sacc, 2 * kb + qb), kf, qfrag(qb, ks)));
+            }
+            if (ks == 1) __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto pv_plain = [&]() {                                    // O += V^T P^T, unit the V addresses point to
 #pragma unroll
-        for (int s = 0; s < 8; s++) {
-            Mma32<T>::run(oacc[s & 3], v_frag(s), pf[s >> 2]);
-            if (s == 3) __builtin_amdgcn_sched_barrier(0);
+        for (int db = 0; db < 8; db++) {
+            const u32x4 vf = v_frag(db);
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) put4(oacc[db >> 1], (2 * db + qb) & 3, mma16(get4(oacc[db >> 1], (2 * db + qb) & 3), vf, pf[qb]));
+            if (db == 3) __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto mask_unit = [&](int u) {
-        const int rel = klim - 32 * u;
 #pragma unroll
-        for (int r = 0; r < 16; r++)
-            if (8 * (r >> 2) + (r & 3) > rel) sacc[r] = -INFINITY;
+        for (int t = 0; t < 16; t++) {
+            const int kb = t >> 3, qb = (t >> 2) & 1, r = t & 3;
+            if (16 * kb + r > klim[qb] - 32 * u) sacc[t] = -INFINITY;
+        }
     };
     // Probabilities of unit u with the row maxima formed first (the safe form, also the wave's first unit in the fast form): the
     // reference of a row is raised when the row's maximum lies more than 8 above it (always on first use).  Adds the row sums to l.
     auto softmax_exact = [&](int u, bool apply_mask, const bool first) {
         if (apply_mask) mask_unit(u);
-        float m = -INFINITY;
 #pragma unroll
-        for (int r = 0; r < 16; r++) m = fmaxf(m, sacc[r]);
-        const float mloc = max_with_partner32(m) * sl2;            // scale > 0: max commutes with the scaling
-        if (first) {
-            m_ref = mloc < INFINITY ? mloc : -INFINITY;            // nothing accumulated yet: no O or l to move
-        } else {
-            // (the accumulators are scaled whether a reference moves or not, by 1 if not: a branch around the scaling costs more,
-            // in copies of all 64 of them, than the scaling)
-            const float m_new = (mloc > m_ref + 8.0f && mloc < INFINITY) ? mloc : m_ref;
-            const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref - m_new);
-            m_ref = m_new;
-            l_run *= alpha;
+        for (int qb = 0; qb < 2; qb++) {
+            float m = -INFINITY;
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+                for (int r = 0; r < 4; r++) m = fmaxf(m, sacc[8 * kb + 4 * qb + r]);
+            const float mloc = max_over_g(m) * sl2;                    // scale > 0: max commutes with the scaling
+            if (first) {
+                m_ref[qb] = mloc < INFINITY ? mloc : -INFINITY;        // nothing accumulated yet: no O or l to move
+            } else {
+                // (the accumulators are scaled whether a reference moves or not, by 1 if not: a branch around the scaling costs
+                // more, in copies of all of them, than the scaling)
+                const float m_new = (mloc > m_ref[qb] + 8.0f && mloc < INFINITY) ? mloc : m_ref[qb];
+                const float alpha = (m_new == -INFINITY) ? 1.0f : __builtin_amdgcn_exp2f(m_ref[qb] - m_new);
+                m_ref[qb] = m_new;
+                l_run[qb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < 8; db++)
+#pragma unroll
+                    for (int r = 0; r < 4; r++) oacc[db >> 1][4 * ((2 * db + qb) & 3) + r] *= alpha;
+            }
+            const float m_use = (m_ref[qb] == -INFINITY) ? 0.0f : m_ref[qb];
+            float ps = 0.0f;
+#pragma unroll
+            for (int e2 = 0; e2 < 4; e2++) {
+                const int t0 = 8 * (e2 >> 1) + 4 * qb + 2 * (e2 & 1);
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[t0], sl2, -m_use));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[t0 + 1], sl2, -m_use));
+                const uint32_t pk = pack2_p<T>(p0, p1);
+                ps = add_pair<T>(pk, ps);
+                pf[qb][e2] = pk;
+            }
+            l_run[qb] += ps;
         }
-        const float m_use = (m_ref == -INFINITY) ? 0.0f : m_ref;
-        float ps = 0.0f;
-#pragma unroll
-        for (int pi = 0; pi < 8; pi++) {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[2 * pi], sl2, -m_use));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[2 * pi + 1], sl2, -m_use));
-            const uint32_t pk = pack2_p<T>(p0, p1);
-            ps = add_pair<T>(pk, ps);
-            pf[pi >> 2][pi & 3] = pk;
-        }
-        l_run += ps;
     };
     // what every wave does once per unit whether it computes or not: before an odd unit the loads of K(t+2) and V(t+1) (t = u / 2:
     // the tiles they replace went out of use at the barrier just passed), after an even unit the barrier that publishes K(t+1), V(t)
@@ -333,13 +359,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         typedef uint32_t u32x8 __attribute__((ext_vector_type(8)));
         // read addresses of unit 0 (the K addresses stand at unit u + 1, the V addresses at unit u - 1)
         const uint32_t koff = (uint32_t)((u + 1) & 3) << 13, voff = (uint32_t)((u - 1) & 3) << 13;
-        const u32x4 kad0 = {k_ad[0] ^ koff, k_ad[1] ^ koff, k_ad[2] ^ koff, k_ad[3] ^ koff};
-        const u32x4 kad1 = {kad0[0] ^ 128u, kad0[1] ^ 128u, kad0[2] ^ 128u, kad0[3] ^ 128u};
+        const u32x4 kad = {k_ad[0] ^ koff, k_ad[1] ^ koff, k_ad[2] ^ koff, k_ad[3] ^ koff};
         const u32x4 vad = {v_ad[0] ^ voff, v_ad[1] ^ voff, v_ad[2] ^ voff, v_ad[3] ^ voff};
         const u32x4 klo = {k_lane_off, k_lane_off ^ 64u, k_lane_off ^ 128u, k_lane_off ^ 192u};
         const uint32_t vlo = v_lane_off;
-        const float negm = (m_ref == -INFINITY) ? -0.0f : -m_ref;
-        float ps = 0.0f;
+        const float negm0 = (m_ref[0] == -INFINITY) ? -0.0f : -m_ref[0], negm1 = (m_ref[1] == -INFINITY) ? -0.0f : -m_ref[1];
+        float ps0 = 0.0f, ps1 = 0.0f;
         const int tl = u >> 1;
         unsigned long long kptr = (unsigned long long)(uintptr_t)((const unsigned char*)K + (long long)((tl + 2) * BC + 16 * wave_s) * k_row_bytes);
         unsigned long long vptr = (unsigned long long)(uintptr_t)((const unsigned char*)V + (long long)((tl + 1) * BC + 16 * wave_s) * v_row_bytes);
@@ -352,24 +377,25 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         const int phase = __builtin_amdgcn_readfirstlane((u - 1) & 3);
         // (with masked_last the run is n whole units and then unit u + n, masked first; n >= 1)
         int mask_follows = __builtin_amdgcn_readfirstlane(masked_last ? 1 : 0);
-        const int mask_rel = klim - 32 * (u + n);
+        const int mask_rel0 = klim[0] - 32 * (u + n), mask_rel1 = klim[1] - 32 * (u + n);
         const float ninf = -INFINITY;
         if (masked_last) n++;
         u32x4 p0 = pf[0], p1 = pf[1];
 #define PREFILL_LOOP_OPERANDS \
             : "+{v[0:15]}"(oacc[0]), "+{v[16:31]}"(oacc[1]), "+{v[32:47]}"(oacc[2]), "+{v[48:63]}"(oacc[3]), "+{v[64:79]}"(sacc), \
-              "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v170}"(ps), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft), "+{s59}"(mask_follows) \
-            : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad0), "{v[156:159]}"(kad1), "{v[160:163]}"(vad), \
-              "{v[164:167]}"(klo), "{v168}"(vlo), "{v169}"(negm), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), "{v171}"(mask_rel), "{v174}"(ninf) \
+              "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v167}"(ps0), "+{v168}"(ps1), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft), "+{s59}"(mask_follows) \
+            : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad), "{v[156:159]}"(vad), \
+              "{v[160:163]}"(klo), "{v164}"(vlo), "{v165}"(negm0), "{v166}"(negm1), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), \
+              "{v171}"(mask_rel0), "{v172}"(mask_rel1), "{v173}"(ninf) \
             : "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", \
               "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \
-              "v150", "v151", "v172", "v173", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", \
+              "v150", "v151", "v169", "v170", "v176", "v177", "v178", "v179", "v180", "v181", "v182", "v183", "v184", "v185", "v186", \
               "v187", "v188", "v189", "v190", "v191", "s54", "s55", "scc", "vcc", "memory"
         if constexpr (std::is_same<T, f16_t>::value) asm volatile(PREFILL_LOOP_F16 PREFILL_LOOP_OPERANDS);
         else asm volatile(PREFILL_LOOP_BF16 PREFILL_LOOP_OPERANDS);
 #undef PREFILL_LOOP_OPERANDS
         pf[0] = p0; pf[1] = p1;
-        l_run += ps;
+        l_run[0] += ps0; l_run[1] += ps1;
         for (int i = 0; i < (n & 3); i++) { next_k_unit(); next_v_unit(); }
         k_unit += n & ~3; v_unit += n & ~3;
     };
@@ -385,7 +411,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #pragma unroll
     for (int r = 0; r < 16; r++) sacc[r] = 0.0f;
     pf[0] = u32x4{0u, 0u, 0u, 0u}; pf[1] = u32x4{0u, 0u, 0u, 0u};
-    m_ref = -INFINITY; l_run = 0.0f;
+    m_ref[0] = m_ref[1] = -INFINITY; l_run[0] = l_run[1] = 0.0f;
     while (k_unit & 3) next_k_unit();           // (a second attempt starts from unit 0 again)
     while (v_unit & 3) next_v_unit();
     k_unit = 0; v_unit = 0;
@@ -440,7 +466,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     if (nunits - 1 < nu && nunits > 0) pv_plain();       // P V of the workgroup's last unit
     STAMP(4);
     if (!safe) {
-        const bool left_range = __builtin_amdgcn_ballot_w64(!(l_run < 1.2676506e30f)) != 0ull;
+        const bool left_range = __builtin_amdgcn_ballot_w64(!(l_run[0] < 1.2676506e30f) || !(l_run[1] < 1.2676506e30f)) != 0ull;
         if (lane == 0) redo_flag[wave] = left_range ? 1u : 0u;
         __syncthreads();                        // the flags are written, and every wave is past its last fragment read
         const u32x4 fl = *(const u32x4*)redo_flag;
@@ -456,28 +482,38 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     if (item + 1 < nitems) { decode(item + 1, bh_next, qt_next); open_pass(bh_next, qt_next); }
     STAMP(8);
     // ---- epilogue: normalise, store
-    const float l_tot = sum_with_partner32(l_run);
-    const float inv = l_tot > 0.0f ? 1.0f / l_tot : 0.0f;
+    float l_tot[2], inv[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; qb++) {
+        l_tot[qb] = sum_over_g(l_run[qb]);
+        inv[qb] = l_tot[qb] > 0.0f ? 1.0f / l_tot[qb] : 0.0f;
+    }
+#pragma unroll
+    for (int db = 0; db < 8; db++)
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) oacc[db >> 1][4 * ((2 * db + qb) & 3) + r] *= inv[qb];
+    if (a.lse && g4 == 0) {
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++)
+            if (qi[qb] < a.Sq)
+                a.lse[(long long)bh * a.Sq + qi[qb]] = l_tot[qb] > 0.0f ? (m_ref[qb] + __builtin_amdgcn_logf(l_tot[qb])) * LN2 : -INFINITY;
+    }
     if (Elem<OutT>::BYTES == 4 && a.vec_out) {
-        // fp32 O through LDS: the lane holds 16-byte pieces of ONE row (64 rows per store instruction, each a partial line); staged
-        // per wave, one half of the head dimension at a time, as [32 rows][256 B + 16] (the pad keeps neighbouring rows on different
-        // banks, and leaves every LDS address a lane constant plus an immediate) in the V half of the tile memory (the K half is
-        // receiving the next pass's tiles) and written back as 256-byte row halves, whole lines, with non-temporal stores (O is
-        // written once and would otherwise displace K and V tiles that other workgroups re-read).
+        // fp32 O through LDS: the lane holds 16-byte pieces of two rows (one per query block; a store instruction would touch 32 rows,
+        // each a partial line); staged per wave, one half of the head dimension at a time, as [32 rows][256 B + 16] (the pad keeps
+        // neighbouring rows on different banks, and leaves every LDS address a lane constant plus an immediate) in the V half of
+        // the tile memory (the K half is receiving the next pass's tiles) and written back as 256-byte row halves, whole lines,
+        // with non-temporal stores (O is written once and would otherwise displace K and V tiles that other workgroups re-read).
         constexpr int SROW = 272;
         unsigned char* stg = smem + 2 * KBYTES + wave_s * (32 * SROW);
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) oacc[i][r] *= inv;
-        if (a.lse && h == 0 && qi < a.Sq)
-            a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
         // (lane constants from an opaque copy of the lane index: they are then formed here, not ahead of the loops)
         int lnw = lane;
         asm volatile("" : "+v"(lnw));
-        unsigned char* wr = stg + (lnw & 31) * SROW + (lnw >> 5) * 16;                  // chunk 8 (i % 2) + 2 g + h of row l32
+        unsigned char* wr = stg + (lnw & 15) * SROW + (lnw >> 4) * 16;                  // piece (db % 4, g) of row 16 qb + c
         const unsigned char* rd = stg + (lnw >> 4) * SROW + (lnw & 15) * 16;           // chunk lane % 16 of row 4 q + lane / 16
-        // the wave's 32 output rows: a uniform base, a 32-bit lane offset (the launcher checks that 32 rows span less than 4 GB)
+        // the wave's 32 output rows: a uniform base, a 32-bit lane offset
         unsigned char* obase = (unsigned char*)((float*)a.o + ((long long)(bh * a.Sq + q0 + wave_s * 32) << 7));
         constexpr uint32_t row_bytes = 512u;
         const uint32_t lane_off = (uint32_t)(lnw >> 4) * row_bytes + (uint32_t)(lnw & 15) * 16u;
@@ -485,11 +521,12 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #pragma unroll
         for (int half = 0; half < 2; half++) {
 #pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int d4 = 0; d4 < 4; d4++)
 #pragma unroll
-                for (int g = 0; g < 4; g++)
-                    *(f32x4*)(wr + (8 * i + 2 * g) * 16) = f32x4{oacc[2 * half + i][4 * g + 0], oacc[2 * half + i][4 * g + 1],
-                                                                 oacc[2 * half + i][4 * g + 2], oacc[2 * half + i][4 * g + 3]};
+                for (int qb = 0; qb < 2; qb++) {
+                    const int db = 4 * half + d4, at = 4 * ((2 * db + qb) & 3);
+                    *(f32x4*)(wr + qb * 16 * SROW + d4 * 64) = f32x4{oacc[db >> 1][at], oacc[db >> 1][at + 1], oacc[db >> 1][at + 2], oacc[db >> 1][at + 3]};
+                }
             f32x4 piece[8];
 #pragma unroll
             for (int q = 0; q < 8; q++) piece[q] = *(const f32x4*)(rd + 4 * q * SROW);
@@ -507,16 +544,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             if (half == 0) STAMP(9);
 #endif
         }
-    } else if (qi < a.Sq) {
+    } else {
         typedef typename Raw2<OutT>::type out_t;
-        out_t* __restrict__ O = (out_t*)a.o + ((long long)(bh * a.Sq + qi) << 7);
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int qb = 0; qb < 2; qb++) {
+            if (qi[qb] >= a.Sq) continue;
+            out_t* __restrict__ O = (out_t*)a.o + ((long long)(bh * a.Sq + qi[qb]) << 7);
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int d0 = i * 32 + 8 * g + 4 * h;
-                const float v0 = oacc[i][4 * g + 0] * inv, v1 = oacc[i][4 * g + 1] * inv;
-                const float v2 = oacc[i][4 * g + 2] * inv, v3 = oacc[i][4 * g + 3] * inv;
+            for (int db = 0; db < 8; db++) {
+                const int d0 = 16 * db + 4 * g4, at = 4 * ((2 * db + qb) & 3);
+                const float v0 = oacc[db >> 1][at], v1 = oacc[db >> 1][at + 1], v2 = oacc[db >> 1][at + 2], v3 = oacc[db >> 1][at + 3];
                 if constexpr (Elem<OutT>::BYTES == 4) {
                     O[d0] = as_u32(v0); O[d0 + 1] = as_u32(v1); O[d0 + 2] = as_u32(v2); O[d0 + 3] = as_u32(v3);
                 } else {
@@ -527,8 +564,6 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
                 }
             }
         }
-        if (a.lse && h == 0)
-            a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
     }
     STAMP(6);
 #ifdef PREFILL_DBG
@@ -563,6 +598,9 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
     a.paired = (a.causal && a.qoff == 0 && a.Sq == a.Sk && a.qtiles >= 2 && a.qtiles % 2 == 0) ? 1 : 0;
     const long long nblk = (long long)(a.paired ? a.qtiles / 2 : a.qtiles) * a.B * a.H;
     if (nblk > 0x7FFFFFFFLL || nblk <= 0) return hipErrorInvalidValue;
+    a.nvb = (int)nblk;
+    a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));
+    a.dunits = make_fastdiv((uint32_t)(a.qtiles / 2 > 0 ? a.qtiles / 2 : 1)); a.dqtiles = make_fastdiv((uint32_t)a.qtiles);
     // two workgroups fit a CU (LDS): that many run at once, each taking its virtual blocks in turn (a multiple of the eight
     // XCDs, which the block order counts on)
     int dev = 0;
@@ -574,9 +612,6 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
         if (dev >= 0 && dev < 64) cu_count[dev] = cus;
     }
     const long long resident = (long long)(2 * cus) / 8 * 8;
-    a.nvb = (int)nblk;
-    a.dgroup = make_fastdiv((uint32_t)(a.H / a.Hkv));
-    a.dunits = make_fastdiv((uint32_t)(a.qtiles / 2 > 0 ? a.qtiles / 2 : 1)); a.dqtiles = make_fastdiv((uint32_t)a.qtiles);
     const unsigned grid = (unsigned)((resident >= 8 && nblk > resident) ? resident : nblk);
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, a);
     return hipGetLastError();

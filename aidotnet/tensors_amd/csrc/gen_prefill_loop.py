@@ -6,62 +6,67 @@ The routine is written out by hand because the kernel's time follows what its wa
 scalar work of the tile loads reduced to what the loads need, waits only where a fragment can still be outstanding.  The code is
 four blocks, one per position of a unit in the two LDS stages (unit u uses block (u - 1) % 4), so every LDS offset is an
 immediate; a run enters at the block of its first unit (through that block's cold start, which requests the first seven
-fragments) and leaves behind any block.
+fragments) and leaves behind any block; with s59 set one more unit follows the run whose logits are masked first (the unit on the
+causal diagonal).
 
-Per unit u a block issues, as the C++ form of the block (full_block) does:
-  slots 0..7   P(u-1) V: v_mfma into the four O accumulators; beside them FMA + exp2 of the logits of unit u (two per slot)
-  slots 8..15  S(u+1) = K Q^T: v_mfma chain into the logit registers; beside them packed convert + row sum (one pair per slot)
-  every slot   the LDS read of the fragment seven MFMAs ahead (ring of eight), one wait per two MFMAs, counted from the reads in flight
-  odd units    the direct-to-LDS loads of K(t+2), V(t+1), one per slot 0..7, while s57 / s58 say a K / V tile is left to load
-               (K and V rows are 256 bytes apart: the four loads of a wave's share differ by an immediate offset)
-  even units   the tile barrier at slot 9, behind this unit's last fragment read and ahead of the first read of the next unit
-
-Register assignment (fixed; the kernel binds its variables to these registers at the asm statement):
-  v[0:63] O accumulators, v[64:79] logits, v[80:87] P (two k-steps), v[88:119] Q fragments, v[120:151] fragment ring,
-  v[152:159] K read addresses per k-step, v[160:163] V read addresses per head-dim block, v[164:167] lane offsets of the four K
-  wave-loads, v168 lane offset of the V wave-loads, v169 minus the exponent reference, v170 running row sum,
-  v172 v173 scratch, v[176:191] exponentials.
-  s[40:41] / s[42:43] source of this wave's next K / V tile load, s44 s45 unused, s[46:47] s[48:49] one K / V tile in bytes, s50 s51 LDS destination of this wave's K / V loads in stage 0, s52 scale * log2(e), s53 units left,
-  s[54:55] scratch, s56 block of the first unit, s57 s58 odd units that still load a K / V tile, s59 whether a masked unit
-  follows the run (then v171 holds the lane's key limit inside that unit and v174 minus infinity).
-
-A second argument names parts to leave out (dma, barrier, valu, lds, vmwait): timing experiments only, the results are wrong.
+No arguments: the routine into attention_prefill_loop.inc beside this script.  FILE PARTS: the routine into FILE with the comma-
+separated PARTS left out (dma, barrier, valu, lds: timing experiments only, the results are wrong).
 """
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def gen(kind, dma=True, ablate=()):
-    mfma = "v_mfma_f32_32x32x16_" + kind
+def gen(kind, ablate=()):
+    """One routine on v_mfma_f32_16x16x32.  A wave's 32 queries are two blocks of 16 (qb), a unit's 32 keys two blocks of 16 (kb),
+    the head dimension eight blocks of 16 (db); every fragment read from LDS feeds two MFMAs (one per query block).  Lane (c, g) =
+    (lane % 16, lane / 16) holds query c of a block and keys / dims 4 g + r of a block.  Per unit u a block has 16 slots, slot i
+    consuming fragment i:
+      slots 0..7   the V^T fragment of d-block i: P(u-1) V into the accumulators of both query blocks; beside them FMA + exp2 of the
+                   logits of unit u (two per slot)
+      slots 8..15  the K fragment (kb, ks) = ((i - 8) % 2, (i - 8) / 2): the S(u+1) chains of both query blocks; beside them packed
+                   convert + row sum (one pair per slot)
+      every slot   the LDS read of the fragment seven slots ahead (ring of eight), one wait per two slots, counted from the reads in flight
+      odd units    the direct-to-LDS loads of K(t+2), V(t+1), one per slot 0..7, while s57 / s58 say a K / V tile is left to load
+                   (K and V rows are 256 bytes apart: the four loads of a wave's share differ by an immediate offset)
+      even units   the tile barrier at slot 9, behind this unit's last fragment read and ahead of the first read of the next unit
+
+    Registers (fixed; the kernel binds its variables to them at the asm statement): v[0:63] O (block (db, qb) at 4 (2 db + qb)),
+    v[64:79] logits (block (kb, qb) at 64 + 4 (2 kb + qb)), v[80:87] P (qb 0, qb 1), v[88:119] Q (block (qb, ks) at
+    88 + 4 (4 qb + ks)), v[120:151] fragment ring, v[152:155] K read addresses per ks (kb by an offset), v[156:159] V read
+    addresses per pair of d-blocks, v[160:163] lane offsets of the four K wave-loads, v164 of the V wave-loads, v165 v166 minus the
+    exponent reference of query block 0 / 1, v167 v168 their running row sums, v169 v170 scratch, v171 v172 the lane's key limit
+    inside a masked unit per query block, v173 minus infinity, v[176:191] exponentials.
+    s[40:41] / s[42:43] source of this wave's next K / V tile load, s[46:47] s[48:49] one K / V tile in bytes, s50 s51 LDS
+    destination of this wave's K / V loads in stage 0, s52 scale * log2(e), s53 units left, s56 block of the first unit, s57 s58
+    odd units that still load a K / V tile, s59 whether a masked unit follows the run."""
+    mfma = "v_mfma_f32_16x16x32_" + kind
     cvt = "v_cvt_pk_%s_f32" % kind
     dot = "v_dot2c_f32_%s_e32" % kind
     ones = "0x3c003c00" if kind == "f16" else "0x3f803f80"
     out = []
     emit = out.append
-    queue = []          # LDS read instructions issued and not yet known complete, oldest first: fragment ids (block, index)
+    queue = []
 
-    def fr(j):          # ring register tuple of stream position j
-        b = 120 + 4 * (j % 8)
-        return b
+    def fr(j):
+        return 120 + 4 * (j % 8)
 
     def read_frag(blk, f):
-        """LDS reads of fragment f (0..7 V^T, 8..15 K) of block blk (0..3) into its ring slot."""
         b = fr(f)
         if "lds" in ablate:
             return
         if f < 8:
-            voff = blk * 8192 + 16 * (f >> 2) * 256
-            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b, b + 1, 160 + (f & 3), voff))
-            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b + 2, b + 3, 160 + (f & 3), voff + 2048))
+            voff = blk * 8192 + (f & 1) * 32
+            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b, b + 1, 156 + (f >> 1), voff))
+            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b + 2, b + 3, 156 + (f >> 1), voff + 4096))
             queue.append((blk, f)); queue.append((blk, f))
         else:
-            koff = ((blk + 2) & 3) * 8192
-            emit("ds_read_b128 v[%d:%d], v%d offset:%d" % (b, b + 3, 152 + (f - 8), koff))
+            j = f - 8
+            koff = ((blk + 2) & 3) * 8192 + (j & 1) * 4096
+            emit("ds_read_b128 v[%d:%d], v%d offset:%d" % (b, b + 3, 152 + (j >> 1), koff))
             queue.append((blk, f))
 
     def wait_frag(blk, f):
-        """Wait until every read of fragment (blk, f) has returned (reads return in issue order)."""
         last = -1
         for n, q in enumerate(queue):
             if q == (blk, f):
@@ -75,70 +80,71 @@ def gen(kind, dma=True, ablate=()):
 
     label = "L_prefill_%s_" % kind
     first7 = lambda blk: [(blk, f) for f in range(7) for _ in (0, 1)]
-    # entry: s56 = phase of the first unit ((u - 1) % 4), s53 = units to run (at least one); each phase has its cold start
     for j in (1, 2, 3):
         emit("s_cmp_eq_u32 s56, %d" % j)
         emit("s_cbranch_scc1 %spre%d_%%=" % (label, j))
-    for j in range(4):                      # (the compare chain above falls through into phase 0)
+    for j in range(4):
         emit("%spre%d_%%=:" % (label, j))
         del queue[:]
         for f in range(7):
             read_frag(j, f)
         emit("s_branch %sblk%d_%%=" % (label, j))
+
     def slot(blk, i, is_b, dma):
-        """Slot i of block blk: the wait for its fragments (one wait per pair of slots), the MFMA, the fragment read seven ahead, this
-        wave's tile load of the slot (B blocks, when dma), the vector work."""
         if not is_b and i == 9:
-            emit("s_waitcnt lgkmcnt(0)" if "vmwait" in ablate else "s_waitcnt vmcnt(0) lgkmcnt(0)")
+            emit("s_waitcnt vmcnt(0) lgkmcnt(0)")
             del queue[:]
             if "barrier" not in ablate:
                 emit("s_barrier")
         if (i & 1) == 0:
             wait_frag(blk, i + 1)
         else:
-            wait_frag(blk, i)               # (nothing to wait for unless the barrier slot came between)
+            wait_frag(blk, i)
+        f4 = "v[%d:%d]" % (fr(i), fr(i) + 3)
         if i < 8:
-            acc = 16 * (i & 3)
-            emit("%s v[%d:%d], v[%d:%d], v[%d:%d], v[%d:%d]" % (mfma, acc, acc + 15, fr(i), fr(i) + 3, 80 + 4 * (i >> 2), 83 + 4 * (i >> 2), acc, acc + 15))
+            for qb in (0, 1):
+                o = 4 * (2 * i + qb)
+                emit("%s v[%d:%d], %s, v[%d:%d], v[%d:%d]" % (mfma, o, o + 3, f4, 80 + 4 * qb, 83 + 4 * qb, o, o + 3))
         else:
-            k = i - 8
-            c = "0" if k == 0 else "v[64:79]"
-            emit("%s v[64:79], v[%d:%d], v[%d:%d], %s" % (mfma, fr(i), fr(i) + 3, 88 + 4 * k, 91 + 4 * k, c))
-        # the fragment seven MFMAs ahead
+            j = i - 8
+            ks, kb = j >> 1, j & 1
+            for qb in (0, 1):
+                sb = 64 + 4 * (2 * kb + qb)
+                qv = 88 + 4 * (4 * qb + ks)
+                emit("%s v[%d:%d], %s, v[%d:%d], %s" % (mfma, sb, sb + 3, f4, qv, qv + 3, "0" if ks == 0 else "v[%d:%d]" % (sb, sb + 3)))
         f = i + 7
         if f < 16:
             read_frag(blk, f)
         else:
             read_frag((blk + 1) & 3, f - 16)
         if dma and "dma" not in ablate:
-            # K wave-loads 0..3 in slots 0..3, V wave-loads in slots 4..7: rows are 256 bytes apart, so wave-load n lies 1024 bytes
-            # behind wave-load 0 in memory and in LDS alike, and the instruction's offset moves both addresses
             n = i & 3
-            ptr, lane = (40, 164 + n) if i < 4 else (42, 168)
+            ptr, lane = (40, 160 + n) if i < 4 else (42, 164)
             emit("global_load_lds_dwordx4 v%d, s[%d:%d] offset:%d" % (lane, ptr, ptr + 1, 1024 * n))
         if "valu" in ablate:
             pass
         elif i < 8:
             if i == 0:
-                emit("s_nop 3")             # the logits were written by the MFMA chain of the previous block
-            emit("v_fma_f32 v172, v%d, s52, v169" % (64 + 2 * i))
-            emit("v_fma_f32 v173, v%d, s52, v169" % (65 + 2 * i))
-            emit("v_exp_f32_e32 v%d, v172" % (176 + 2 * i))
-            emit("v_exp_f32_e32 v%d, v173" % (177 + 2 * i))
+                emit("s_nop 1")
+            for t in (2 * i, 2 * i + 1):
+                qb = (t >> 2) & 1
+                emit("v_fma_f32 v%d, v%d, s52, v%d" % (169 + (t & 1), 64 + t, 165 + qb))
+            for t in (2 * i, 2 * i + 1):
+                emit("v_exp_f32_e32 v%d, v%d" % (176 + t, 169 + (t & 1)))
         else:
             p = i - 8
-            emit("%s v%d, v%d, v%d" % (cvt, 80 + p, 176 + 2 * p, 177 + 2 * p))
-            emit("%s v170, %s, v%d" % (dot, ones, 80 + p))
+            qb, e2 = p >> 2, p & 3
+            t0 = 8 * (e2 >> 1) + 4 * qb + 2 * (e2 & 1)
+            emit("%s v%d, v%d, v%d" % (cvt, 80 + 4 * qb + e2, 176 + t0, 177 + t0))
+            emit("%s v%d, %s, v%d" % (dot, 167 + qb, ones, 80 + 4 * qb + e2))
 
     for blk in range(4):
-        is_b = (blk & 1) == 0               # odd units: tile loads; even units: tile barrier
-        kstage = (blk >> 1) & 1             # stage of the K tile this block loads; the V tile goes to the other one
+        is_b = (blk & 1) == 0
+        kstage = (blk >> 1) & 1
         emit("%sblk%d_%%=:" % (label, blk))
         del queue[:]
-        queue.extend(first7(blk))           # what the cold start, or the block before, has left outstanding
+        queue.extend(first7(blk))
         if is_b:
-            # the tile loads come four to a group (K in slots 0..3, V in slots 4..7); a group whose tile is not to be loaded (s57 /
-            # s58 count the odd units that still have a K / V tile to load) runs a copy of its slots without them
             for group in (0, 1):
                 left, ptr, tile, dst, stage = (57, 40, 46, 50, kstage) if group == 0 else (58, 42, 48, 51, kstage ^ 1)
                 none = "%snone%d_%d_%%=" % (label, blk, group)
@@ -171,38 +177,42 @@ def gen(kind, dma=True, ablate=()):
         emit("s_cbranch_scc1 %sfin%d_%%=" % (label, blk))
         if blk == 3:
             emit("s_branch %sblk0_%%=" % label)
-    # The run is through.  With s59 set, one more unit follows whose logits are masked first (the unit on the causal diagonal):
-    # element r of the unit goes to -inf (v174) where its key offset 8 (r / 4) + r % 4 lies beyond the lane's limit v171.
     for blk in range(4):
         emit("%sfin%d_%%=:" % (label, blk))
         emit("s_cmp_eq_u32 s59, 0")
         emit("s_cbranch_scc1 %sexit_%%=" % label)
         emit("s_mov_b32 s59, 0")
         emit("s_mov_b32 s53, 1")
-        emit("s_nop 7")                     # the last MFMA of the logit chain has to have written its registers
         emit("s_nop 7")
-        for r in range(16):
-            emit("v_cmp_gt_i32_e32 vcc, %d, v171" % (8 * (r >> 2) + (r & 3)))
-            emit("v_cndmask_b32_e32 v%d, v%d, v174, vcc" % (64 + r, 64 + r))
+        emit("s_nop 7")
+        for t in range(16):
+            kb, qb, r = t >> 3, (t >> 2) & 1, t & 3
+            emit("v_cmp_gt_i32_e32 vcc, %d, v%d" % (16 * kb + r, 171 + qb))
+            emit("v_cndmask_b32_e32 v%d, v%d, v173, vcc" % (64 + t, 64 + t))
         emit("s_branch %sblk%d_%%=" % (label, (blk + 1) & 3))
     emit("%sexit_%%=:" % label)
     emit("s_waitcnt lgkmcnt(0)")
     return out
 
 
-def main():
-    import sys
-    ablate = tuple(sys.argv[2].split(",")) if len(sys.argv) > 2 else ()
-    name = sys.argv[1] if len(sys.argv) > 1 else os.path.join(HERE, "attention_prefill_loop.inc")
+def write(name, ablate=()):
     with open(name, "w") as fh:
-        fh.write("// Generated by gen_prefill_loop.py (the steady-state loop of attn_prefill_kernel as gfx950 assembly); do not edit.\n")
+        fh.write("// Generated by gen_prefill_loop.py (the run of whole units of attn_prefill_kernel as gfx950 assembly); do not edit.\n")
         for kind in ("f16", "bf16"):
-            lines = gen(kind, True, ablate)
+            lines = gen(kind, ablate)
             fh.write("#define PREFILL_LOOP_%s \\\n" % kind.upper())
             for n, line in enumerate(lines):
                 sep = "\\n" if line.endswith(":") else "\\n\\t"
                 fh.write('    "%s%s"%s\n' % (line, sep, " \\" if n + 1 < len(lines) else ""))
             fh.write("// %d instructions\n" % sum(1 for x in lines if not x.endswith(":")))
+
+
+def main():
+    import sys
+    if len(sys.argv) > 1:
+        write(sys.argv[1], tuple(sys.argv[2].split(",")) if len(sys.argv) > 2 else ())
+    else:
+        write(os.path.join(HERE, "attention_prefill_loop.inc"))
 
 
 if __name__ == "__main__":
