@@ -261,8 +261,9 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     auto get4 = [&](const f32x16& v, int at) -> f32x4 { return f32x4{v[4 * at], v[4 * at + 1], v[4 * at + 2], v[4 * at + 3]}; };
     auto put4 = [&](f32x16& v, int at, const f32x4& x) { v[4 * at] = x[0]; v[4 * at + 1] = x[1]; v[4 * at + 2] = x[2]; v[4 * at + 3] = x[3]; };
     // a value of the four lanes (g = 0..3) that share a query: maximum / sum over them
-    auto max_over_g = [&](float v) -> float { v = fmaxf(v, __shfl_xor(v, 16, 64)); return max_with_partner32(v); };
-    auto sum_over_g = [&](float v) -> float { v += __shfl_xor(v, 16, 64); return sum_with_partner32(v); };
+    // (two lane-swap instructions of the vector pipe each, no trip through the LDS crossbar)
+    auto max_over_g = [&](float v) -> float { return max_with_partner32(max_with_partner16(v)); };
+    auto sum_over_g = [&](float v) -> float { return sum_with_partner32(sum_with_partner16(v)); };
 
     // ---- plain (not interleaved) forms of the three steps of a unit
     auto qk_plain = [&]() {                                    // S of the unit the K addresses point to

@@ -156,6 +156,18 @@ __device__ __forceinline__ void half_swap(float v, float& lo_half, float& hi_hal
 }
 __device__ __forceinline__ float max_with_partner32(float v) { float a, b; half_swap(v, a, b); return fmaxf(a, b); }
 __device__ __forceinline__ float sum_with_partner32(float v) { float a, b; half_swap(v, a, b); return a + b; }
+// The same between the lanes l and l ^ 16 (v_permlane16_swap: the odd 16-lane rows of one operand change places with the even rows
+// of the other, so with both operands v one result holds the even row's value of every row pair and the other the odd row's).
+__device__ __forceinline__ void row_swap(float v, float& even_row, float& odd_row)
+{
+    uint32_t u = as_u32(v);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    uint32_t a = r[0], b = r[1];
+    even_row = as_f32(a);
+    odd_row = as_f32(b);
+}
+__device__ __forceinline__ float max_with_partner16(float v) { float a, b; row_swap(v, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float sum_with_partner16(float v) { float a, b; row_swap(v, a, b); return a + b; }
 
 // One interleaved rotary pair: (xe, xo) -> (xe c - xo s, xe s + xo c).  One definition for the stand-alone kernels and for the
 // GEMM pass that rotates while it sums, so that both round alike (HipAttentionKernels.cs:958-989 is the reference form).
