@@ -83,7 +83,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 
     // Direct-to-LDS loads.  This wave's share of a tile: K wave-loads 4 w .. 4 w + 3 and the same of V, each 4 keys x 256 B; lane ->
     // (key = 4 * load + lane / 16, chunk position lane % 16).  LDS layout [key][256 B]: 16-byte chunk c of key k sits at position
-    // c ^ (k & 15) in a K tile (b128 fragment reads) and at c ^ ((k & 3) << 2) in a V tile (transposing reads).
+    // c ^ (k & 15) in a K tile (b128 fragment reads) and at c ^ ((k & 3) << 2) ^ ((k >> 2 & 1) << 1) in a V tile (transposing reads:
+    // a half-wave reads eight keys, 4 g .. 4 g + 7, 32 bytes each, and the position spreads them over all 64 banks).
     const int ld_key = lane >> 4, ld_pos = lane & 15;
     // Q, K, V and O are dense [batch, head, row, 128] arrays (the launcher checks): row r of (batch, head) pair j is row
     // j * rows + r of the array, 256 bytes a row in the 16-bit types.
@@ -125,7 +126,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
 #pragma unroll
-            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+            for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off ^ (uint32_t)((i & 1) << 5), dst + i * 1024);
         } else {
             int ln = lane;
             asm volatile("" : "+v"(ln));
@@ -133,7 +134,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
             for (int i = 0; i < 4; i++) {
                 const int key = 4 * (wave_s * 4 + i) + (ln >> 4);
                 const int gkey = min(tile * BC + key, Sk - 1);
-                attn_dma16(V + (long long)gkey * 128 + ((ln & 15) ^ ((key & 3) << 2)) * 8, dst + i * 1024);
+                attn_dma16(V + (long long)gkey * 128 + ((ln & 15) ^ ((key & 3) << 2) ^ (((key >> 2) & 1) << 1)) * 8, dst + i * 1024);
             }
         }
     };
@@ -208,8 +209,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     // XOR (8 KB when leaving an even unit, 24 KB when leaving an odd one).
     //   K fragment (block kb, k-step ks): key 16 kb + c, chunk (4 ks + g) ^ c; the k-steps differ by an XOR of bits 6-7, kb by 4 KB
     //   V^T fragment of d-block db: two transposing reads 16 keys apart; in the 16-lane group g lane c addresses key 4 g + c / 4 and
-    //   the 8 bytes at head-dim 4 (c % 4) of the block; d-block pairs differ by an XOR of bits 6-7, the odd block by 32 bytes
-    uint32_t k_ad[4], v_ad[4];
+    //   the 8 bytes at head-dim 4 (c % 4) of the block; the d-blocks differ by an XOR of bits 5-7
+    uint32_t k_ad[4], v_ad[8];
     int k_unit = 0, v_unit = 0;
     {
         // (from an opaque copy of the lane index, so that these are formed here, per pass, rather than kept across the passes)
@@ -217,11 +218,11 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         asm volatile("" : "+v"(ln));
         const int cp = ln & 15, gp = ln >> 4;
         const uint32_t k_lane = cp * 256 + ((gp ^ cp) << 4);
-        const uint32_t v_lane = (4 * gp + (cp >> 2)) * 256 + ((((cp & 3) >> 1) ^ (((cp >> 2) & 3) << 2)) << 4) + (cp & 1) * 8;
+        const uint32_t v_lane = (4 * gp + (cp >> 2)) * 256 + ((((cp & 3) >> 1) ^ (((cp >> 2) & 3) << 2) ^ ((gp & 1) << 1)) << 4) + (cp & 1) * 8;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) k_ad[ks] = (lds0 + k_lane) ^ (uint32_t)(ks << 6);
 #pragma unroll
-        for (int j = 0; j < 4; j++) v_ad[j] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(j << 6);
+        for (int j = 0; j < 8; j++) v_ad[j] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(j << 5);
     }
     auto next_k_unit = [&]() {
         const uint32_t x = (k_unit & 1) ? 24576u : 8192u;
@@ -232,14 +233,14 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
     auto next_v_unit = [&]() {
         const uint32_t x = (v_unit & 1) ? 24576u : 8192u;
 #pragma unroll
-        for (int i = 0; i < 4; i++) v_ad[i] ^= x;
+        for (int i = 0; i < 8; i++) v_ad[i] ^= x;
         v_unit++;
     };
     auto k_frag = [&](int kb, int ks) -> u32x4 {
         return *(const __attribute__((address_space(3))) u32x4*)(k_ad[ks] + kb * 4096);
     };
     auto v_frag = [&](int db) -> u32x4 {
-        const uint32_t ad = v_ad[db >> 1] + (db & 1) * 32;
+        const uint32_t ad = v_ad[db];
         u32x2 w0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)ad));
         u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 16 * 256)));
         return u32x4{w0[0], w0[1], w1[0], w1[1]};
@@ -361,9 +362,10 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         // read addresses of unit 0 (the K addresses stand at unit u + 1, the V addresses at unit u - 1)
         const uint32_t koff = (uint32_t)((u + 1) & 3) << 13, voff = (uint32_t)((u - 1) & 3) << 13;
         const u32x4 kad = {k_ad[0] ^ koff, k_ad[1] ^ koff, k_ad[2] ^ koff, k_ad[3] ^ koff};
-        const u32x4 vad = {v_ad[0] ^ voff, v_ad[1] ^ voff, v_ad[2] ^ voff, v_ad[3] ^ voff};
+        const u32x4 vad0 = {v_ad[0] ^ voff, v_ad[1] ^ voff, v_ad[2] ^ voff, v_ad[3] ^ voff};
+        const u32x4 vad1 = {v_ad[4] ^ voff, v_ad[5] ^ voff, v_ad[6] ^ voff, v_ad[7] ^ voff};
         const u32x4 klo = {k_lane_off, k_lane_off ^ 64u, k_lane_off ^ 128u, k_lane_off ^ 192u};
-        const uint32_t vlo = v_lane_off;
+        const uint32_t vlo = v_lane_off, vlo_odd = v_lane_off ^ 32u;
         const float negm0 = (m_ref[0] == -INFINITY) ? -0.0f : -m_ref[0], negm1 = (m_ref[1] == -INFINITY) ? -0.0f : -m_ref[1];
         float ps0 = 0.0f, ps1 = 0.0f;
         const int tl = u >> 1;
@@ -385,8 +387,8 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
 #define PREFILL_LOOP_OPERANDS \
             : "+{v[0:15]}"(oacc[0]), "+{v[16:31]}"(oacc[1]), "+{v[32:47]}"(oacc[2]), "+{v[48:63]}"(oacc[3]), "+{v[64:79]}"(sacc), \
               "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v167}"(ps0), "+{v168}"(ps1), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft), "+{s59}"(mask_follows) \
-            : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad), "{v[156:159]}"(vad), \
-              "{v[160:163]}"(klo), "{v164}"(vlo), "{v165}"(negm0), "{v166}"(negm1), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), \
+            : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad), "{v[192:195]}"(vad0), "{v[196:199]}"(vad1), \
+              "{v[160:163]}"(klo), "{v164}"(vlo), "{v174}"(vlo_odd), "{v165}"(negm0), "{v166}"(negm1), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), \
               "{v171}"(mask_rel0), "{v172}"(mask_rel1), "{v173}"(ninf) \
             : "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", \
               "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \

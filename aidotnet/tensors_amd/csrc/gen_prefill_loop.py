@@ -33,8 +33,8 @@ def gen(kind, ablate=()):
 
     Registers (fixed; the kernel binds its variables to them at the asm statement): v[0:63] O (block (db, qb) at 4 (2 db + qb)),
     v[64:79] logits (block (kb, qb) at 64 + 4 (2 kb + qb)), v[80:87] P (qb 0, qb 1), v[88:119] Q (block (qb, ks) at
-    88 + 4 (4 qb + ks)), v[120:151] fragment ring, v[152:155] K read addresses per ks (kb by an offset), v[156:159] V read
-    addresses per pair of d-blocks, v[160:163] lane offsets of the four K wave-loads, v164 of the V wave-loads, v165 v166 minus the
+    88 + 4 (4 qb + ks)), v[120:151] fragment ring, v[152:155] K read addresses per ks (kb by an offset), v[192:199] V read
+    addresses per d-block, v[160:163] lane offsets of the four K wave-loads, v164 / v174 of the even / odd V wave-loads, v165 v166 minus the
     exponent reference of query block 0 / 1, v167 v168 their running row sums, v169 v170 scratch, v171 v172 the lane's key limit
     inside a masked unit per query block, v173 minus infinity, v[176:191] exponentials.
     s[40:41] / s[42:43] source of this wave's next K / V tile load, s[46:47] s[48:49] one K / V tile in bytes, s50 s51 LDS
@@ -56,9 +56,9 @@ def gen(kind, ablate=()):
         if "lds" in ablate:
             return
         if f < 8:
-            voff = blk * 8192 + (f & 1) * 32
-            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b, b + 1, 156 + (f >> 1), voff))
-            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b + 2, b + 3, 156 + (f >> 1), voff + 4096))
+            voff = blk * 8192
+            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b, b + 1, 192 + f, voff))
+            emit("ds_read_b64_tr_b16 v[%d:%d], v%d offset:%d" % (b + 2, b + 3, 192 + f, voff + 4096))
             queue.append((blk, f)); queue.append((blk, f))
         else:
             j = f - 8
@@ -119,7 +119,7 @@ def gen(kind, ablate=()):
             read_frag((blk + 1) & 3, f - 16)
         if dma and "dma" not in ablate:
             n = i & 3
-            ptr, lane = (40, 160 + n) if i < 4 else (42, 164)
+            ptr, lane = (40, 160 + n) if i < 4 else (42, 174 if n & 1 else 164)
             emit("global_load_lds_dwordx4 v%d, s[%d:%d] offset:%d" % (lane, ptr, ptr + 1, 1024 * n))
         if "valu" in ablate:
             pass
