@@ -30,22 +30,27 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # same counter reads for a 1 GiB device copy; the runs and factors are in profiles/ (one summary per kernel).  None = not
 # measured yet.
 TRAFFIC_BYTES = {
-    # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes)
-    "gemm_f16_8192": int((787044 * 2.0 + 131352) * 1024),
-    "gemm_bf16_8192": int((786877 * 2.0 + 131584) * 1024),
-    "gemm_f16_proj": int((17124 * 2.0 + 24579) * 1024),
-    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49178) * 1024),
-    "gemm_f32_proj": int((43100 * 2.0 + 49152) * 1024),
+    # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes), last three dispatches of each kernel
+    "gemm_f16_8192": int((787084 * 2.0 + 131176) * 1024),
+    "gemm_bf16_8192": int((787028 * 2.0 + 131270) * 1024),
+    "gemm_f16_proj": int((17114 * 2.0 + 24582) * 1024),
+    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49168) * 1024),
+    "gemm_f32_proj": int((43085 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
     "decode_bf16": int((1048770 * 2.0 + 512) * 1024),
-    "attn_f16_prefill": int((139311 * 2.0 + 132113) * 1024),
-    "attn_bf16_prefill": int((139768 * 2.0 + 132113) * 1024),
-    "attn_f32_prefill": int((22644 * 2.0 + 12480) * 1024),
+    "attn_f16_prefill": int((132442 * 2.0 + 132112) * 1024),
+    "attn_bf16_prefill": int((132484 * 2.0 + 132122) * 1024),
+    "attn_f32_prefill": int((22643 * 2.0 + 12480) * 1024),
+    # two launches each: the skinny kernel, then the pass that sums its K ranges (the 4096-wide summing pass: 8 ranges of 32 x 4096 fp32
+    # partials read back, 2073 KiB on the counter, 256 KiB written)
     "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
-    # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass)
+    "gemm_bf16_decode_qkv": int(((50203 + 3863) * 2.0 + 7680 + 768) * 1024),
+    "gemm_bf16_decode_qkv_rope": int(((50203 + 3864) * 2.0 + 7680 + 768) * 1024),
+    # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass; the summing pass of the 16-row product
+    # reads its 16 ranges of 16 x 4096 fp32 partials back: 4 MiB, 2049 KiB on the counter)
     "decode_bf16_gqa": int(((262417 + 1108) * 2.0 + 1040 + 512) * 1024),
     "decode_f32_gqa": int(((525392 + 1108) * 2.0 + 2176 + 512) * 1024),
-    "gemm_f32_m16": int(((33827 + 1026) * 2.0 + 2048 + 256) * 1024),
+    "gemm_f32_m16": int(((33819 + 2049) * 2.0 + 4096 + 256) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
@@ -175,6 +180,33 @@ def _events_time(torch, fn, steps, warmup, min_warm_ms=MIN_WARM_MS):
     return ms, wall_ms, stats
 
 
+def _summarize_profile(directory, last):
+    """Reads what rocprofv3 wrote under `directory` (CSV output) and prints, per kernel, the figures of its LAST `last` dispatches
+    only: the timed region of a configuration is what it launches last, its warm-up launches come before.  Kernel-trace files give
+    the duration (us), counter-collection files the counter values (per dispatch).  Needs no GPU."""
+    import collections
+    import csv
+    import glob
+    for f in sorted(glob.glob(os.path.join(directory, "**", "*kernel_trace.csv"), recursive=True)):
+        per = collections.defaultdict(list)
+        for row in csv.DictReader(open(f)):
+            per[row["Kernel_Name"]].append((int(row["Start_Timestamp"]), int(row["End_Timestamp"])))
+        print("# %s: duration in us over the last %d dispatches of each kernel" % (os.path.relpath(f, directory), last))
+        for name, v in sorted(per.items(), key=lambda kv: -sum(e - s for s, e in kv[1])):
+            v.sort()
+            tail = [(e - s) / 1e3 for s, e in v[-last:]]
+            print("%-130s calls=%d last=%d avg=%.2f min=%.2f max=%.2f (all calls avg %.2f)" % (
+                name[:130], len(v), len(tail), sum(tail) / len(tail), min(tail), max(tail), sum((e - s) / 1e3 for s, e in v) / len(v)))
+    for f in sorted(glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True)):
+        per = collections.defaultdict(lambda: collections.defaultdict(list))
+        for row in csv.DictReader(open(f)):
+            per[row["Kernel_Name"]][row["Counter_Name"]].append(float(row["Counter_Value"]))
+        print("# %s: counter value per dispatch, mean over the last %d dispatches of each kernel" % (os.path.relpath(f, directory), last))
+        for name, cs in per.items():
+            print("%-130s %s" % (name[:130], "  ".join("%s=%.6g (n=%d)" % (c, sum(v[-last:]) / len(v[-last:]), len(v)) for c, v in sorted(cs.items()))))
+    return 0
+
+
 def _roof_flops(kind, flops, ms, traffic=None):
     ach = flops / (ms * 1e-3) / 1e12
     return {"bound": "mfma", "achieved": round(ach, 3), "peak": PEAK_TFLOPS[kind], "unit": "TFLOP/s",
@@ -204,7 +236,13 @@ def main() -> int:
     ap.add_argument("--clock-probe", type=float, default=0.0, metavar="SECONDS",
                     help="NOT the metric: keep the headline GEMM (then the bf16 causal prefill) queued for SECONDS each and sample the "
                          "engine clock the driver reports meanwhile; prints one JSON line with the median clock and the rate")
+    ap.add_argument("--summarize-profile", default=None, metavar="DIR",
+                    help="NOT a run: print per-kernel durations and counter values from the CSV files rocprofv3 wrote under DIR, over the "
+                         "last --last dispatches of each kernel (the timed region; warm-up launches come first)")
+    ap.add_argument("--last", type=int, default=20, help="dispatches per kernel that --summarize-profile looks at")
     args = ap.parse_args()
+    if args.summarize_profile:
+        return _summarize_profile(args.summarize_profile, max(1, args.last))
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (the path shards without "
               "communication over (batch, head) and over row slabs of C)" % args.gpus, file=sys.stderr)
