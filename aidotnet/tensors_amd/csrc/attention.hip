@@ -478,13 +478,18 @@ __global__ __launch_bounds__(256, MINB) void attn_fwd_kernel(const AttnArgs a)
 #define ATTN_HEAD_GROUP 4
 // Depth of the register ring that prefetches MFMA operand fragments from LDS inside a tile; must divide 8.
 #define AIDN_ATTN_RING 4
-template <typename T, typename OutT>
-__global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
+template <typename T, typename OutT, int D = 128>
+__global__ __launch_bounds__(256, D == 128 ? 2 : 1) void attn_fwd_dl_kernel(const AttnArgs a)
 {
     typedef uint16_t raw_t;
-    constexpr int D = 128, BC = 64, BR = 128;
-    constexpr int KBYTES = BC * 256, VBYTES = BC * 256;
+    static_assert(D == 128 || D == 256, "head dimension 128 (two workgroups per CU) or 256 (one)");
+    constexpr int BC = 64, BR = 128;
+    constexpr int ROWB = 2 * D;                     // bytes of a K or V row in a tile
+    constexpr int KBYTES = BC * ROWB, VBYTES = BC * ROWB;
     constexpr int DSTEPS = D / 16, DT = D / 32;
+    constexpr int CH = ROWB / 16;                   // 16-byte chunks per row
+    constexpr int KPL = 1024 / ROWB;                // keys per wave-load (64 lanes x 16 bytes)
+    constexpr int NL = 16 / KPL;                    // wave-loads per wave and tile (a wave loads 16 keys of K and 16 of V)
 
     extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
 
@@ -562,53 +567,56 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
         else { long long nt = lastkey / BC + 1; if (nt < ntiles) ntiles = (int)nt; }
     }
 
-    // LDS: K ring [2][KBYTES] then V ring [2][VBYTES].  This wave's DMA per tile: K wave-loads 4w..4w+3 and V
-    // wave-loads 4w..4w+3, each 4 keys x 256 B; lane -> (key = 4 * load + lane / 16, chunk position = lane % 16).
+    // LDS: K ring [2][KBYTES] then V ring [2][VBYTES].  This wave's DMA per tile: NL wave-loads of K and NL of V, each KPL keys
+    // x ROWB bytes (4 x 256 at head dimension 128, 2 x 512 at 256); lane -> (key = KPL * load + lane / CH, chunk position = lane % CH).
     // For a tile that lies fully inside the sequence the source address is a scalar base (tile, wave, load) plus
     // a per-lane byte offset fixed for the whole kernel, so issuing a load costs no vector arithmetic.
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
     const int wave_s = __builtin_amdgcn_readfirstlane(wave);
-    const int ld_key = lane >> 4, ld_pos = lane & 15;
+    const int ld_key = lane / CH, ld_pos = lane % CH;
     const long long k_row_bytes = a.ks[2] * 2, v_row_bytes = a.vs[2] * 2;
-    uint32_t k_lane_off[4];
+    // (the swizzle of a lane's chunk depends on its key inside the wave's 16: load i, lane key ld_key -> key KPL i + ld_key; for V only
+    // on the key's two low bits, which at 4 keys per load are ld_key for every load and at 2 keys per load alternate with the load)
+    uint32_t k_lane_off[NL], v_lane_off[2];
 #pragma unroll
-    for (int i = 0; i < 4; i++) k_lane_off[i] = (uint32_t)(ld_key * k_row_bytes) + ((ld_pos ^ (4 * i + ld_key)) << 4);
-    const uint32_t v_lane_off = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (ld_key << 2)) << 4);
+    for (int i = 0; i < NL; i++) k_lane_off[i] = (uint32_t)(ld_key * k_row_bytes) + ((ld_pos ^ (KPL * i + ld_key)) << 4);
+#pragma unroll
+    for (int i = 0; i < 2; i++) v_lane_off[i] = (uint32_t)(ld_key * v_row_bytes) + ((ld_pos ^ (((KPL * i + ld_key) & 3) << 2)) << 4);
     auto issue_k = [&](int tile) {
-        const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * 4096;
+        const uint32_t dst = lds0 + (tile & 1) * KBYTES + wave_s * (16 * ROWB);
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)K + (long long)(tile * BC + 16 * wave_s) * k_row_bytes;
             if (a.stream) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) attn_dma16_base_stream(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+                for (int i = 0; i < NL; i++) attn_dma16_base_stream(src + KPL * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
             } else {
 #pragma unroll
-                for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
+                for (int i = 0; i < NL; i++) attn_dma16_base(src + KPL * i * k_row_bytes, k_lane_off[i], dst + i * 1024);
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                int key = 4 * (wave * 4 + i) + ld_key;               // key inside the tile
+            for (int i = 0; i < NL; i++) {
+                int key = KPL * (wave * NL + i) + ld_key;          // key inside the tile
                 int gkey = min(tile * BC + key, Sk - 1);           // clamp: rows past the end are masked later
                 attn_dma16(K + (long long)gkey * a.ks[2] + (ld_pos ^ (key & 15)) * 8, dst + i * 1024);
             }
         }
     };
     auto issue_v = [&](int tile) {
-        const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * 4096;
+        const uint32_t dst = lds0 + 2 * KBYTES + (tile & 1) * VBYTES + wave_s * (16 * ROWB);
         if (tile * BC + BC <= Sk) {
             const unsigned char* src = (const unsigned char*)V + (long long)(tile * BC + 16 * wave_s) * v_row_bytes;
             if (a.stream) {
 #pragma unroll
-                for (int i = 0; i < 4; i++) attn_dma16_base_stream(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+                for (int i = 0; i < NL; i++) attn_dma16_base_stream(src + KPL * i * v_row_bytes, v_lane_off[i & 1], dst + i * 1024);
             } else {
 #pragma unroll
-                for (int i = 0; i < 4; i++) attn_dma16_base(src + 4 * i * v_row_bytes, v_lane_off, dst + i * 1024);
+                for (int i = 0; i < NL; i++) attn_dma16_base(src + KPL * i * v_row_bytes, v_lane_off[i & 1], dst + i * 1024);
             }
         } else {
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                int key = 4 * (wave * 4 + i) + ld_key;
+            for (int i = 0; i < NL; i++) {
+                int key = KPL * (wave * NL + i) + ld_key;
                 int gkey = min(tile * BC + key, Sk - 1);
                 attn_dma16(V + (long long)gkey * a.vs[2] + (ld_pos ^ ((key & 3) << 2)) * 8, dst + i * 1024);
             }
@@ -637,8 +645,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     // V^T (transposing reads): in a 16-lane group lane j addresses key (base + j / 4), 8 bytes at head-dim
     // 4 (j % 4) of the 16-wide block; chunk position (c + 4 dt) ^ ((key & 3) << 2).
     const int jl = lane & 15;
-    const uint32_t k_lane = l32 * 256 + ((h ^ (l32 & 15)) << 4);
-    const uint32_t v_lane = (4 * h + (jl >> 2)) * 256 + ((16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3) * 16 + (jl & 1) * 8
+    const uint32_t k_lane = l32 * ROWB + ((h ^ (l32 & 15)) << 4);
+    const uint32_t v_lane = (4 * h + (jl >> 2)) * ROWB + ((16 * ((lane >> 4) & 1) + 4 * (jl & 3)) >> 3) * 16 + (jl & 1) * 8
                           + ((jl >> 2) << 6);
 
     // last key a query may see (sequence end and causal diagonal folded into one 32-bit bound); klim carries the
@@ -680,11 +688,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     // Per tile (64 keys = two 32-key sub-tiles) the work of a wave is pipelined so that the exponentials sit in
     // the shadow of the matrix pipe:   S0 = QK(sub 0) | S1 = QK(sub 1) with exp(S0) | PV(sub 0) with exp(S1) | PV(sub 1)
     // invariant per-lane read addresses; ring stage, sub-tile and key block enter as immediate offsets
-    uint32_t k_ad[DSTEPS], v_ad[DT];
+    // (the swizzle occupies address bits 4-7: a step or d-block index beyond them -- bit 8, head dimension 256 -- is a plain offset)
+    uint32_t k_ad[8], v_ad[4];
 #pragma unroll
-    for (int s = 0; s < DSTEPS; s++) k_ad[s] = (lds0 + k_lane) ^ (uint32_t)(s << 5);
+    for (int s = 0; s < 8; s++) k_ad[s] = (lds0 + k_lane) ^ (uint32_t)(s << 5);
 #pragma unroll
-    for (int i = 0; i < DT; i++) v_ad[i] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(i << 6);
+    for (int i = 0; i < 4; i++) v_ad[i] = (lds0 + 2 * KBYTES + v_lane) ^ (uint32_t)(i << 6);
 
     auto tile_body = [&](const int j, auto stage_c) {
         constexpr int stage = decltype(stage_c)::value;
@@ -712,12 +721,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             // Fragment addresses: the swizzle is an XOR on address bits that only the lane's chunk index occupies,
             // so one base per tile and lane serves every step (XOR with a constant, then an immediate offset).
             auto k_frag = [&](int kt, int s) -> u32x4 {
-                return *(const __attribute__((address_space(3))) u32x4*)(k_ad[s] + stage * KBYTES + kt * 32 * 256);
+                return *(const __attribute__((address_space(3))) u32x4*)(k_ad[s & 7] + (s >> 3) * 256 + stage * KBYTES + kt * 32 * ROWB);
             };
-            auto v_frag8 = [&](int kt, int s) -> u32x4 {          // s = 4 * (16-key half) + head-dim block
-                const uint32_t ad = v_ad[s & 3] + stage * VBYTES + (32 * kt + 16 * (s >> 2)) * 256;
+            auto v_frag8 = [&](int kt, int s) -> u32x4 {          // s = DT * (16-key half) + head-dim block
+                const uint32_t ad = v_ad[(s % DT) & 3] + ((s % DT) >> 2) * 256 + stage * VBYTES + (32 * kt + 16 * (s / DT)) * ROWB;
                 u32x2 w0 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)ad));
-                u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 8 * 256)));
+                u32x2 w1 = __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4a*)(ad + 8 * ROWB)));
                 return u32x4{w0[0], w0[1], w1[0], w1[1]};
             };
 
@@ -728,7 +737,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
 #pragma unroll
             for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
             constexpr int R = AIDN_ATTN_RING;
-            static_assert(8 % R == 0, "the fragment ring is indexed s % R over 8 steps");
+            static_assert(DSTEPS % R == 0 && DSTEPS == 2 * DT, "the fragment ring is indexed s % R over DSTEPS steps in every phase");
+            constexpr int EV = DSTEPS / 8;          // steps per pair of exponentials (eight pairs per 32-key sub-tile)
             u32x4 fr[R];
 #pragma unroll
             for (int s = 0; s < R; s++) fr[s] = k_frag(0, s);
@@ -738,14 +748,14 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             if (spread) {
                 const unsigned char* ksrc = (const unsigned char*)K + (long long)((j + 1) * BC + 16 * wave_s) * k_row_bytes;
                 const unsigned char* vsrc = (const unsigned char*)V + (long long)((j + 1) * BC + 16 * wave_s) * v_row_bytes;
-                const uint32_t kdst = lds0 + (stage ^ 1) * KBYTES + wave_s * 4096;
-                const uint32_t vdst = lds0 + 2 * KBYTES + (stage ^ 1) * VBYTES + wave_s * 4096;
+                const uint32_t kdst = lds0 + (stage ^ 1) * KBYTES + wave_s * (16 * ROWB);
+                const uint32_t vdst = lds0 + 2 * KBYTES + (stage ^ 1) * VBYTES + wave_s * (16 * ROWB);
 #pragma unroll
                 for (int s = 0; s < DSTEPS; s++) {
                     Mma32<T>::run(s0, fr[s % R], qf[s]);
                     fr[s % R] = s + R < DSTEPS ? k_frag(0, s + R) : k_frag(1, s + R - DSTEPS);
-                    if (s < 4) attn_dma16_base(ksrc + 4 * s * k_row_bytes, k_lane_off[s], kdst + s * 1024);
-                    else attn_dma16_base(vsrc + 4 * (s - 4) * v_row_bytes, v_lane_off, vdst + (s - 4) * 1024);
+                    if (s < NL) attn_dma16_base(ksrc + KPL * s * k_row_bytes, k_lane_off[s], kdst + s * 1024);
+                    else attn_dma16_base(vsrc + KPL * (s - NL) * v_row_bytes, v_lane_off[(s - NL) & 1], vdst + (s - NL) * 1024);
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
@@ -768,10 +778,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             for (int s = 0; s < DSTEPS; s++) {
                 Mma32<T>::run(s1, fr[s % R], qf[s]);
                 fr[s % R] = s + R < DSTEPS ? k_frag(1, s + R) : v_frag8(0, s + R - DSTEPS);
-                uint32_t pk;
-                exp_pair(s0[2 * s], s0[2 * s + 1], m_use, pk, psum);
-                asm volatile("" : "+v"(pk), "+v"(psum));       // keeps the exponentials here, between the MFMAs
-                p0f[s >> 2][s & 3] = pk;
+                if (s % EV == 0) {
+                    const int e = s / EV;
+                    uint32_t pk;
+                    exp_pair(s0[2 * e], s0[2 * e + 1], m_use, pk, psum);
+                    asm volatile("" : "+v"(pk), "+v"(psum));       // keeps the exponentials here, between the MFMAs
+                    p0f[e >> 2][e & 3] = pk;
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             if (need_mask) mask_sub(1, s1);
@@ -779,13 +792,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             // ---- O^T += V[0:32]^T P0^T interleaved with P1 = exp(S1) against the standing reference
             float psum1 = 0.0f;
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                Mma32<T>::run(oacc[s & 3], fr[s % R], p0f[s >> 2]);
-                fr[s % R] = s + R < 8 ? v_frag8(0, s + R) : v_frag8(1, s + R - 8);
-                uint32_t pk;
-                exp_pair(s1[2 * s], s1[2 * s + 1], m_use, pk, psum1);
-                asm volatile("" : "+v"(pk), "+v"(psum1));
-                p1f[s >> 2][s & 3] = pk;
+            for (int s = 0; s < 2 * DT; s++) {
+                Mma32<T>::run(oacc[s % DT], fr[s % R], p0f[s / DT]);
+                fr[s % R] = s + R < 2 * DT ? v_frag8(0, s + R) : v_frag8(1, s + R - 2 * DT);
+                if (s % EV == 0) {
+                    const int e = s / EV;
+                    uint32_t pk;
+                    exp_pair(s1[2 * e], s1[2 * e + 1], m_use, pk, psum1);
+                    asm volatile("" : "+v"(pk), "+v"(psum1));
+                    p1f[e >> 2][e & 3] = pk;
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             l_run += psum;
@@ -808,9 +824,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
             // ---- O^T += V[32:64]^T P1^T
             __builtin_amdgcn_s_setprio(2);
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                Mma32<T>::run(oacc[s & 3], fr[s % R], p1f[s >> 2]);
-                if (s + R < 8) fr[s % R] = v_frag8(1, s + R);
+            for (int s = 0; s < 2 * DT; s++) {
+                Mma32<T>::run(oacc[s % DT], fr[s % R], p1f[s / DT]);
+                if (s + R < 2 * DT) fr[s % R] = v_frag8(1, s + R);
             }
             __builtin_amdgcn_s_setprio(0);
         }
@@ -827,7 +843,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     if (a.part) {
         // grouped decode over several splits: query row qi is head hd * Sq + qi of the caller; unnormalised partial for the merge
         if (qi < a.Sq) {
-            float* __restrict__ P = a.part + (((long long)bh * a.Sq + qi) * a.nsplit + split) * 130;
+            float* __restrict__ P = a.part + (((long long)bh * a.Sq + qi) * a.nsplit + split) * (D + 2);
             if (h == 0) { P[0] = m_ref; P[1] = l_tot; }
 #pragma unroll
             for (int i = 0; i < DT; i++)
@@ -841,26 +857,31 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_dl_kernel(const AttnArgs a)
     } else
     if (Elem<OutT>::BYTES == 4 && a.vec_out && a.stage_out) {
         // fp32 O through LDS: the lane holds 16-byte pieces of ONE row (64 rows per store instruction, each a partial line);
-        // staged per wave as [32 rows][512 B] (chunk c of row r at position c ^ r, conflict-free both ways) and written back
-        // as whole 512-byte rows, two per instruction.  The tile memory is idle here: every wave left the last tile at the
-        // barrier that ends the loop; the barrier below keeps the next pass's loads off the staged rows.
-        unsigned char* stg = smem + wave * 16384;
+        // staged per wave as [32 rows][4 D bytes] (chunk c of row r at position c ^ r, conflict-free both ways) and written back
+        // as whole rows, 1024 bytes per instruction (two rows at head dimension 128, one at 256).  The tile memory is idle here:
+        // every wave left the last tile at the barrier that ends the loop; the barrier below keeps the next pass's loads off the
+        // staged rows.
+        constexpr int OROWB = 4 * D, OCH = OROWB / 16, RPI = 64 / OCH;
+        unsigned char* stg = smem + wave * (32 * OROWB);
 #pragma unroll
         for (int i = 0; i < DT; i++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int c = 8 * i + 2 * g + h;
-                *(f32x4*)(stg + l32 * 512 + ((c ^ l32) << 4)) =
+                *(f32x4*)(stg + l32 * OROWB + ((c ^ l32) << 4)) =
                     f32x4{oacc[i][4 * g + 0] * inv, oacc[i][4 * g + 1] * inv, oacc[i][4 * g + 2] * inv, oacc[i][4 * g + 3] * inv};
             }
         if (a.lse && h == 0 && qi < a.Sq)
             a.lse[(long long)bh * a.Sq + qi] = l_tot > 0.0f ? (m_ref + __builtin_amdgcn_logf(l_tot)) * LN2 : -INFINITY;
-        const int c = lane & 31;
+        // (the lane index is taken through an opaque copy: the row addresses below are then formed here, not ahead of the tile loop)
+        int ln = lane;
+        asm volatile("" : "+v"(ln));
+        const int c = ln % OCH;
 #pragma unroll
-        for (int q = 0; q < 16; q++) {
-            const int r = 2 * q + (lane >> 5);
+        for (int q = 0; q < 32 / RPI; q++) {
+            const int r = RPI * q + ln / OCH;
             const int row = q0 + wave * 32 + r;
-            const f32x4 v = *(const f32x4*)(stg + r * 512 + ((c ^ r) << 4));
+            const f32x4 v = *(const f32x4*)(stg + r * OROWB + ((c ^ r) << 4));
             f32x4* dst = (f32x4*)((float*)a.o + b * a.os[0] + hd * a.os[1] + (long long)row * a.os[2] + c * 4);
             // non-temporal: O is written once and would otherwise displace K and V tiles that other workgroups re-read
             // (alternated in one process: causal B4 H32 S2048 835 -> 879 TFLOP/s, unmasked 973 -> 999, never slower)
@@ -939,15 +960,16 @@ __global__ __launch_bounds__(128) void attn_split_merge_kernel(const AttnArgs a)
     if (t == 0 && a.lse) a.lse[row] = L > 0.0f ? (M + __builtin_amdgcn_logf(L)) * LN2 : -INFINITY;
 }
 
-template <typename T, typename OutT>
+template <typename T, typename OutT, int D = 128>
 static hipError_t launch_attn_dl(AttnArgs a, hipStream_t stream)
 {
-    auto kern = attn_fwd_dl_kernel<T, OutT>;
-    constexpr int smem = 2 * (64 * 256 + 64 * 256);
+    auto kern = attn_fwd_dl_kernel<T, OutT, D>;
+    constexpr int smem = 2 * (64 * 2 * D + 64 * 2 * D);      // K and V tiles, two stages each (64 KB; 128 KB at head dimension 256)
     static unsigned long long attr_done = 0;
     if (hipError_t e = ensure_dynamic_smem((const void*)kern, smem, &attr_done)) return e;
     a.qtiles = (a.Sq + 127) / 128;
     a.stage_out = 1;
+    if (D != 128 && a.nsplit > 1) return hipErrorInvalidValue;      // (the merge pass of the key ranges is written for 128)
     if (a.nsplit > 1) {
         // few query tiles over a long key sequence: every tile's keys are cut into ranges that run side by side; a merge pass follows
         a.paired = 0;
@@ -1195,6 +1217,12 @@ hipError_t attn_fwd(hipStream_t stream, int kind, const AttnParams& p)
         else if (p.D <= 64) err = full ? (p.D <= 32 ? launch_attn<float, float, 32, 64, true, 2>(a, stream) : launch_attn<float, float, 64, 64, true, 2>(a, stream))
                                   : (p.D <= 32 ? launch_attn<float, float, 32, 64, false, 2>(a, stream) : launch_attn<float, float, 64, 64, false, 2>(a, stream));
         else err = dispatch_attn_d<float, float, 32>(a, full, stream);
+    }
+    else if (p.D == 256 && !full && a.vec_in && !p.block_table && g_attn_allow_dl && rows32 && p.scale > 0.0f && p.allow_fast_path != 2) {
+        // head dimension 256, plain / causal, aligned rows: the phase-structured kernel at that width (64-key tiles of 512-byte rows,
+        // one workgroup per CU); allow_fast_path 2 (test hook) pins the older form below
+        if (kind == 1) err = p.out16 ? launch_attn_dl<f16_t, f16_t, 256>(a, stream) : launch_attn_dl<f16_t, float, 256>(a, stream);
+        else err = p.out16 ? launch_attn_dl<bf16_t, bf16_t, 256>(a, stream) : launch_attn_dl<bf16_t, float, 256>(a, stream);
     }
     else if (p.D == 256 && !full && a.vec_in && !p.block_table && g_attn_allow_dl) {
         // head dimension 256, plain / causal, aligned contiguous K/V: the direct-to-LDS form on 32-key tiles (Q streamed)

@@ -474,6 +474,52 @@ def test_fp32_d64_direct_load_form_matches_oracle_and_general_form(be, eng, D, B
     assert np.array_equal(outs[True][0], outs[False][0]) and np.array_equal(outs[True][1], outs[False][1])
 
 
+# --------------------------------------------------------------- head dimension 256, 16-bit: the phase-structured kernel at that width
+D256_CASES = [
+    (1, 1, 1, 1, 1, False, 0),
+    (1, 2, 2, 5, 9, False, 0),
+    (2, 3, 3, 128, 128, True, 0),
+    (1, 2, 1, 130, 200, True, 70),        # GQA, bottom-right causal, ragged tiles
+    (1, 4, 4, 257, 63, True, 0),          # Sq > Sk top-left causal: one partial K/V tile
+    (2, 2, 2, 64, 1000, False, 0),
+    (1, 2, 2, 1, 1025, True, 1024),       # decode shape through the prefill kernel
+    (1, 1, 1, 300, 300, True, 0),
+    (1, 2, 2, 512, 512, True, 0),         # paired causal query tiles (two passes per workgroup)
+    (1, 2, 2, 1024, 1024, True, 0),
+    (3, 4, 2, 200, 456, False, 0),
+]
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
+@pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", D256_CASES)
+def test_half_d256_kernel_matches_oracle_and_the_other_forms(be, kind, B, H, Hkv, Sq, Sk, causal, offset):
+    D = 256
+    rng = np.random.default_rng(B + 3 * H + 7 * Sq + 11 * Sk + len(kind) + 256)
+    q, k, v = _rand(rng, B, H, Sq, D), _rand(rng, B, Hkv, Sk, D), _rand(rng, B, Hkv, Sk, D)
+    (qb, qw), (kb, kw), (vb, vw) = round_to(q, kind), round_to(k, kind), round_to(v, kind)
+    scale = 1.0 / math.sqrt(D)
+    o64, lse64 = oracle.attention_f64(qw, kw, vw, scale, causal, offset)
+    dt = TORCH16[kind]
+    args = (be.WrapTensor(from_bits16(qb, dt)), be.WrapTensor(from_bits16(kb, dt)), be.WrapTensor(from_bits16(vb, dt)))
+    outs = {}
+    try:
+        # True: the 64-key-tile kernel of 512-byte rows; 2: the 32-key-tile direct-to-LDS form; False: the general kernel
+        for fast in (True, 2, False):
+            be.SetAttentionFastPath(fast)
+            out = torch.full((B, H, Sq, D), float("nan"), device="cuda")
+            lse = torch.full((B, H, Sq), float("nan"), device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out), be.WrapTensor(lse), B, H, Sq, Sk, D, scale, causal, offset, Hkv)
+            outs[fast] = (out.cpu().numpy(), lse.cpu().numpy())
+            assert mixed_err(outs[fast][0], o64) <= HALF_TOL
+            assert mixed_err(outs[fast][1], lse64) <= 1e-3
+            out16 = torch.zeros((B, H, Sq, D), dtype=dt, device="cuda")
+            be.FlashAttentionHalf(kind, *args, be.WrapTensor(out16), None, B, H, Sq, Sk, D, scale, causal, offset, Hkv, True)
+            assert mixed_err(out16.float().cpu().numpy(), o64) <= HALF_TOL
+        assert mixed_err(outs[True][0], outs[False][0]) <= 1e-2 and mixed_err(outs[2][0], outs[False][0]) <= 1e-2
+    finally:
+        be.SetAttentionFastPath(True)
+
+
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
                                                                    (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
