@@ -148,7 +148,8 @@ class Mi355Backend:
 
     def SetAttentionFastPath(self, enabled) -> None:
         """Test hook: False routes every attention shape through the general kernel; 2 / 3 keep the fast paths and pin unsplit
-        head-dimension-128 prefill to the phase-structured / the software-pipelined kernel (True: chosen by pass length)."""
+        head-dimension-128 prefill to the phase-structured / the software-pipelined kernel (True: chosen by pass length); at head
+        dimension 256, 2 pins the older 32-key-tile form in place of the 64-key-tile kernel."""
         self._check(self._lib.aidn_mi355_set_attention_fast_path(self._ctx, int(enabled) if enabled in (2, 3) and enabled is not True else (1 if enabled else 0)))
 
     def ReserveWorkspace(self, size_in_bytes: int) -> None:

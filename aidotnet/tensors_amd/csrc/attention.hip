@@ -671,9 +671,15 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void attn_fwd_dl_kernel(cons
             m_ref = m_new;
             l_run *= alpha;
 #pragma unroll
-            for (int i = 0; i < DT; i++)
+            for (int i = 0; i < DT; i++) {
+                // (head dimension 256: the accumulators live in accumulation registers, which the multiply cannot read.  The two
+                // opaque statements pin them there on both sides of it, so that the copies to and from vector registers are made
+                // here, on this rare path, and not once per tile on the common one.)
+                if constexpr (D == 256) asm volatile("" : "+a"(oacc[i]));
 #pragma unroll
                 for (int r = 0; r < 16; r++) oacc[i][r] *= alpha;
+                if constexpr (D == 256) asm volatile("" : "+a"(oacc[i]));
+            }
         }
     };
     // p = exp2(s * c - m) of two scores, rounded and packed; the row sum accumulates the rounded values (the
@@ -736,7 +742,7 @@ __global__ __launch_bounds__(256, D == 128 ? 2 : 1) void attn_fwd_dl_kernel(cons
             f32x16 s0, s1;
 #pragma unroll
             for (int r = 0; r < 16; r++) { s0[r] = 0.0f; s1[r] = 0.0f; }
-            constexpr int R = AIDN_ATTN_RING;
+            constexpr int R = AIDN_ATTN_RING;       // (head dimension 256, one wave per SIMD: 2 and 4 measure the same, 8 costs registers and 5-15 %)
             static_assert(DSTEPS % R == 0 && DSTEPS == 2 * DT, "the fragment ring is indexed s % R over DSTEPS steps in every phase");
             constexpr int EV = DSTEPS / 8;          // steps per pair of exponentials (eight pairs per 32-key sub-tile)
             u32x4 fr[R];

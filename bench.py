@@ -442,6 +442,8 @@ def main() -> int:
     gemm_case("gemm_bf16_vocab50257", "bf16", 64, 50257, 768, hbm=True, rotate=6, extra=True)
     gemm_case("gemm_bf16_vocab50257_packed", "bf16", 64, 50257, 768, hbm=True, rotate=6, extra=True, packed=True)
     attn_case("attn_f32_prefill_b32", "f32", 32, 12, 512, 64, extra=True)
+    attn_case("attn_f16_prefill_d256", "f16", 2, 32, 2048, 256, extra=True)
+    attn_case("attn_bf16_prefill_d256", "bf16", 2, 32, 2048, 256, extra=True)
     out["others"] = others
 
     if args.copy_calibration:

@@ -350,7 +350,8 @@ AIDN_API int aidn_mi355_set_gemm_tile(void* ctx, int tile);
  * paths are then not taken), so the parity suite can hold the kernels against each other; unsplit
  * head-dim-128 prefill on dense 16-bit arrays has two kernels (the software-pipelined one is the default, the
  * phase-structured one takes the other layouts): enabled == 2 pins the phase-structured one, enabled == 3 the
- * software-pipelined one wherever it applies (each of the three is checked against the others).  Per context.
+ * software-pipelined one wherever it applies (each of the three is checked against the others); at head dimension 256
+ * enabled == 2 pins the older 32-key-tile form in place of the 64-key-tile kernel.  Per context.
  * No counterpart in the reference. */
 AIDN_API int aidn_mi355_set_attention_fast_path(void* ctx, int enabled);
 

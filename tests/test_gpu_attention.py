@@ -521,6 +521,42 @@ def test_half_d256_kernel_matches_oracle_and_the_other_forms(be, kind, B, H, Hkv
 
 
 @pytest.mark.parametrize("kind", ["f16", "bf16"])
+def test_half_d256_causal_b2_h32_s2048_every_slice(be, kind):
+    # the full grid of the head-dimension-256 kernel (1024 query tiles in pairs, one workgroup per CU, two rounds): one slice against
+    # the oracle, every (batch, head) slice against a float64 softmax of the same rounded inputs computed on the device (whole LSE
+    # column, eight sampled rows of O), so that a wrong head / tile / pass remap cannot hide
+    B, H, S, D = 2, 32, 2048, 256
+    dt = TORCH16[kind]
+    g = torch.Generator(device="cuda"); g.manual_seed(256)
+    q = torch.randn(B, H, S, D, device="cuda", generator=g).to(dt)
+    k = torch.randn(B, H, S, D, device="cuda", generator=g).to(dt)
+    v = torch.randn(B, H, S, D, device="cuda", generator=g).to(dt)
+    scale = 1.0 / math.sqrt(D)
+    out = torch.full((B, H, S, D), float("nan"), device="cuda")
+    lse = torch.empty(B, H, S, device="cuda")
+    be.FlashAttentionHalf(kind, be.WrapTensor(q), be.WrapTensor(k), be.WrapTensor(v), be.WrapTensor(out), be.WrapTensor(lse),
+                          B, H, S, S, D, scale, True)
+    assert torch.isfinite(out).all() and torch.isfinite(lse).all()
+    assert torch.allclose(out[:, :, 0], v[:, :, 0].float(), atol=1e-6)
+    qs, ks, vs = (t[1:2, 17:18].float().cpu().numpy() for t in (q, k, v))
+    o64, lse64 = oracle.attention_f64(qs, ks, vs, scale, True)
+    assert mixed_err(out[1, 17].cpu().numpy(), o64[0, 0]) <= HALF_TOL
+    assert mixed_err(lse[1, 17].cpu().numpy(), lse64[0, 0]) <= 1e-3
+    rng = np.random.default_rng(6)
+    causal_mask = torch.ones(S, S, device="cuda", dtype=torch.bool).tril()
+    for b in range(B):
+        for h in range(H):
+            q64, k64, v64 = q[b, h].double(), k[b, h].double(), v[b, h].double()
+            logits = ((q64 @ k64.T) * scale).masked_fill(~causal_mask, float("-inf"))
+            lse_ref = torch.logsumexp(logits, dim=1)
+            assert float((lse[b, h].double() - lse_ref).abs().max()) <= (1e-3 if kind == "f16" else 4e-3), (b, h)
+            rows = torch.from_numpy(rng.choice(S, 8, replace=False)).cuda()
+            o_ref = torch.softmax(logits[rows], dim=1) @ v64
+            err = ((out[b, h][rows].double() - o_ref).abs() / (1 + o_ref.abs())).max()
+            assert float(err) <= HALF_TOL, (b, h)
+
+
+@pytest.mark.parametrize("kind", ["f16", "bf16"])
 @pytest.mark.parametrize("B,H,Hkv,Sq,Sk,causal,offset", FAST_CASES + [(2, 4, 2, 17, 40, True, 23), (1, 4, 4, 70, 70, True, 0),
                                                                    (1, 2, 2, 512, 512, True, 0), (1, 3, 3, 200, 50, True, 0)])
 def test_half_d64_direct_load_form_matches_oracle_and_general_form(be, kind, B, H, Hkv, Sq, Sk, causal, offset):
