@@ -31,26 +31,27 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # measured yet.
 TRAFFIC_BYTES = {
     # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes), last three dispatches of each kernel
-    "gemm_f16_8192": int((787084 * 2.0 + 131176) * 1024),
-    "gemm_bf16_8192": int((787028 * 2.0 + 131270) * 1024),
-    "gemm_f16_proj": int((17114 * 2.0 + 24582) * 1024),
+    "gemm_f16_8192": int((786913 * 2.0 + 131190) * 1024),
+    "gemm_bf16_8192": int((787068 * 2.0 + 131347) * 1024),
+    "gemm_f16_proj": int((17114 * 2.0 + 24583) * 1024),
     "gemm_f16_proj_f32out": int((17048 * 2.0 + 49168) * 1024),
-    "gemm_f32_proj": int((43085 * 2.0 + 49152) * 1024),
+    "gemm_f32_proj": int((43087 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
     "decode_bf16": int((1048770 * 2.0 + 512) * 1024),
-    "attn_f16_prefill": int((132442 * 2.0 + 132112) * 1024),
-    "attn_bf16_prefill": int((132484 * 2.0 + 132122) * 1024),
-    "attn_f32_prefill": int((22643 * 2.0 + 12480) * 1024),
-    # two launches each: the skinny kernel, then the pass that sums its K ranges (the 4096-wide summing pass: 8 ranges of 32 x 4096 fp32
-    # partials read back, 2073 KiB on the counter, 256 KiB written)
-    "gemm_bf16_decode_proj": int(((17442 + 2073) * 2.0 + 4096 + 256) * 1024),
+    "attn_f16_prefill": int((132503 * 2.0 + 132106) * 1024),
+    "attn_bf16_prefill": int((132416 * 2.0 + 132110) * 1024),
+    "attn_f32_prefill": int((22635 * 2.0 + 12480) * 1024),
+    # two launches each: the skinny kernel, then the pass that sums its K ranges
+    "gemm_bf16_decode_proj": int(((17442 + 2071) * 2.0 + 4096 + 256) * 1024),
     "gemm_bf16_decode_qkv": int(((50203 + 3863) * 2.0 + 7680 + 768) * 1024),
     "gemm_bf16_decode_qkv_rope": int(((50203 + 3864) * 2.0 + 7680 + 768) * 1024),
     # profiles/grouped_decode_and_fp32_few_row_gemm_mi355x.md (kernel + its merge / summing pass; the summing pass of the 16-row product
     # reads its 16 ranges of 16 x 4096 fp32 partials back: 4 MiB, 2049 KiB on the counter)
-    "decode_bf16_gqa": int(((262417 + 1108) * 2.0 + 1040 + 512) * 1024),
+    "decode_bf16_gqa": int(((262418 + 1108) * 2.0 + 1040 + 512) * 1024),
     "decode_f32_gqa": int(((525392 + 1108) * 2.0 + 2176 + 512) * 1024),
     "gemm_f32_m16": int(((33819 + 2049) * 2.0 + 4096 + 256) * 1024),
+    "attn_f16_prefill_d256": int((135628 * 2.0 + 131597) * 1024),
+    "attn_bf16_prefill_d256": int((135805 * 2.0 + 131636) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
