@@ -544,6 +544,18 @@ def test_config2_square_8192_baseline_distribution_sampled_rows(be, kind):
     assert mixed_err(c32[rows].cpu().numpy(), truth) <= 1e-4
     assert mixed_err(c16[rows].float().cpu().numpy(), truth) <= HALF_TOL
     assert torch.equal(c16, c32.to(dt)), "16-bit output is not the RNE narrowing of the fp32 accumulator"
+    # eight of the sampled rows through the CPU oracle itself (the restated reduced-precision GEMM, fp32 accumulation in its own
+    # order: 8 x 8192 x 8192), which ties the device-side float64 truth above to the oracle's arithmetic at this size
+    sub = rows[:8]
+    a_bits = a[sub].contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    b_bits = b.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+    want16, want32 = (oracle.hgemm if kind == "f16" else oracle.bf16gemm)(a_bits, b_bits, 8, n, n)
+    assert mixed_err(np.asarray(want32).reshape(8, n), truth[:8]) <= 1e-4
+    assert mixed_err(c32[sub].cpu().numpy(), np.asarray(want32).reshape(8, n)) <= 1e-4
+    # (two fp32 sums in different orders, each rounded once: at most one unit in the last place of the storage type apart, relative
+    # to 1 + |x| -- near zero the sums cancel and bit patterns say nothing)
+    want16_t = torch.from_numpy(np.asarray(want16).reshape(8, n).view(np.int16).copy()).view(dt).float().numpy()
+    assert mixed_err(c16[sub].float().cpu().numpy(), want16_t) <= (2.0 ** -10 if kind == "f16" else 2.0 ** -7)
     # the reduced-precision result differs from the product of the unrounded inputs' fp32 GEMM: not a widened fp32 path
     assert bool(torch.isfinite(c32).all())
 
