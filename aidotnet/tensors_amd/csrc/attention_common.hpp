@@ -27,6 +27,7 @@ struct AttnArgs {
     long long qs[3], ks[3], vs[3], os[3];
     int qtiles;
     int nvb;       // pipelined prefill kernel: virtual blocks (the grid's workgroups take them in turn)
+    int alt_from;  // pipelined prefill kernel: first workgroup of the second half of a resident grid (shares its CU with an earlier one)
     FastDiv dgroup, dunits, dqtiles;      // pipelined prefill kernel: H / Hkv, qtiles / 2, qtiles as divisors
     int hgroup;    // general kernel, causal: > 0 heads per group of the workgroup order of a large grid; < 0 the placement of a small one
     // fast kernel, grouped decode: the workgroup's key range is split `split` of nsplit (chunk keys each) and, when part is not

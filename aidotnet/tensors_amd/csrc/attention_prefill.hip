@@ -20,7 +20,10 @@
 #ifdef PREFILL_LOOP_FILE
 #include PREFILL_LOOP_FILE
 #else
-#include "attention_prefill_loop.inc"
+#ifndef PREFILL_LOOP_INC
+#define PREFILL_LOOP_INC "attention_prefill_loop.inc"
+#endif
+#include PREFILL_LOOP_INC
 #endif
 
 namespace aidn {
@@ -73,6 +76,7 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         }
         if (npass == 2 && (k & 1)) qt = a.qtiles - 1 - qt;
     };
+    const bool alt_flavour = (int)blockIdx.x >= a.alt_from;
     const int nitems = (int)blockIdx.x < a.nvb ? ((a.nvb - 1 - (int)blockIdx.x) / (int)gridDim.x + 1) * npass : 0;
 
     const uint32_t lds0 = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) void*)smem);
@@ -382,13 +386,16 @@ __global__ __launch_bounds__(256, 2) void attn_prefill_kernel(const AttnArgs a)
         int mask_follows = __builtin_amdgcn_readfirstlane(masked_last ? 1 : 0);
         const int mask_rel0 = klim[0] - 32 * (u + n), mask_rel1 = klim[1] - 32 * (u + n);
         const float ninf = -INFINITY;
+        // (the routine has two flavours that differ in the wave priority of every other unit: the workgroups of the second half of a
+        // resident grid share their CUs with those of the first half and take the other flavour, so the two take turns in leading)
+        const int flavour = __builtin_amdgcn_readfirstlane(alt_flavour ? 1 : 0);
         if (masked_last) n++;
         u32x4 p0 = pf[0], p1 = pf[1];
 #define PREFILL_LOOP_OPERANDS \
             : "+{v[0:15]}"(oacc[0]), "+{v[16:31]}"(oacc[1]), "+{v[32:47]}"(oacc[2]), "+{v[48:63]}"(oacc[3]), "+{v[64:79]}"(sacc), \
               "+{v[80:83]}"(p0), "+{v[84:87]}"(p1), "+{v167}"(ps0), "+{v168}"(ps1), "+{s[40:41]}"(kptr), "+{s[42:43]}"(vptr), "+{s53}"(count), "+{s57}"(kleft), "+{s58}"(vleft), "+{s59}"(mask_follows) \
             : "{v[88:103]}"(qlo), "{v[104:119]}"(qhi), "{v[152:155]}"(kad), "{v[192:195]}"(vad0), "{v[196:199]}"(vad1), \
-              "{v[160:163]}"(klo), "{v164}"(vlo), "{v174}"(vlo_odd), "{v165}"(negm0), "{v166}"(negm1), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), \
+              "{v[160:163]}"(klo), "{v164}"(vlo), "{v174}"(vlo_odd), "{v165}"(negm0), "{v166}"(negm1), "{s[44:51]}"(sc), "{s52}"(sl2s), "{s56}"(phase), "{s60}"(flavour), \
               "{v171}"(mask_rel0), "{v172}"(mask_rel1), "{v173}"(ninf) \
             : "v120", "v121", "v122", "v123", "v124", "v125", "v126", "v127", "v128", "v129", "v130", "v131", "v132", "v133", "v134", \
               "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145", "v146", "v147", "v148", "v149", \
@@ -616,6 +623,7 @@ static hipError_t launch_prefill(AttnArgs a, hipStream_t stream)
     }
     const long long resident = (long long)(2 * cus) / 8 * 8;
     const unsigned grid = (unsigned)((resident >= 8 && nblk > resident) ? resident : nblk);
+    a.alt_from = cus;              // workgroup b + (number of CUs) lands on the CU of workgroup b (measured: every CU of a full grid)
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), smem, stream, a);
     return hipGetLastError();
 }

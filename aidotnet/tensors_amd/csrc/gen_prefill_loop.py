@@ -17,7 +17,7 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def gen(kind, ablate=()):
+def gen(kind, ablate=(), flip=0, period=1):
     """One routine on v_mfma_f32_16x16x32.  A wave's 32 queries are two blocks of 16 (qb), a unit's 32 keys two blocks of 16 (kb),
     the head dimension eight blocks of 16 (db); every fragment read from LDS feeds two MFMAs (one per query block).  Lane (c, g) =
     (lane % 16, lane / 16) holds query c of a block and keys / dims 4 g + r of a block.  Per unit u a block has 16 slots, slot i
@@ -39,7 +39,16 @@ def gen(kind, ablate=()):
     inside a masked unit per query block, v173 minus infinity, v[176:191] exponentials.
     s[40:41] / s[42:43] source of this wave's next K / V tile load, s[46:47] s[48:49] one K / V tile in bytes, s50 s51 LDS
     destination of this wave's K / V loads in stage 0, s52 scale * log2(e), s53 units left, s56 block of the first unit, s57 s58
-    odd units that still load a K / V tile, s59 whether a masked unit follows the run."""
+    odd units that still load a K / V tile, s59 whether a masked unit follows the run, s60 the priority flavour (below).
+
+    Wave priority: the two workgroups of a CU run this routine side by side, and a SIMD serves the older of two waves of equal
+    priority first -- left alone the older workgroup gets about 63 % of the issue slots, finishes early, and the younger one runs the
+    last fifth of the launch on its own.  Each unit therefore starts with s_setprio ((unit / period) % 2) ^ flip: the workgroups of
+    the first and of the second half of the grid (which share the CUs) take the flavours flip = 0 and flip = 1, so that at any time
+    one of the two leads and they take turns; the routine leaves at priority 0.  Measured on causal and unmasked B4 H32 S2048 and
+    causal S8192: the gap between the two workgroups' finish times halves (30 -> 16 us of 148) and the launch is 0.5-2.5 % shorter
+    (alternating every second unit measures the same; also keeping the younger workgroup raised outside the routine closes the gap
+    to 4 us and gains nothing more: the board's power management pays a lone workgroup back in clock)."""
     mfma = "v_mfma_f32_16x16x32_" + kind
     cvt = "v_cvt_pk_%s_f32" % kind
     dot = "v_dot2c_f32_%s_e32" % kind
@@ -78,7 +87,7 @@ def gen(kind, ablate=()):
         emit("s_waitcnt lgkmcnt(%d)" % left)
         del queue[:last + 1]
 
-    label = "L_prefill_%s_" % kind
+    label = "L_prefill_%s%s_" % (kind, "_alt" if flip else "")
     first7 = lambda blk: [(blk, f) for f in range(7) for _ in (0, 1)]
     for j in (1, 2, 3):
         emit("s_cmp_eq_u32 s56, %d" % j)
@@ -142,6 +151,8 @@ def gen(kind, ablate=()):
         is_b = (blk & 1) == 0
         kstage = (blk >> 1) & 1
         emit("%sblk%d_%%=:" % (label, blk))
+        if "prio" not in ablate:
+            emit("s_setprio %d" % ((((blk // period) & 1) ^ flip)))
         del queue[:]
         queue.extend(first7(blk))
         if is_b:
@@ -191,6 +202,8 @@ def gen(kind, ablate=()):
             emit("v_cndmask_b32_e32 v%d, v%d, v173, vcc" % (64 + t, 64 + t))
         emit("s_branch %sblk%d_%%=" % (label, (blk + 1) & 3))
     emit("%sexit_%%=:" % label)
+    if "prio" not in ablate:
+        emit("s_setprio 0")
     emit("s_waitcnt lgkmcnt(0)")
     return out
 
@@ -198,8 +211,12 @@ def gen(kind, ablate=()):
 def write(name, ablate=()):
     with open(name, "w") as fh:
         fh.write("// Generated by gen_prefill_loop.py (the run of whole units of attn_prefill_kernel as gfx950 assembly); do not edit.\n")
+        period = 2 if "period2" in ablate else 1
         for kind in ("f16", "bf16"):
-            lines = gen(kind, ablate)
+            # both priority flavours in one statement (s60 != 0 selects the second): one set of register bindings in the kernel
+            lines = ["s_cmp_eq_u32 s60, 0", "s_cbranch_scc0 L_prefill_%s_second_%%=" % kind]
+            lines += gen(kind, ablate, 0, period) + ["s_branch L_prefill_%s_end_%%=" % kind, "L_prefill_%s_second_%%=:" % kind]
+            lines += gen(kind, ablate, 1, period) + ["L_prefill_%s_end_%%=:" % kind]
             fh.write("#define PREFILL_LOOP_%s \\\n" % kind.upper())
             for n, line in enumerate(lines):
                 sep = "\\n" if line.endswith(":") else "\\n\\t"
