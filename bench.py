@@ -31,16 +31,16 @@ METRIC = "GEMM & fused-attn TFLOP/s (% MFMA peak), decode-attn GB/s, 1x MI355X"
 # measured yet.
 TRAFFIC_BYTES = {
     # profiles/hbm_traffic_pmc_mi355x.md: FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 (KiB -> bytes), last three dispatches of each kernel
-    "gemm_f16_8192": int((786913 * 2.0 + 131190) * 1024),
-    "gemm_bf16_8192": int((787068 * 2.0 + 131347) * 1024),
-    "gemm_f16_proj": int((17114 * 2.0 + 24583) * 1024),
-    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49168) * 1024),
-    "gemm_f32_proj": int((43087 * 2.0 + 49152) * 1024),
+    "gemm_f16_8192": int((786920 * 2.0 + 131340) * 1024),
+    "gemm_bf16_8192": int((787044 * 2.0 + 131400) * 1024),
+    "gemm_f16_proj": int((17114 * 2.0 + 24584) * 1024),
+    "gemm_f16_proj_f32out": int((17048 * 2.0 + 49165) * 1024),
+    "gemm_f32_proj": int((43104 * 2.0 + 49152) * 1024),
     "gemm_f32_1024": int((12318 * 2.0 + 4096) * 1024),
     "decode_bf16": int((1048770 * 2.0 + 512) * 1024),
-    "attn_f16_prefill": int((132503 * 2.0 + 132106) * 1024),
-    "attn_bf16_prefill": int((132416 * 2.0 + 132110) * 1024),
-    "attn_f32_prefill": int((22635 * 2.0 + 12480) * 1024),
+    "attn_f16_prefill": int((144204 * 2.0 + 132098) * 1024),
+    "attn_bf16_prefill": int((144033 * 2.0 + 132102) * 1024),
+    "attn_f32_prefill": int((22634 * 2.0 + 12480) * 1024),
     # two launches each: the skinny kernel, then the pass that sums its K ranges
     "gemm_bf16_decode_proj": int(((17442 + 2071) * 2.0 + 4096 + 256) * 1024),
     "gemm_bf16_decode_qkv": int(((50203 + 3863) * 2.0 + 7680 + 768) * 1024),
@@ -50,8 +50,8 @@ TRAFFIC_BYTES = {
     "decode_bf16_gqa": int(((262418 + 1108) * 2.0 + 1040 + 512) * 1024),
     "decode_f32_gqa": int(((525392 + 1108) * 2.0 + 2176 + 512) * 1024),
     "gemm_f32_m16": int(((33819 + 2049) * 2.0 + 4096 + 256) * 1024),
-    "attn_f16_prefill_d256": int((135628 * 2.0 + 131597) * 1024),
-    "attn_bf16_prefill_d256": int((135805 * 2.0 + 131636) * 1024),
+    "attn_f16_prefill_d256": int((135459 * 2.0 + 131620) * 1024),
+    "attn_bf16_prefill_d256": int((135583 * 2.0 + 131635) * 1024),
 }
 # MI355X published dense peaks
 PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
