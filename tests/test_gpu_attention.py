@@ -177,7 +177,33 @@ def test_strided_qkv_from_packed_projection(be):
     assert mixed_err(lse.cpu().numpy(), lse_w) <= FP32_TOL
 
 
-@pytest.mark.parametrize("kind,D", [("bf16", 128), ("f16", 128), ("f32", 64), ("bf16", 64)])
+@pytest.mark.parametrize("kind,D", [("bf16", 128), ("f16", 128), ("bf16", 256), ("f16", 256), ("bf16", 64)])
+def test_strided_16bit_qkv_from_packed_projection(be, kind, D):
+    # the same packed [B*S, 3*dModel] activation in the 16-bit types: K and V rows 3*dModel elements apart go through the
+    # direct-to-LDS tile loads of the head-dimension-128 / 256 kernels (row stride as a run-time value), O is written [B,S,H,d]
+    from aidotnet.tensors_amd import AttnDesc
+    rng = np.random.default_rng(D + len(kind))
+    B, S, H = 2, 203, 3
+    dm = H * D
+    qkv = _rand(rng, B * S, 3 * dm)
+    bits, wide = round_to(qkv, kind)
+    dt = TORCH16[kind]
+    t = from_bits16(bits, dt)
+    out = torch.full((B, S, H, D), float("nan"), device="cuda")
+    d = AttnDesc(B=B, H=H, Hkv=H, Sq=S, Sk=S, D=D, scale=1 / math.sqrt(D), causal=1)
+    for name in ("q_strides", "k_strides", "v_strides"):
+        getattr(d, name)[:] = [S * 3 * dm, D, 3 * dm]
+    d.o_strides[:] = [S * dm, D, dm]
+    lse = torch.empty(B, H, S, device="cuda")
+    be._attn(kind, be.WrapTensor(t), _Off(t, dm), _Off(t, 2 * dm), be.WrapTensor(out), be.WrapTensor(lse), None, None, None, d)
+    x = wide.reshape(B, S, 3, H, D)
+    q, k, v = (np.ascontiguousarray(x[:, :, i].transpose(0, 2, 1, 3)) for i in range(3))
+    o64, lse64 = oracle.attention_f64(q, k, v, 1 / math.sqrt(D), True, 0)
+    assert mixed_err(out.cpu().numpy().transpose(0, 2, 1, 3), o64) <= HALF_TOL
+    assert mixed_err(lse.cpu().numpy(), lse64) <= 1e-3
+
+
+@pytest.mark.parametrize("kind,D", [("bf16", 128), ("f16", 128), ("f32", 64), ("bf16", 64), ("bf16", 256), ("f16", 256)])
 def test_output_layouts_of_the_direct_to_lds_kernels(be, kind, D):
     # The kernels that stage O through LDS write whole rows; the same call with O laid out [B,S,H,D] (row stride H*D), with a
     # dense O, and with an O that starts 4 bytes off a 16-byte boundary (element-wise stores) must give the same numbers.
